@@ -1,0 +1,160 @@
+/*
+ * C ABI of the gfx950 fused multi-head-attention library (libfmha_hip.so).
+ *
+ * Plain pointers and sizes only -- no torch / ATen types -- so the library can be
+ * bound from C, C++, ctypes or any FFI.  All tensor pointers are DEVICE pointers;
+ * the library never allocates, frees or synchronises: kernels are enqueued on the
+ * HIP stream the caller passes and the call returns immediately.
+ *
+ * What each entry point replaces in the reference (shmsong/NvFuserExamples):
+ * the reference has no C ABI; its boundary is the torch dispatcher
+ * (fmha/fmha_manual.cpp:1240-1250) and behind it NVFuserOpBase<T>::run
+ * (common/manual_scheduled_kernel.h:13-19), which JIT-compiles and launches one
+ * nvFuser-generated kernel per op.  The launch functions below take the place of
+ * that run() call for the three fused kernels
+ *   FMHAKernel                       fmha/fmha_manual.cpp:20-409
+ *   FMHATrainKernel                  fmha/fmha_manual.cpp:411-807
+ *   FMHATrainKernelSaveIntermediate  fmha/fmha_manual.cpp:809-1214
+ * with shapes, scale, mask layout and dropout as run-time arguments instead of
+ * compile-time constants (fmha/fmha_manual.cpp:24-29,68,421).
+ */
+#ifndef FMHA_CAPI_H_
+#define FMHA_CAPI_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of q/k/v/o, masks and gradients */
+enum { FMHA_DTYPE_F16 = 0, FMHA_DTYPE_BF16 = 1 };
+
+/* how the mask tensor enters the scores */
+enum {
+  FMHA_MASK_NONE = 0,
+  FMHA_MASK_ADDITIVE = 1, /* score += mask                    (train ops, fmha_manual.cpp:463) */
+  FMHA_MASK_KEEP01 = 2    /* score += (1 - mask) * mask_neg   (inference op, fmha_manual.cpp:64-71) */
+};
+
+/* dropout source */
+enum {
+  FMHA_DROP_NONE = 0,
+  FMHA_DROP_PHILOX = 1,  /* keep decisions from Philox4x32-10 keyed by (seed, offset) */
+  FMHA_DROP_TENSOR = 2   /* caller supplies a multiplicative [bh,sq,sk] tensor (fmha_manual.cpp:478-480) */
+};
+
+/* return codes */
+enum {
+  FMHA_OK = 0,
+  FMHA_E_NULL = -1,        /* a required pointer is NULL */
+  FMHA_E_DTYPE = -2,       /* unknown dtype */
+  FMHA_E_SHAPE = -3,       /* non-positive size or unsupported head dim (64 and 128 are built) */
+  FMHA_E_ALIGN = -4,       /* q/k/v/o/gradient base pointer not 16-byte aligned */
+  FMHA_E_ARG = -5,         /* scale / p_drop / mask description out of range */
+  FMHA_E_UNSUPPORTED = -6, /* combination not built (see fmha_strerror) */
+  FMHA_E_LAUNCH = -7       /* the HIP runtime refused the launch */
+};
+
+/*
+ * Forward.  Layout (as the reference, fmha/fmha_manual.cpp:39-47): heads folded into
+ * dim 0, everything contiguous:
+ *   q [bh,sq,d]   k [bh,sk,d]   v [bh,sk,d]   o [bh,sq,d]
+ * Mask element (b,i,j) is read at
+ *   mask[(b / mask_bh_div) * mask_stride_b + i * mask_stride_q + j]
+ * so [bh,sq,sk] is (div 1, stride_b sq*sk, stride_q sk), a [B,1,1,sk] padding mask
+ * over bh = B*H is (div H, stride_b sk, stride_q 0).
+ * Computes  O = (dropout(softmax(scale * q k^T + mask_term [+ causal]))) v
+ * with fp32 accumulation and fp32 softmax, the probabilities rounded to the
+ * element type before the second product (fmha_manual.cpp:87) and O rounded on
+ * store (fmha_manual.cpp:95).
+ */
+typedef struct fmha_fwd_params {
+  const void *q, *k, *v;
+  void *o;
+  float *lse; /* optional [bh,sq]: log(sum_j exp(score_ij)), saved for the backward */
+
+  const void *mask; /* optional, element type = dtype */
+  int32_t mask_kind;
+  int32_t causal; /* 1: key j is visible to query i iff j <= i (no tensor involved) */
+  int64_t mask_bh_div, mask_stride_b, mask_stride_q;
+  float mask_neg; /* used by FMHA_MASK_KEEP01; -10000 in the reference */
+
+  int32_t drop_kind;
+  const void *drop_mask; /* FMHA_DROP_TENSOR: [bh,sq,sk], element type = dtype */
+  float p_drop;          /* FMHA_DROP_PHILOX: drop probability in [0,1) */
+  float drop_scale;      /* factor on kept probabilities: 2 on the legacy ops, 1/(1-p) otherwise */
+  uint64_t seed, offset; /* FMHA_DROP_PHILOX */
+
+  /* optional [bh,sq,sk] outputs of the save-intermediates op (fmha_manual.cpp:891-897):
+   * softmax before dropout and after dropout*scale, element type = dtype.
+   * Only with FMHA_DROP_TENSOR or FMHA_DROP_NONE. */
+  void *save_softmax, *save_dropout;
+
+  int32_t bh, sq, sk, d;
+  int32_t dtype;
+  float scale; /* > 0; 1/8 in the reference (fmha_manual.cpp:68) */
+  int32_t flags; /* reserved, pass 0 */
+} fmha_fwd_params;
+
+/* Enqueue the forward kernel on `hip_stream` (a hipStream_t; NULL = default stream). */
+int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream);
+
+/*
+ * Backward (no counterpart in the reference, which has no backward kernel:
+ * README.md:1).  Inputs are those of the forward plus the upstream gradient
+ * `dout`, the forward output `o` and the saved `lse`; the dropout decisions are
+ * regenerated from (seed, offset) or re-read from drop_mask, never stored.
+ *   dv = (P o Z)^T dout ; dP = (dout v^T) o Z ; delta_i = sum_d dout_id o_id
+ *   dS = P o (dP - delta) ; dq = scale dS k ; dk = scale dS^T q
+ * `delta` is caller-provided scratch of bh*sq floats (written, then read).
+ */
+typedef struct fmha_bwd_params {
+  const void *q, *k, *v, *o, *dout;
+  const float *lse;
+  float *delta;
+  void *dq, *dk, *dv;
+
+  const void *mask;
+  int32_t mask_kind;
+  int32_t causal;
+  int64_t mask_bh_div, mask_stride_b, mask_stride_q;
+  float mask_neg;
+
+  int32_t drop_kind;
+  const void *drop_mask;
+  float p_drop;
+  float drop_scale;
+  uint64_t seed, offset;
+
+  int32_t bh, sq, sk, d;
+  int32_t dtype;
+  float scale;
+  int32_t flags; /* reserved, pass 0 */
+} fmha_bwd_params;
+
+int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);
+
+/*
+ * Materialise the Philox keep decisions the kernels use for (seed, offset, p_drop)
+ * as a [bh,sq,sk] tensor of bytes (1 keep, 0 drop) in device memory.  For tests and
+ * for callers that need the mask itself; the fused kernels never read such a tensor.
+ * (No counterpart in the reference, whose dropout mask is a caller-made tensor:
+ * test_train_mha.py:28.)
+ */
+int fmha_philox_keep_mask(uint64_t seed, uint64_t offset, float p_drop, int32_t bh, int32_t sq,
+                          int32_t sk, uint8_t *out, void *hip_stream);
+
+/* 8-bit threshold the keep rule compares against: keep iff random_byte >= threshold. */
+uint32_t fmha_drop_threshold(float p_drop);
+
+/* Static description of a return code. */
+const char *fmha_strerror(int code);
+
+/* Library version, "major.minor". */
+const char *fmha_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMHA_CAPI_H_ */

@@ -1,0 +1,207 @@
+"""ctypes binding of ``libfmha_hip.so`` (the C ABI declared in ``include/fmha_capi.h``).
+
+This is the thinnest possible host layer: torch is used only for device memory and
+the current HIP stream.  There is no CPU fallback -- if the library is missing the
+import of :func:`lib` raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfmha_hip.so")
+
+F16, BF16 = 0, 1
+MASK_NONE, MASK_ADDITIVE, MASK_KEEP01 = 0, 1, 2
+DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
+
+EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_philox_keep_mask", "fmha_drop_threshold",
+           "fmha_strerror", "fmha_version")
+
+
+class FwdParams(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("lse", C.c_void_p),
+        ("mask", C.c_void_p), ("mask_kind", C.c_int32), ("causal", C.c_int32),
+        ("mask_bh_div", C.c_int64), ("mask_stride_b", C.c_int64), ("mask_stride_q", C.c_int64),
+        ("mask_neg", C.c_float),
+        ("drop_kind", C.c_int32), ("drop_mask", C.c_void_p), ("p_drop", C.c_float), ("drop_scale", C.c_float),
+        ("seed", C.c_uint64), ("offset", C.c_uint64),
+        ("save_softmax", C.c_void_p), ("save_dropout", C.c_void_p),
+        ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
+        ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
+    ]
+
+
+class BwdParams(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("dout", C.c_void_p),
+        ("lse", C.c_void_p), ("delta", C.c_void_p),
+        ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+        ("mask", C.c_void_p), ("mask_kind", C.c_int32), ("causal", C.c_int32),
+        ("mask_bh_div", C.c_int64), ("mask_stride_b", C.c_int64), ("mask_stride_q", C.c_int64),
+        ("mask_neg", C.c_float),
+        ("drop_kind", C.c_int32), ("drop_mask", C.c_void_p), ("p_drop", C.c_float), ("drop_scale", C.c_float),
+        ("seed", C.c_uint64), ("offset", C.c_uint64),
+        ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
+        ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
+    ]
+
+
+class FmhaError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"fmha error {code}: {msg}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Load the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m nvfuserexamples_amd.build` "
+                "(there is no fallback path)")
+        L = C.CDLL(LIB_PATH)
+        L.fmha_fwd_launch.argtypes = [C.POINTER(FwdParams), C.c_void_p]
+        L.fmha_fwd_launch.restype = C.c_int
+        L.fmha_bwd_launch.argtypes = [C.POINTER(BwdParams), C.c_void_p]
+        L.fmha_bwd_launch.restype = C.c_int
+        L.fmha_philox_keep_mask.argtypes = [C.c_uint64, C.c_uint64, C.c_float, C.c_int32, C.c_int32,
+                                            C.c_int32, C.c_void_p, C.c_void_p]
+        L.fmha_philox_keep_mask.restype = C.c_int
+        L.fmha_drop_threshold.argtypes = [C.c_float]
+        L.fmha_drop_threshold.restype = C.c_uint32
+        L.fmha_strerror.argtypes = [C.c_int]
+        L.fmha_strerror.restype = C.c_char_p
+        L.fmha_version.restype = C.c_char_p
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise FmhaError(rc, lib().fmha_strerror(rc).decode())
+
+
+def _dtype_code(t):
+    import torch
+    if t.dtype == torch.float16:
+        return F16
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise FmhaError(-2, "tensors must be float16 or bfloat16")
+
+
+def _stream_ptr():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def mask_layout(mask, bh, sq, sk):
+    """(bh_div, stride_b, stride_q) of a mask shaped [bh,sq,sk], [bh,1,sk], [B,1,1,sk] or [B,1,sq,sk]."""
+    if mask.dim() == 4:
+        if mask.shape[1] != 1:
+            raise FmhaError(-5, "4-d masks must be [B,1,sq|1,sk]")
+        mask = mask.reshape(mask.shape[0], mask.shape[2], mask.shape[3])
+    if mask.dim() != 3 or mask.shape[2] != sk or mask.shape[1] not in (1, sq) or bh % mask.shape[0]:
+        raise FmhaError(-5, f"mask shape {tuple(mask.shape)} does not broadcast over [{bh},{sq},{sk}]")
+    if not mask.is_contiguous():
+        raise FmhaError(-5, "mask must be contiguous")
+    div = bh // mask.shape[0]
+    return mask, div, mask.shape[1] * sk, (0 if mask.shape[1] == 1 else sk)
+
+
+def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False, scale=None,
+        drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
+        want_lse=False, save=False, flags=0, out=None):
+    """Launch the forward on the current stream.  Returns (o, lse|None, softmax|None, dropout|None)."""
+    import torch
+    bh, sq, d = q.shape
+    sk = k.shape[1]
+    P = FwdParams()
+    P.dtype = _dtype_code(q)
+    for t in (q, k, v):
+        if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype):
+            raise FmhaError(-5, "q/k/v must be contiguous device tensors of one dtype")
+    o = out if out is not None else torch.empty_like(q)
+    lse = torch.empty((bh, sq), dtype=torch.float32, device=q.device) if want_lse else None
+    P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+    P.lse = lse.data_ptr() if lse is not None else None
+    P.bh, P.sq, P.sk, P.d = bh, sq, sk, d
+    P.scale = float(scale) if scale is not None else d ** -0.5
+    P.causal = int(bool(causal))
+    P.mask_neg = mask_neg
+    if mask is not None:
+        mask, div, sb, sqs = mask_layout(mask, bh, sq, sk)
+        if mask.dtype != q.dtype:
+            raise FmhaError(-5, "mask dtype must match q")
+        P.mask, P.mask_kind = mask.data_ptr(), mask_kind
+        P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = div, sb, sqs
+    P.drop_kind = drop_kind
+    if drop_kind == DROP_TENSOR:
+        if drop_mask is None or drop_mask.dtype != q.dtype or not drop_mask.is_contiguous():
+            raise FmhaError(-5, "drop_mask must be a contiguous tensor of q's dtype")
+        P.drop_mask = drop_mask.data_ptr()
+    P.p_drop = p_drop
+    if drop_scale is None:
+        drop_scale = 1.0 / (1.0 - p_drop) if drop_kind == DROP_PHILOX else 1.0
+    P.drop_scale = drop_scale
+    P.seed, P.offset = seed, offset
+    sm = dr = None
+    if save:
+        sm = torch.empty((bh, sq, sk), dtype=q.dtype, device=q.device)
+        dr = torch.empty((bh, sq, sk), dtype=q.dtype, device=q.device)
+        P.save_softmax, P.save_dropout = sm.data_ptr(), dr.data_ptr()
+    P.flags = flags
+    check(lib().fmha_fwd_launch(C.byref(P), _stream_ptr()))
+    return o, lse, sm, dr
+
+
+def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False,
+        scale=None, drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
+        flags=0, delta=None, grads=None):
+    """Launch the backward on the current stream.  Returns (dq, dk, dv)."""
+    import torch
+    bh, sq, d = q.shape
+    sk = k.shape[1]
+    P = BwdParams()
+    P.dtype = _dtype_code(q)
+    for t in (q, k, v, o, dout):
+        if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype):
+            raise FmhaError(-5, "q/k/v/o/dout must be contiguous device tensors of one dtype")
+    if delta is None:
+        delta = torch.empty((bh, sq), dtype=torch.float32, device=q.device)
+    dq, dk, dv = grads if grads is not None else (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    P.q, P.k, P.v, P.o, P.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), dout.data_ptr()
+    P.lse, P.delta = lse.data_ptr(), delta.data_ptr()
+    P.dq, P.dk, P.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    P.bh, P.sq, P.sk, P.d = bh, sq, sk, d
+    P.scale = float(scale) if scale is not None else d ** -0.5
+    P.causal = int(bool(causal))
+    P.mask_neg = mask_neg
+    if mask is not None:
+        mask, div, sb, sqs = mask_layout(mask, bh, sq, sk)
+        P.mask, P.mask_kind = mask.data_ptr(), mask_kind
+        P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = div, sb, sqs
+    P.drop_kind = drop_kind
+    if drop_kind == DROP_TENSOR:
+        P.drop_mask = drop_mask.data_ptr()
+    P.p_drop = p_drop
+    if drop_scale is None:
+        drop_scale = 1.0 / (1.0 - p_drop) if drop_kind == DROP_PHILOX else 1.0
+    P.drop_scale = drop_scale
+    P.seed, P.offset = seed, offset
+    P.flags = flags
+    check(lib().fmha_bwd_launch(C.byref(P), _stream_ptr()))
+    return dq, dk, dv
+
+
+def philox_keep_mask(seed, offset, p_drop, bh, sq, sk, device="cuda"):
+    """uint8 [bh,sq,sk] device tensor of the keep decisions the kernels use."""
+    import torch
+    out = torch.empty((bh, sq, sk), dtype=torch.uint8, device=device)
+    check(lib().fmha_philox_keep_mask(seed, offset, p_drop, bh, sq, sk, out.data_ptr(), _stream_ptr()))
+    return out

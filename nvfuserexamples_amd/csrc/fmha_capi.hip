@@ -1,0 +1,166 @@
+// C-ABI entry points of libfmha_hip.so: argument validation, variant selection and
+// launch.  Declared in include/fmha_capi.h.  No allocation, no synchronisation.
+#include "../../include/fmha_capi.h"
+#include "fmha_launch.h"
+
+#include <cmath>
+#include <cstdlib>
+
+using namespace fmha;
+
+namespace {
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool aligned8(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+
+__global__ void philox_keep_mask_kernel(DropCtx c, int sq, int sk, long long total, uint8_t *out) {
+  // one thread per (bh, q, 4-key group): writes up to four bytes
+  const long long kg = (sk + 3) / 4;
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long k4 = idx % kg;
+  const long long row = idx / kg;
+  const int q = (int)(row % sq);
+  const long long bh = row / sq;
+  const uint32_t wd = drop_word(c, (uint32_t)bh, (uint32_t)q, (uint32_t)k4);
+  uint8_t *dst = out + row * sk + k4 * 4;
+  for (int t = 0; t < 4; ++t)
+    if (k4 * 4 + t < sk) dst[t] = drop_keep_byte(wd, t, c.thr) ? 1 : 0;
+}
+
+DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
+  DropCtx c;
+  c.seed_lo = (uint32_t)seed;
+  c.seed_hi = (uint32_t)(seed >> 32);
+  c.off_lo = (uint32_t)offset;
+  c.off_hi = (uint32_t)(offset >> 32);
+  c.thr = fmha_drop_threshold(p);
+  c.qb4 = (uint32_t)((sq + 3) / 4);
+  c.kb4 = (uint32_t)((sk + 3) / 4);
+  return c;
+}
+
+// Tuning override for experiments: FMHA_FWD_QB=1|2 forces the query blocks per wave.
+int env_int(const char *name, int dflt) {
+  const char *e = std::getenv(name);
+  return e ? std::atoi(e) : dflt;
+}
+
+} // namespace
+
+extern "C" {
+
+uint32_t fmha_drop_threshold(float p_drop) {
+  double t = std::floor((double)p_drop * 256.0 + 0.5);
+  if (t < 0) t = 0;
+  if (t > 255) t = 255;
+  return (uint32_t)t;
+}
+
+const char *fmha_strerror(int code) {
+  switch (code) {
+  case FMHA_OK: return "ok";
+  case FMHA_E_NULL: return "a required pointer is NULL";
+  case FMHA_E_DTYPE: return "unknown dtype (0 = fp16, 1 = bf16)";
+  case FMHA_E_SHAPE: return "bad shape: sizes must be positive and head dim must be 64 or 128";
+  case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned";
+  case FMHA_E_ARG: return "argument out of range (scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
+  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox)";
+  case FMHA_E_LAUNCH: return "HIP launch failed";
+  default: return "unknown error code";
+  }
+}
+
+const char *fmha_version(void) { return "0.1"; }
+
+int fmha_philox_keep_mask(uint64_t seed, uint64_t offset, float p_drop, int32_t bh, int32_t sq,
+                          int32_t sk, uint8_t *out, void *hip_stream) {
+  if (!out) return FMHA_E_NULL;
+  if (bh <= 0 || sq <= 0 || sk <= 0) return FMHA_E_SHAPE;
+  if (!(p_drop >= 0.f && p_drop < 1.f)) return FMHA_E_ARG;
+  const DropCtx c = make_drop_ctx(seed, offset, p_drop, sq, sk);
+  const long long total = (long long)bh * sq * ((sk + 3) / 4);
+  const int nt = 256;
+  const long long nb = (total + nt - 1) / nt;
+  if (nb > 0x7fffffffLL) return FMHA_E_SHAPE;
+  hipLaunchKernelGGL(philox_keep_mask_kernel, dim3((unsigned)nb), dim3(nt), 0, (hipStream_t)hip_stream, c,
+                     sq, sk, total, out);
+  return hipGetLastError() == hipSuccess ? FMHA_OK : FMHA_E_LAUNCH;
+}
+
+int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
+  if (!p || !p->q || !p->k || !p->v || !p->o) return FMHA_E_NULL;
+  if (p->dtype != FMHA_DTYPE_F16 && p->dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
+  if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;
+  if (p->d != 64 && p->d != 128) return FMHA_E_SHAPE;
+  if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->o)) return FMHA_E_ALIGN;
+  if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return FMHA_E_ARG;
+  if (p->mask_kind < FMHA_MASK_NONE || p->mask_kind > FMHA_MASK_KEEP01) return FMHA_E_ARG;
+  if (p->drop_kind < FMHA_DROP_NONE || p->drop_kind > FMHA_DROP_TENSOR) return FMHA_E_ARG;
+  if (p->mask_kind != FMHA_MASK_NONE) {
+    if (!p->mask) return FMHA_E_NULL;
+    if (p->mask_bh_div < 1 || p->mask_stride_b < 0 || p->mask_stride_q < 0) return FMHA_E_ARG;
+  }
+  if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
+  if (p->drop_kind == FMHA_DROP_TENSOR && !p->drop_mask) return FMHA_E_NULL;
+  if (p->drop_kind != FMHA_DROP_NONE && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
+  const bool saving = p->save_softmax || p->save_dropout;
+  if (saving && (p->drop_kind == FMHA_DROP_PHILOX || p->causal)) return FMHA_E_UNSUPPORTED;
+  if (p->drop_kind == FMHA_DROP_TENSOR && p->causal) return FMHA_E_UNSUPPORTED;
+
+  FwdArgs a;
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.lse = p->lse;
+  a.mask = p->mask_kind ? p->mask : nullptr;
+  a.drop_mask = p->drop_kind == FMHA_DROP_TENSOR ? p->drop_mask : nullptr;
+  a.save_softmax = p->save_softmax;
+  a.save_dropout = p->save_dropout;
+  a.mask_sb = p->mask_stride_b;
+  a.mask_sq = p->mask_stride_q;
+  a.mask_div = p->mask_kind ? (int32_t)p->mask_bh_div : 1;
+  if (p->mask_kind == FMHA_MASK_KEEP01) {
+    a.mask_a = -p->mask_neg * FMHA_LOG2E;
+    a.mask_b = p->mask_neg * FMHA_LOG2E;
+  } else {
+    a.mask_a = FMHA_LOG2E;
+    a.mask_b = 0.f;
+  }
+  // 8-byte vector accesses to [.., sk] rows need every row start on an 8-byte boundary
+  bool vec = (p->sk % 4) == 0;
+  if (a.mask) vec = vec && aligned8(a.mask) && (a.mask_sb % 4) == 0 && (a.mask_sq % 4) == 0;
+  if (a.drop_mask) vec = vec && aligned8(a.drop_mask);
+  if (a.save_softmax) vec = vec && aligned8(a.save_softmax);
+  if (a.save_dropout) vec = vec && aligned8(a.save_dropout);
+  a.mask_vec = vec ? 1 : 0;
+  a.bh = p->bh; a.sq = p->sq; a.sk = p->sk;
+  a.nqt = 0;
+  a.scale_l2 = p->scale * FMHA_LOG2E;
+  a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
+  a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
+  a.flags = p->flags;
+
+  FwdVariant v;
+  v.mask = a.mask != nullptr;
+  v.causal = p->causal != 0;
+  v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
+  // Two query blocks per wave halve the LDS traffic per MFMA; use them once there is
+  // enough work to fill the chip with 256-row tiles.
+  v.qb = (p->sq >= 256 && (long long)p->bh * ((p->sq + 255) / 256) >= 512) ? 2 : 1;
+  const int force = env_int("FMHA_FWD_QB", 0);
+  if (force == 1 || force == 2) v.qb = force;
+
+  hipStream_t s = (hipStream_t)hip_stream;
+  int rc;
+  if (p->dtype == FMHA_DTYPE_F16)
+    rc = p->d == 64 ? fwd_dispatch_f16_d64(a, v, s) : fwd_dispatch_f16_d128(a, v, s);
+  else
+    rc = p->d == 64 ? fwd_dispatch_bf16_d64(a, v, s) : fwd_dispatch_bf16_d128(a, v, s);
+  return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
+}
+
+int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
+  (void)p;
+  (void)hip_stream;
+  return FMHA_E_UNSUPPORTED;
+}
+
+} // extern "C"

@@ -1,0 +1,148 @@
+// Shared device-side building blocks of the gfx950 attention kernels:
+// element-type traits (fp16 / bf16), MFMA 32x32x16 wrappers, the LDS transpose
+// read, cross-half-wave exchange and the Philox4x32-10 dropout rule.
+//
+// Register layouts used throughout (wave64, v_mfma_f32_32x32x16_{f16,bf16}):
+//   A operand: lane l holds row (l % 32), contraction indices 8*(l / 32) .. +7
+//   B operand: lane l holds col (l % 32), contraction indices 8*(l / 32) .. +7
+//   C/D      : lane l holds col (l % 32); register r (0..15) is row
+//              8*(r / 4) + 4*(l / 32) + (r % 4)
+// Because A and B index the contraction dimension the same way, any permutation of
+// that dimension applied to both operands leaves the product unchanged; the kernels
+// use this to feed an accumulator tile straight back in as the B operand of the
+// next product without moving data between lanes.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fmha {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4v __attribute__((__vector_size__(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define FMHA_LOG2E 1.4426950408889634f
+#define FMHA_LN2 0.6931471805599453f
+#define FMHA_DEV __device__ __forceinline__
+
+template <typename T> struct Elem;
+
+template <> struct Elem<_Float16> {
+  using v8 = f16x8;
+  using v4 = f16x4;
+  static FMHA_DEV f32x16 mfma(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <> struct Elem<__bf16> {
+  using v8 = bf16x8;
+  using v4 = bf16x4;
+  static FMHA_DEV f32x16 mfma(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// 16-byte and 8-byte register images used for type-agnostic moves.
+union Pack16 {
+  u32x4 u;
+  f16x8 h;
+  bf16x8 b;
+};
+union Pack8 {
+  u32x2 u;
+  f16x4 h;
+  bf16x4 b;
+  i16x4v s;
+};
+
+template <typename T> FMHA_DEV typename Elem<T>::v8 as_v8(u32x4 u);
+template <> FMHA_DEV f16x8 as_v8<_Float16>(u32x4 u) { Pack16 p; p.u = u; return p.h; }
+template <> FMHA_DEV bf16x8 as_v8<__bf16>(u32x4 u) { Pack16 p; p.u = u; return p.b; }
+
+template <typename T> FMHA_DEV typename Elem<T>::v4 as_v4(u32x2 u);
+template <> FMHA_DEV f16x4 as_v4<_Float16>(u32x2 u) { Pack8 p; p.u = u; return p.h; }
+template <> FMHA_DEV bf16x4 as_v4<__bf16>(u32x2 u) { Pack8 p; p.u = u; return p.b; }
+
+// ds_read_b64_tr_b16: within each group of 16 lanes the instruction reads a
+// 4 (rows) x 16 (cols) matrix of 16-bit elements -- lane i of the group supplies
+// the address of row i/4, columns 4*(i%4)..+3 -- and returns to lane i the four
+// row values of column i.  `byte_addr` is an LDS byte address.
+FMHA_DEV u32x2 lds_read_tr16(const char *lds_ptr) {
+  typedef __attribute__((address_space(3))) i16x4v lds_vec;
+  Pack8 p;
+  p.s = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_vec *)(lds_ptr));
+  return p.u;
+}
+
+// Exchange between lane l and lane l^32 (v_permlane32_swap), reduced with max / add.
+FMHA_DEV float xhalf_max(float x) {
+  int v = __float_as_int(x);
+  auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__int_as_float(r[0]), __int_as_float(r[1]));
+}
+FMHA_DEV float xhalf_sum(float x) {
+  int v = __float_as_int(x);
+  auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return __int_as_float(r[0]) + __int_as_float(r[1]);
+}
+
+FMHA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+FMHA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---------------------------------------------------------------- Philox4x32-10
+// Salmon et al., SC'11; constants and round function as in Random123.
+struct Philox {
+  static constexpr uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u;
+  static constexpr uint32_t W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+  static __host__ __device__ inline void run(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                             uint32_t k0, uint32_t k1, uint32_t out[4]) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+      uint64_t p0 = (uint64_t)M0 * c0;
+      uint64_t p1 = (uint64_t)M1 * c2;
+      uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+      uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+      c1 = (uint32_t)p1;
+      c3 = (uint32_t)p0;
+      c0 = n0;
+      c2 = n2;
+      k0 += W0;
+      k1 += W1;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+  }
+};
+
+// Dropout keep rule.  Elements are grouped into 4 (queries) x 4 (keys) blocks and one
+// Philox call serves a block:
+//   key = (seed_lo, seed_hi); ctr = (offset_lo, offset_hi, blk_lo, blk_hi)
+//   blk = (bh * ceil(sq/4) + q/4) * ceil(sk/4) + k/4
+//   random byte of element (q,k) = (out[q%4] >> 8*(k%4)) & 0xff; keep iff byte >= thr
+struct DropCtx {
+  uint32_t seed_lo, seed_hi, off_lo, off_hi;
+  uint32_t thr;
+  uint32_t qb4, kb4; // ceil(sq/4), ceil(sk/4)
+};
+
+// The 32-bit word holding the four key-consecutive random bytes of query row q,
+// keys 4*k4 .. 4*k4+3.
+FMHA_DEV uint32_t drop_word(const DropCtx &c, uint32_t bh, uint32_t q, uint32_t k4) {
+  uint64_t blk = ((uint64_t)bh * c.qb4 + (q >> 2)) * c.kb4 + k4;
+  uint32_t o[4];
+  Philox::run(c.off_lo, c.off_hi, (uint32_t)blk, (uint32_t)(blk >> 32), c.seed_lo, c.seed_hi, o);
+  uint32_t s = q & 3u;
+  return s == 0 ? o[0] : s == 1 ? o[1] : s == 2 ? o[2] : o[3];
+}
+
+FMHA_DEV bool drop_keep_byte(uint32_t word, int t, uint32_t thr) {
+  return ((word >> (8 * t)) & 0xffu) >= thr;
+}
+
+} // namespace fmha

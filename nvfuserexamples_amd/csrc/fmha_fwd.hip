@@ -1,0 +1,56 @@
+// Instantiates the forward kernel for one (element type, head dim) pair, chosen with
+// -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128}, and exports its dispatcher.
+#include "fmha_launch.h"
+
+#if FMHA_TU_BF16
+#define FMHA_TU_T __bf16
+#define FMHA_TU_TNAME bf16
+#else
+#define FMHA_TU_T _Float16
+#define FMHA_TU_TNAME f16
+#endif
+#define FMHA_CAT3(a, b, c) a##b##_d##c
+#define FMHA_NAME(t, d) FMHA_CAT3(fwd_dispatch_, t, d)
+
+namespace fmha {
+namespace {
+
+constexpr int kNW = 4;
+
+template <int QB, bool MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
+  using Cfg = FwdCfg<FMHA_TU_D>;
+  auto kern = fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+  if (attr != hipSuccess) return 2;
+  constexpr int QT = kNW * QB * 32;
+  a.nqt = (a.sq + QT - 1) / QT;
+  const long long nblk = (long long)a.bh * a.nqt;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(kNW * 64), Cfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+template <int QB, bool MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
+  if (drop == 0) return launch<QB, MASK, CAUSAL, 0>(a, s);
+  if (drop == 1) return launch<QB, MASK, CAUSAL, 1>(a, s);
+  return 1;
+}
+
+template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
+  if (v.mask) return v.causal ? by_drop<QB, true, true>(a, v.drop, s) : by_drop<QB, true, false>(a, v.drop, s);
+  return v.causal ? by_drop<QB, false, true>(a, v.drop, s) : by_drop<QB, false, false>(a, v.drop, s);
+}
+
+} // namespace
+
+int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
+  if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
+    if (v.causal) return 1;
+    return v.mask ? launch<1, true, false, 2>(a, s) : launch<1, false, false, 2>(a, s);
+  }
+  if (v.qb == 2) return by_mask<2>(a, v, s);
+  return by_mask<1>(a, v, s);
+}
+
+} // namespace fmha

@@ -1,0 +1,24 @@
+// Internal interface between the C-ABI translation unit and the per-(element type,
+// head dim) kernel translation units.  Each kernel TU is compiled once per
+// combination with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} and exports one
+// dispatcher per pass.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "fmha_fwd_kernel.h"
+
+namespace fmha {
+
+struct FwdVariant {
+  int qb;       // 32-query blocks per wave (1 or 2)
+  bool mask;    // a mask tensor is read
+  bool causal;
+  int drop;     // 0 none, 1 Philox, 2 tensor / save-intermediates
+};
+
+// Return 0 on success, 1 if the variant is not built, 2 if the launch failed.
+int fwd_dispatch_f16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_f16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_bf16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_bf16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+
+} // namespace fmha
