@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fused multi-head attention on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic input, launched
+through the C ABI (``libfmha_hip.so``) on torch's current HIP stream:
+
+  workload "fwd"     BERT-large attention forward, B32 H16 S512 D64 fp16, additive
+                     [B,1,1,S] padding mask (valid length U{256..512}), scale 1/8
+  workload "fwdbwd"  the same shape as a train step: forward (saving the row
+                     log-sum-exp) + backward, Philox dropout p=0.1
+
+Inputs are resident in HBM before the timed region; several input sets are rotated
+so that consecutive steps do not find their operands in the 256 MB last-level cache.
+Prints ONE JSON line.  ``value`` is forward TFLOP/s (4*BH*S*S*D flops per step); the
+train-step figure (14*BH*S*S*D) rides along under ``fwd_bwd`` when that path is built.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
+PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
+
+B, H, S, D = 32, 16, 512, 64
+
+
+def make_inputs(torch, capi, nsets, seed=0, train=False):
+    g = torch.Generator().manual_seed(seed)
+    sets = []
+    for i in range(nsets):
+        q, k, v = (torch.randn(B * H, S, D, generator=g).to(torch.float16).cuda() for _ in range(3))
+        lens = torch.randint(S // 2, S + 1, (B,), generator=g)
+        mask = torch.zeros(B, 1, 1, S)
+        for b in range(B):
+            mask[b, 0, 0, lens[b]:] = -10000.0
+        mask = mask.to(torch.float16).cuda()
+        d = dict(q=q, k=k, v=v, mask=mask, o=torch.empty_like(q))
+        if train:
+            d["dout"] = torch.randn(B * H, S, D, generator=g).to(torch.float16).cuda()
+            d["lse"] = torch.empty(B * H, S, dtype=torch.float32, device="cuda")
+            d["delta"] = torch.empty(B * H, S, dtype=torch.float32, device="cuda")
+            d["dq"], d["dk"], d["dv"] = (torch.empty_like(q) for _ in range(3))
+        sets.append(d)
+    return sets
+
+
+def fwd_params(capi, t, train=False):
+    P = capi.FwdParams()
+    P.q, P.k, P.v, P.o = (t[n].data_ptr() for n in ("q", "k", "v", "o"))
+    P.mask, P.mask_kind = t["mask"].data_ptr(), capi.MASK_ADDITIVE
+    P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = H, S, 0
+    P.bh, P.sq, P.sk, P.d = B * H, S, S, D
+    P.dtype, P.scale = capi.F16, 0.125
+    if train:
+        P.lse = t["lse"].data_ptr()
+        P.drop_kind, P.p_drop, P.drop_scale = capi.DROP_PHILOX, 0.1, 1.0 / 0.9
+        P.seed, P.offset = 0x1234, 0
+    return P
+
+
+def bwd_params(capi, t):
+    P = capi.BwdParams()
+    for n in ("q", "k", "v", "o", "dout", "lse", "delta", "dq", "dk", "dv"):
+        setattr(P, n, t[n].data_ptr())
+    P.mask, P.mask_kind = t["mask"].data_ptr(), capi.MASK_ADDITIVE
+    P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = H, S, 0
+    P.bh, P.sq, P.sk, P.d = B * H, S, S, D
+    P.dtype, P.scale = capi.F16, 0.125
+    P.drop_kind, P.p_drop, P.drop_scale = capi.DROP_PHILOX, 0.1, 1.0 / 0.9
+    P.seed, P.offset = 0x1234, 0
+    return P
+
+
+def time_steps(torch, step, steps, warmup):
+    """HIP events on the stream the kernels are launched on (torch's current stream)."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall / steps
+
+
+def cpu_baseline(torch, budget_s=12.0):
+    """The reference's eager composition (its ground truth) on the host cores, fp32,
+    on the reference-sized CPU case B8 H12 S128 D64 with a [B,1,1,S] padding mask."""
+    from oracle import eager
+    b, h, s, d = 8, 12, 128, 64
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(b * h, s, d, generator=g) for _ in range(3))
+    lens = torch.randint(s // 2, s + 1, (b,), generator=g)
+    keep = torch.zeros(b, 1, s)
+    for i in range(b):
+        keep[i, 0, :lens[i]] = 1.0
+    keep = keep.repeat_interleave(h, 0)  # [bh,1,s] 0/1 mask as the inference op takes it
+    cores = torch.get_num_threads()
+    for _ in range(3):
+        eager.infer_mha(q, k, v, keep)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        eager.infer_mha(q, k, v, keep)
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 2000:
+            break
+    flops = 4.0 * b * h * s * s * d
+    return {"value": round(flops * n / el / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{n} iterations of the eager fp32 composition (matmul, mask add, softmax, matmul) at "
+                      f"B{b} H{h} S{s} D{d} in {el:.1f} s, torch CPU with {cores} threads",
+            "ms_per_iter": round(el / n * 1e3, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--sets", type=int, default=4, help="input sets rotated to defeat the last-level cache")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-bwd", action="store_true", help="skip the train-step (fwd+bwd) leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; attention shards over batch*heads without "
+              "communication, so N GPUs would each run this same kernel on their slice. Use --gpus 1.",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from nvfuserexamples_amd import capi
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    L = capi.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    # ---- forward (headline)
+    sets = make_inputs(torch, capi, args.sets)
+    fps = [fwd_params(capi, t) for t in sets]
+    rc = L.fmha_fwd_launch(C.byref(fps[0]), stream)
+    capi.check(rc)
+
+    def fwd_step(i):
+        L.fmha_fwd_launch(C.byref(fps[i % len(fps)]), stream)
+
+    ms, wall_ms = time_steps(torch, fwd_step, args.steps, args.warmup)
+    flops = 4.0 * B * H * S * S * D
+    bytes_ = 4.0 * B * H * S * D * 2 + B * S * 2
+    tflops = flops / (ms * 1e-3) / 1e12
+    # warm-cache figure for reference: one input set only
+    def fwd_warm(i):
+        L.fmha_fwd_launch(C.byref(fps[0]), stream)
+    ms_warm, _ = time_steps(torch, fwd_warm, args.steps, args.warmup)
+    del sets, fps
+
+    out = {
+        "metric": "MHA fwd TFLOP/s (B32,H16,S512,D64 fp16)", "value": round(tflops, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "BERT-large attention forward: B32 H16 S512 D64 fp16, additive [B,1,1,S] "
+                               "padding mask (valid length U{256..512}), scale 1/8, no dropout",
+                   "layout": "[B*H,S,D] contiguous", "input_sets_rotated": args.sets},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_MFMA_TFLOPS, 4), "traffic": None,
+                     "kernel": "fmha_fwd_kernel<f16,D64>", "flops_per_launch": flops,
+                     "algorithmic_bytes_per_launch": bytes_,
+                     "hbm_achieved_GBps": round(bytes_ / (ms * 1e-3) / 1e9, 1),
+                     "hbm_frac": round(bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                     "launch_us": round(ms * 1e3, 2)},
+        "fwd_warm_cache": {"ms_per_step": round(ms_warm, 5),
+                           "tflops": round(flops / (ms_warm * 1e-3) / 1e12, 2)},
+        "host_wall_ms_per_step": round(wall_ms, 5),
+    }
+
+    # ---- train step (forward with LSE + Philox dropout, then backward)
+    if not args.no_bwd:
+        tsets = make_inputs(torch, capi, args.sets, seed=1, train=True)
+        tf = [fwd_params(capi, t, train=True) for t in tsets]
+        tb = [bwd_params(capi, t) for t in tsets]
+        rc_f = L.fmha_fwd_launch(C.byref(tf[0]), stream)
+        rc_b = L.fmha_bwd_launch(C.byref(tb[0]), stream)
+        if rc_f == 0 and rc_b == 0:
+            def train_step(i):
+                L.fmha_fwd_launch(C.byref(tf[i % len(tf)]), stream)
+                L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream)
+            steps = max(10, args.steps // 2)
+            ms_t, _ = time_steps(torch, train_step, steps, max(5, args.warmup // 2))
+            def bwd_step(i):
+                L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream)
+            ms_b, _ = time_steps(torch, bwd_step, steps, max(5, args.warmup // 2))
+            fl_t = 14.0 * B * H * S * S * D
+            out["fwd_bwd"] = {
+                "workload": "same shape, train step: fwd (+LSE) + bwd, Philox dropout p=0.1, padding mask",
+                "ms_per_step": round(ms_t, 5), "tflops": round(fl_t / (ms_t * 1e-3) / 1e12, 2),
+                "frac_of_mfma_peak": round(fl_t / (ms_t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, 4),
+                "bwd_only_ms": round(ms_b, 5),
+                "bwd_only_tflops": round(10.0 * B * H * S * S * D / (ms_b * 1e-3) / 1e12, 2), "steps": steps}
+        else:
+            out["fwd_bwd"] = {"error": f"fwd rc={rc_f} bwd rc={rc_b}: " + L.fmha_strerror(rc_b or rc_f).decode()}
+        del tsets
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -158,8 +158,8 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
 }
 
 int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
-  (void)p;
   (void)hip_stream;
+  if (!p) return FMHA_E_NULL;
   return FMHA_E_UNSUPPORTED;
 }
 

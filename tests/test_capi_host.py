@@ -1,0 +1,108 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what
+include/fmha_capi.h declares, argument validation returns the documented codes before
+anything is launched, and the torch extension registers the reference's operator names
+(reference fmha/fmha_manual.cpp:1240-1250)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+import oracle
+from nvfuserexamples_amd import capi
+from conftest import ROOT
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "fmha_capi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmha_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = capi.lib()
+    names = _declared_functions()
+    assert set(names) == set(capi.EXPORTS)
+    for n in names:
+        assert hasattr(L, n), n
+    assert L.fmha_version().decode().count(".") == 1
+
+
+def test_strerror_and_threshold():
+    L = capi.lib()
+    assert L.fmha_strerror(0) == b"ok"
+    msgs = {L.fmha_strerror(c) for c in range(-7, 1)}
+    assert len(msgs) == 8 and all(msgs)
+    for p in (0.0, 0.05, 0.1, 0.25, 0.5, 0.9, 0.999):
+        assert L.fmha_drop_threshold(p) == oracle.drop_threshold(p)
+
+
+def _valid_params():
+    P = capi.FwdParams()
+    P.q = P.k = P.v = P.o = 0x1000  # never dereferenced: every call below fails validation first
+    P.bh, P.sq, P.sk, P.d = 2, 64, 64, 64
+    P.dtype, P.scale = capi.F16, 0.125
+    return P
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda P: setattr(P, "q", None), -1),
+    (lambda P: setattr(P, "dtype", 7), -2),
+    (lambda P: setattr(P, "d", 80), -3),
+    (lambda P: setattr(P, "sq", 0), -3),
+    (lambda P: setattr(P, "k", 0x1008), -4),
+    (lambda P: setattr(P, "scale", 0.0), -5),
+    (lambda P: setattr(P, "scale", float("nan")), -5),
+    (lambda P: setattr(P, "mask_kind", 9), -5),
+    (lambda P: setattr(P, "mask_kind", 1), -1),                       # mask kind without a pointer
+    (lambda P: (setattr(P, "drop_kind", 1), setattr(P, "p_drop", 1.0)), -5),
+    (lambda P: setattr(P, "drop_kind", 2), -1),                       # tensor dropout without a tensor
+    (lambda P: (setattr(P, "save_softmax", 0x1000), setattr(P, "causal", 1)), -6),
+    (lambda P: (setattr(P, "save_softmax", 0x1000), setattr(P, "drop_kind", 1), setattr(P, "p_drop", 0.1)), -6),
+])
+def test_forward_validation_codes(mutate, code):
+    P = _valid_params()
+    mutate(P)
+    assert capi.lib().fmha_fwd_launch(C.byref(P), None) == code
+
+
+def test_null_params_and_keep_mask_validation():
+    L = capi.lib()
+    assert L.fmha_fwd_launch(None, None) == -1
+    assert L.fmha_bwd_launch(None, None) == -1
+    assert L.fmha_philox_keep_mask(0, 0, 0.1, 1, 4, 4, None, None) == -1
+    assert L.fmha_philox_keep_mask(0, 0, 1.5, 1, 4, 4, 0x1000, None) == -5
+    assert L.fmha_philox_keep_mask(0, 0, 0.1, 0, 4, 4, 0x1000, None) == -3
+
+
+def test_extension_registers_reference_operator_names():
+    import mha_manual  # noqa: F401  (import registers the ops, as in reference test.py:2)
+    for name in ("fmha_nvfuser", "fmha_train_nvfuser", "fmha_train_saveim_nvfuser", "fmha_fwd", "fmha_bwd",
+                 "fmha_philox_keep_mask"):
+        assert hasattr(torch.ops.mha_manual, name)
+    s = torch.ops.mha_manual.fmha_train_saveim_nvfuser.default._schema
+    assert [a.name for a in s.arguments] == ["input", "qk", "v", "pad_mask", "dropout_mask"]
+    assert str(s.returns[0].type) == "List[Tensor]"
+    s = torch.ops.mha_manual.fmha_nvfuser.default._schema
+    assert [a.name for a in s.arguments] == ["input", "qk", "v", "amask"]
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    """There is no CPU implementation behind the ops: CPU tensors must raise, not fall back."""
+    import mha_manual  # noqa: F401
+    z = torch.zeros(1, 4, 64, dtype=torch.float16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        torch.ops.mha_manual.fmha_nvfuser(z, z, z, torch.zeros(1, 4, 4, dtype=torch.float16))
+
+
+def test_package_has_no_oracle_dependency():
+    """The shipped code may not import or call the CPU oracle."""
+    pkg = os.path.join(ROOT, "nvfuserexamples_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text and "fmha_oracle" not in text, f
+    text = open(os.path.join(ROOT, "fmha", "fmha_manual.cpp")).read()
+    assert "oracle" not in text

@@ -1,0 +1,152 @@
+"""GPU parity of the forward path, called through the C ABI (ctypes -> libfmha_hip.so).
+
+Bars (fp16): max |O - oracle| <= 2e-3 against the unrounded fp64-accumulated oracle of the
+eager composition (reference test.py:12-18); bf16 is held to 2e-2 (8-bit mantissa: the
+probabilities and the output each carry 2^-9 relative rounding).  The reference itself
+asserts atol=1e-2 (test.py:29).  Dropout keep decisions are bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nvfuserexamples_amd import capi
+from conftest import make_qkv, pad_mask, f32
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"fp16": 2e-3, "bf16": 2e-2}
+TDT = {"fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+def _run(q, k, v, **kw):
+    out = capi.fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+CASES = [
+    # bh, sq, sk, d, dtype, mask, causal
+    (4, 128, 128, 64, "fp16", None, False),
+    (4, 128, 128, 64, "fp16", "keep01", False),       # the reference's inference op layout
+    (6, 128, 128, 64, "fp16", "pad", False),          # [B,1,1,S] padding mask, B = 3
+    (4, 512, 512, 64, "fp16", "pad", False),          # headline sequence length
+    (2, 512, 512, 64, "fp16", "add_full", False),
+    (3, 100, 77, 64, "fp16", None, False),            # ragged
+    (2, 1, 1, 64, "fp16", None, False),               # one query, one key
+    (2, 33, 257, 64, "fp16", "add_full", False),      # ragged, mask rows not 8-byte aligned
+    (2, 320, 320, 64, "fp16", None, True),            # causal
+    (2, 200, 200, 64, "fp16", "pad", True),           # causal + padding
+    (2, 2048, 2048, 64, "fp16", None, False),         # long sequence: many K/V tiles
+    (2, 256, 256, 128, "fp16", None, False),
+    (2, 1024, 1024, 128, "bf16", None, True),         # wide-head bf16 causal
+    (4, 192, 192, 64, "bf16", "pad", False),
+]
+
+
+@pytest.mark.parametrize("qb", [1, 2])
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,mask,causal", CASES)
+def test_forward_matches_oracle(bh, sq, sk, d, dtype, mask, causal, qb, monkeypatch):
+    monkeypatch.setenv("FMHA_FWD_QB", str(qb))
+    std = 0.5 if d == 128 else 1.0
+    q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sq, std=std, dtype=dtype)
+    m, mk = None, capi.MASK_ADDITIVE
+    g = torch.Generator().manual_seed(sq)
+    if mask == "pad":
+        m = pad_mask(bh // 2, sk, sk // 2, sk)
+    elif mask == "keep01":
+        m, mk = torch.empty(bh, sq, sk).random_(2, generator=g), capi.MASK_KEEP01
+    elif mask == "add_full":
+        m = torch.randn(bh, sq, sk, generator=g) * 2
+    if m is not None:
+        m = m.to(TDT[dtype])
+    o, lse, _, _ = _run(q, k, v, mask=None if m is None else m.cuda(), mask_kind=mk, causal=causal, want_lse=True)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=None if m is None else f32(m),
+                           mask_kind="keep01" if mk == capi.MASK_KEEP01 else "additive", causal=causal,
+                           want=("o", "lse"))
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= TOL[dtype]
+    assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= 1e-3
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,causal", [(3, 128, 192, 64, False), (2, 257, 257, 64, True),
+                                                (2, 128, 128, 128, False)])
+def test_philox_dropout_forward_and_mask_bit_exact(bh, sq, sk, d, causal):
+    q, k, v = make_qkv(bh, sq, sk, d, seed=3)
+    seed, offset, p = 0xfeedbeefcafe, (1 << 33) + 5, 0.1
+    o, lse, _, _ = _run(q, k, v, causal=causal, drop_kind=capi.DROP_PHILOX, p_drop=p, seed=seed, offset=offset,
+                        want_lse=True)
+    ref = oracle.attention(f32(q), f32(k), f32(v), causal=causal, philox=True, p_drop=p, drop_scale=1 / (1 - p),
+                           seed=seed, offset=offset, want=("o", "lse"))
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= 2e-3
+    assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= 1e-3
+    # the keep decisions themselves: GPU materialisation == CPU rule, bit for bit
+    km = capi.philox_keep_mask(seed, offset, p, bh, sq, sk).cpu().numpy()
+    assert np.array_equal(km, oracle.keep_mask(seed, offset, p, bh, sq, sk))
+    # and the fused kernel used exactly those decisions: feeding them back as an explicit
+    # dropout tensor reproduces its output to rounding
+    o2, _, _, _ = _run(q, k, v, drop_kind=capi.DROP_TENSOR, drop_mask=torch.from_numpy(km).to(q.dtype).cuda(),
+                       drop_scale=1 / (1 - p)) if not causal else (o, None, None, None)
+    assert np.abs(f32(o2.cpu()) - f32(o.cpu())).max() <= 1e-3
+
+
+def test_train_ops_and_saved_intermediates():
+    """Reference train semantics (test_train_mha.py:14-21) incl. the saved softmax / dropout tensors;
+    the zero pattern of the dropped output is the caller's mask, exactly."""
+    bh, s, d = 8, 128, 64
+    q, k, v = make_qkv(bh, s, s, d, seed=8)
+    g = torch.Generator().manual_seed(2)
+    pm = (torch.empty(bh, s, s).random_(2, generator=g) * -1000).half()
+    dm = torch.empty(bh, s, s).random_(2, generator=g).half()
+    o, _, sm, dr = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0,
+                        save=True)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(pm), drop_mask=f32(dm), drop_scale=2.0,
+                           want=("o", "softmax", "dropout"))
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= 4e-3   # O is up to 2x larger here (x2 scaling)
+    assert np.abs(f32(sm.cpu()) - ref["softmax"]).max() <= 1e-3
+    assert np.abs(f32(dr.cpu()) - ref["dropout"]).max() <= 2e-3
+    live = ref["softmax"] > 1e-6
+    assert np.array_equal((f32(dr.cpu()) == 0)[live], (f32(dm) == 0)[live])
+    o2, _, _, _ = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0)
+    assert torch.equal(o2, o)  # the save pass does not disturb O
+
+
+def test_size_independent_properties_at_headline_shape():
+    """B32 H16 S512 D64 (full size): properties that need no CPU answer, plus oracle parity on a
+    sample of heads."""
+    B, H, S, D = 32, 16, 512, 64
+    q, k, v = make_qkv(B * H, S, S, D, seed=0)
+    m = pad_mask(B, S, S // 2, S).half()
+    qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), m.cuda()
+    o = capi.fwd(qc, kc, vc, mask=mc)[0]
+    # permuting the keys (K, V and the mask together) leaves O unchanged up to rounding
+    perm = torch.randperm(S, generator=torch.Generator().manual_seed(1)).cuda()
+    o_p = capi.fwd(qc, kc[:, perm].contiguous(), vc[:, perm].contiguous(), mask=mc[..., perm].contiguous())[0]
+    assert (o_p.float() - o.float()).abs().max().item() <= 2e-3
+    # linear in V
+    v2 = make_qkv(B * H, S, S, D, seed=5)[2].cuda()
+    o_a = capi.fwd(qc, kc, v2, mask=mc)[0]
+    o_s = capi.fwd(qc, kc, (vc.float() + v2.float()).half(), mask=mc)[0]
+    assert (o_s.float() - (o.float() + o_a.float())).abs().max().item() <= 6e-3
+    # masked keys carry no weight: scrambling V on the padded tail changes nothing
+    lens = (m[:, 0, 0] == 0).sum(-1)
+    v3 = vc.clone().view(B, H, S, D)
+    for b in range(B):
+        v3[b, :, lens[b]:] = 100.0
+    o_t = capi.fwd(qc, kc, v3.view(B * H, S, D), mask=mc)[0]
+    assert torch.equal(o_t, o)
+    torch.cuda.synchronize()
+    heads = [0, 17, 255, 511]
+    ref = oracle.attention(f32(q[heads]), f32(k[heads]), f32(v[heads]),
+                           mask=f32(m[[h // H for h in heads]]).reshape(len(heads), 1, S))["o"]
+    assert np.abs(f32(o[heads].cpu()) - ref).max() <= 2e-3
+
+
+def test_golden_fixture():
+    """Committed seeded vectors (tests/golden/make_fixtures.py): inputs and oracle outputs."""
+    import os
+    f = np.load(os.path.join(os.path.dirname(__file__), "golden", "fwd_small.npz"))
+    q, k, v, m = (torch.from_numpy(f[n]).half() for n in ("q", "k", "v", "mask"))
+    o, lse, _, _ = _run(q, k, v, mask=m.cuda(), drop_kind=capi.DROP_PHILOX, p_drop=float(f["p_drop"]),
+                        seed=int(f["seed"]), offset=int(f["offset"]), want_lse=True)
+    assert np.abs(f32(o.cpu()) - f["o"]).max() <= 2e-3
+    assert np.abs(lse.cpu().numpy() - f["lse"]).max() <= 1e-3
