@@ -1,0 +1,60 @@
+// Instantiates the backward kernels for one (element type, head dim) pair, chosen with
+// -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128}, and exports their dispatcher.
+#include "fmha_launch.h"
+
+#if FMHA_TU_BF16
+#define FMHA_TU_T __bf16
+#define FMHA_TU_TNAME bf16
+#else
+#define FMHA_TU_T _Float16
+#define FMHA_TU_TNAME f16
+#endif
+#define FMHA_CAT3(a, b, c) a##b##_d##c
+#define FMHA_NAME(t, d) FMHA_CAT3(bwd_dispatch_, t, d)
+
+namespace fmha {
+namespace {
+
+constexpr int kNW = 4;
+constexpr int kQB = 1; // 32-query blocks per wave in the dQ kernel
+constexpr int kKB = 1; // 32-key blocks per wave in the dK/dV kernel
+
+template <typename K> int set_lds(K kern, int bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                             bytes) == hipSuccess ? 0 : 2;
+}
+
+template <bool MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s) {
+  using Cfg = BwdCfg<FMHA_TU_D>;
+  auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP>;
+  auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP>;
+  static const int attr = set_lds(kq, Cfg::LDS_BYTES) | set_lds(kk, Cfg::LDS_BYTES);
+  if (attr) return 2;
+  constexpr int QT = kNW * kQB * 32, KT = kNW * kKB * 32;
+  // dQ first: it also writes delta, which the dK/dV kernel reads (same stream => ordered)
+  a.ntile = (a.sq + QT - 1) / QT;
+  long long nblk = (long long)a.bh * a.ntile;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kq, dim3((unsigned)nblk), dim3(kNW * 64), Cfg::LDS_BYTES, s, a);
+  if (hipGetLastError() != hipSuccess) return 2;
+  a.ntile = (a.sk + KT - 1) / KT;
+  nblk = (long long)a.bh * a.ntile;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kk, dim3((unsigned)nblk), dim3(kNW * 64), Cfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+template <bool MASK, bool CAUSAL> int by_drop(BwdArgs &a, int drop, hipStream_t s) {
+  if (drop == 0) return launch<MASK, CAUSAL, 0>(a, s);
+  if (drop == 1) return launch<MASK, CAUSAL, 1>(a, s);
+  return 1;
+}
+
+} // namespace
+
+int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
+  if (v.mask) return v.causal ? by_drop<true, true>(a, v.drop, s) : by_drop<true, false>(a, v.drop, s);
+  return v.causal ? by_drop<false, true>(a, v.drop, s) : by_drop<false, false>(a, v.drop, s);
+}
+
+} // namespace fmha

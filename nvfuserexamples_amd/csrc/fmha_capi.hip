@@ -65,7 +65,7 @@ const char *fmha_strerror(int code) {
   case FMHA_E_SHAPE: return "bad shape: sizes must be positive and head dim must be 64 or 128";
   case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned";
   case FMHA_E_ARG: return "argument out of range (scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
-  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox)";
+  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox; the backward takes Philox dropout only)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
   default: return "unknown error code";
   }
@@ -158,9 +158,62 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
 }
 
 int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
-  (void)hip_stream;
-  if (!p) return FMHA_E_NULL;
-  return FMHA_E_UNSUPPORTED;
+  if (!p || !p->q || !p->k || !p->v || !p->o || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk || !p->dv)
+    return FMHA_E_NULL;
+  if (p->dtype != FMHA_DTYPE_F16 && p->dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
+  if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;
+  if (p->d != 64 && p->d != 128) return FMHA_E_SHAPE;
+  if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->o) || !aligned16(p->dout) ||
+      !aligned16(p->dq) || !aligned16(p->dk) || !aligned16(p->dv))
+    return FMHA_E_ALIGN;
+  if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return FMHA_E_ARG;
+  if (p->mask_kind < FMHA_MASK_NONE || p->mask_kind > FMHA_MASK_KEEP01) return FMHA_E_ARG;
+  if (p->drop_kind < FMHA_DROP_NONE || p->drop_kind > FMHA_DROP_TENSOR) return FMHA_E_ARG;
+  if (p->mask_kind != FMHA_MASK_NONE) {
+    if (!p->mask) return FMHA_E_NULL;
+    if (p->mask_bh_div < 1 || p->mask_stride_b < 0 || p->mask_stride_q < 0) return FMHA_E_ARG;
+  }
+  if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
+  if (p->drop_kind == FMHA_DROP_PHILOX && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
+  if (p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED; // backward regenerates Philox decisions only
+
+  BwdArgs a;
+  a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.dout = p->dout;
+  a.lse = p->lse; a.delta = p->delta;
+  a.dq = p->dq; a.dk = p->dk; a.dv = p->dv;
+  a.mask = p->mask_kind ? p->mask : nullptr;
+  a.mask_sb = p->mask_stride_b;
+  a.mask_sq = p->mask_stride_q;
+  a.mask_div = p->mask_kind ? (int32_t)p->mask_bh_div : 1;
+  if (p->mask_kind == FMHA_MASK_KEEP01) {
+    a.mask_a = -p->mask_neg * FMHA_LOG2E;
+    a.mask_b = p->mask_neg * FMHA_LOG2E;
+  } else {
+    a.mask_a = FMHA_LOG2E;
+    a.mask_b = 0.f;
+  }
+  bool vec = (p->sk % 4) == 0;
+  if (a.mask) vec = vec && aligned8(a.mask) && (a.mask_sb % 4) == 0 && (a.mask_sq % 4) == 0;
+  a.mask_vec = vec ? 1 : 0;
+  a.bh = p->bh; a.sq = p->sq; a.sk = p->sk;
+  a.ntile = 0;
+  a.scale = p->scale;
+  a.scale_l2 = p->scale * FMHA_LOG2E;
+  a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
+  a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
+  a.flags = p->flags;
+
+  BwdVariant v;
+  v.mask = a.mask != nullptr;
+  v.causal = p->causal != 0;
+  v.drop = p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0;
+  hipStream_t s = (hipStream_t)hip_stream;
+  int rc;
+  if (p->dtype == FMHA_DTYPE_F16)
+    rc = p->d == 64 ? bwd_dispatch_f16_d64(a, v, s) : bwd_dispatch_f16_d128(a, v, s);
+  else
+    rc = p->d == 64 ? bwd_dispatch_bf16_d64(a, v, s) : bwd_dispatch_bf16_d128(a, v, s);
+  return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 
 } // extern "C"

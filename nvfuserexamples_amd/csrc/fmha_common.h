@@ -81,6 +81,24 @@ FMHA_DEV u32x2 lds_read_tr16(const char *lds_ptr) {
   return p.u;
 }
 
+// A operand (32 rows x 16 contraction indices) of a product whose contraction index runs
+// over the ROWS of a row-major LDS tile (pitch ROWB bytes) and whose output rows run over
+// its columns -- i.e. the tile is consumed transposed.  For lane l (c32 = l%32, h = l/32)
+// and step c the eight contraction indices are rows
+//   row0 + 4h + 16c + {0,1,2,3, 8,9,10,11}
+// which is the order in which a 32x32 accumulator tile (lane = column, registers = rows)
+// presents them when it is fed back as the B operand; the column is col0 + c32.
+template <typename T, int ROWB>
+FMHA_DEV typename Elem<T>::v8 lds_load_a_transposed(const char *tile, int row0, int col0, int c, int l) {
+  const int i16 = l & 15;
+  const int h = l >> 5;
+  const char *p0 = tile + (row0 + 4 * h + 16 * c + (i16 >> 2)) * ROWB + (col0 + (l & 16) + 4 * (i16 & 3)) * 2;
+  const u32x2 lo = lds_read_tr16(p0);
+  const u32x2 hi = lds_read_tr16(p0 + 8 * ROWB);
+  const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
+  return as_v8<T>(both);
+}
+
 // Exchange between lane l and lane l^32 (v_permlane32_swap), reduced with max / add.
 FMHA_DEV float xhalf_max(float x) {
   int v = __float_as_int(x);
@@ -139,6 +157,12 @@ FMHA_DEV uint32_t drop_word(const DropCtx &c, uint32_t bh, uint32_t q, uint32_t 
   Philox::run(c.off_lo, c.off_hi, (uint32_t)blk, (uint32_t)(blk >> 32), c.seed_lo, c.seed_hi, o);
   uint32_t s = q & 3u;
   return s == 0 ? o[0] : s == 1 ? o[1] : s == 2 ? o[2] : o[3];
+}
+
+// All four words of the block holding query rows 4*q4..4*q4+3 and keys 4*k4..4*k4+3.
+FMHA_DEV void drop_block(const DropCtx &c, uint32_t bh, uint32_t q4, uint32_t k4, uint32_t o[4]) {
+  uint64_t blk = ((uint64_t)bh * c.qb4 + q4) * c.kb4 + k4;
+  Philox::run(c.off_lo, c.off_hi, (uint32_t)blk, (uint32_t)(blk >> 32), c.seed_lo, c.seed_hi, o);
 }
 
 FMHA_DEV bool drop_keep_byte(uint32_t word, int t, uint32_t thr) {

@@ -5,6 +5,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include "fmha_fwd_kernel.h"
+#include "fmha_bwd_kernel.h"
 
 namespace fmha {
 
@@ -20,5 +21,16 @@ int fwd_dispatch_f16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+
+struct BwdVariant {
+  bool mask;
+  bool causal;
+  int drop; // 0 none, 1 Philox
+};
+
+int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_f16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_bf16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_bf16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 
 } // namespace fmha

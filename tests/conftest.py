@@ -45,5 +45,7 @@ def f32(t):
     return t.float().numpy()
 
 
-def rel_to_max(a, b):
-    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+def rel_to_max(a, b, floor=1e-30):
+    """max |a-b| relative to max |b|; `floor` keeps exactly-zero answers (e.g. the gradient of a
+    one-key softmax) from turning rounding dust into an infinite ratio."""
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), floor))
