@@ -25,6 +25,10 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 VALU forms stay off on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # keep MFMA accumulators in architectural VGPRs (no AGPR round trips before the softmax VALU work)
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # the kernels use +-inf deliberately but never produce or consume NaN
+    "-fno-honor-nans",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -134,12 +134,13 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   a.bh = p->bh; a.sq = p->sq; a.sk = p->sk;
   a.nqt = 0;
   a.scale_l2 = p->scale * FMHA_LOG2E;
+  a.inv_scale_l2 = 1.f / a.scale_l2;
   a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
 
   FwdVariant v;
-  v.mask = a.mask != nullptr;
+  v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
   // Two query blocks per wave halve the LDS traffic per MFMA; use them once there is

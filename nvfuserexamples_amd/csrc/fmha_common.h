@@ -111,6 +111,7 @@ FMHA_DEV float xhalf_sum(float x) {
   return __int_as_float(r[0]) + __int_as_float(r[1]);
 }
 
+FMHA_DEV float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 FMHA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 FMHA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -17,7 +17,7 @@ namespace {
 
 constexpr int kNW = 4;
 
-template <int QB, bool MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
+template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
   using Cfg = FwdCfg<FMHA_TU_D>;
   auto kern = fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
   static const hipError_t attr = hipFuncSetAttribute(
@@ -31,15 +31,20 @@ template <int QB, bool MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipSt
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
-template <int QB, bool MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
+template <int QB, int MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<QB, MASK, CAUSAL, 0>(a, s);
   if (drop == 1) return launch<QB, MASK, CAUSAL, 1>(a, s);
   return 1;
 }
 
+template <int QB, int MASK> int by_causal(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
+  return v.causal ? by_drop<QB, MASK, true>(a, v.drop, s) : by_drop<QB, MASK, false>(a, v.drop, s);
+}
+
 template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
-  if (v.mask) return v.causal ? by_drop<QB, true, true>(a, v.drop, s) : by_drop<QB, true, false>(a, v.drop, s);
-  return v.causal ? by_drop<QB, false, true>(a, v.drop, s) : by_drop<QB, false, false>(a, v.drop, s);
+  if (v.mask == kMaskPerKey) return by_causal<QB, kMaskPerKey>(a, v, s);
+  if (v.mask == kMaskFull) return by_causal<QB, kMaskFull>(a, v, s);
+  return by_causal<QB, kMaskNone>(a, v, s);
 }
 
 } // namespace
@@ -47,9 +52,14 @@ template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;
-    return v.mask ? launch<1, true, false, 2>(a, s) : launch<1, false, false, 2>(a, s);
+    if (v.mask == kMaskPerKey) return launch<1, kMaskPerKey, false, 2>(a, s);
+    if (v.mask == kMaskFull) return launch<1, kMaskFull, false, 2>(a, s);
+    return launch<1, kMaskNone, false, 2>(a, s);
   }
+#if FMHA_TU_D == 64
+  // two query blocks per wave only where their accumulators fit the register file
   if (v.qb == 2) return by_mask<2>(a, v, s);
+#endif
   return by_mask<1>(a, v, s);
 }
 

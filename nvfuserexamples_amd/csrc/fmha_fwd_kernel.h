@@ -17,9 +17,18 @@
 // The accumulator layout of S^T (lane = query, registers = keys) is exactly the B
 // operand layout of the second product under a fixed permutation of the key index,
 // and V is fetched with that same permutation, so P never leaves registers.
-// Row max needs one exchange between lane l and l^32 per tile; row sums are kept
-// per lane and combined once at the end.
+//
+// Softmax bookkeeping per lane (one query): a reference exponent m, a partial sum l
+// of the ROUNDED probabilities (accumulated with v_dot2 on the packed pairs, so the
+// denominator matches what the second product actually sums) and the unnormalised
+// accumulator O^T.  The reference m is raised -- and l, O rescaled -- only when a
+// tile's maximum exceeds it by more than 2^8, which keeps every probability below
+// 256 (exact in fp16/bf16 range) and removes the rescale from almost every tile.
+// Row max needs one exchange between lane l and l^32 per tile; the two half-wave
+// partial sums are combined once in the epilogue.
 #pragma once
+#include <type_traits>
+
 #include "fmha_common.h"
 
 namespace fmha {
@@ -33,15 +42,19 @@ struct FwdArgs {
   void *save_softmax, *save_dropout;
   int64_t mask_sb, mask_sq;
   int32_t mask_div;
-  int32_t mask_vec;  // 1: 8-byte mask/drop/save accesses are aligned
+  int32_t mask_vec;  // 1: 8-byte accesses to [.., sk] rows (mask, drop mask, saves) are aligned
   float mask_a, mask_b; // mask term in log2 units = mask_value * mask_a + mask_b
   int32_t bh, sq, sk;
   int32_t nqt;       // query tiles per head
   float scale_l2;    // scale * log2(e)
+  float inv_scale_l2; // 1 / scale_l2
   float drop_scale;
   DropCtx drop;
-  int32_t flags;     // bit0: gather V operands with 16-bit LDS reads instead of the transpose read
+  int32_t flags;
 };
+
+// how the mask tensor is read
+enum { kMaskNone = 0, kMaskPerKey = 1, kMaskFull = 2 };
 
 template <int D> struct FwdCfg {
   static constexpr int BK = 64;           // keys per LDS tile
@@ -50,10 +63,24 @@ template <int D> struct FwdCfg {
   static constexpr int DB = D / 32;       // 32-row blocks of O^T
   static constexpr int ROWB = D * 2 + 16; // LDS row pitch in bytes (16 B pad: conflict-free b128 reads)
   static constexpr int TILEB = BK * ROWB;
-  static constexpr int LDS_BYTES = 4 * TILEB; // {K,V} x 2 stages
+  static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * 4; // {K,V} x 2 stages + per-key mask terms x 2 stages
 };
 
-template <typename T, int D, int QB, int NW, bool MASK, bool CAUSAL, int DROP>
+template <typename T> FMHA_DEV float dot2_ones(typename Elem<T>::v8 v, int pair, float acc);
+template <> FMHA_DEV float dot2_ones<_Float16>(f16x8 v, int pair, float acc) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const h2 one = {(_Float16)1.f, (_Float16)1.f};
+  const h2 x = {v[2 * pair], v[2 * pair + 1]};
+  return __builtin_amdgcn_fdot2(x, one, acc, false);
+}
+template <> FMHA_DEV float dot2_ones<__bf16>(bf16x8 v, int pair, float acc) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  const b2 one = {(__bf16)1.f, (__bf16)1.f};
+  const b2 x = {v[2 * pair], v[2 * pair + 1]};
+  return __builtin_amdgcn_fdot2_f32_bf16(x, one, acc, false);
+}
+
+template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
 __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
@@ -66,9 +93,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   constexpr int CPR = D / 8;                 // 16-byte chunks per row
   constexpr int CPT = BK * CPR / NT;         // chunks per thread per tile
   static_assert(BK * CPR % NT == 0, "tile must divide evenly over the workgroup");
+  static_assert(NT >= BK, "per-key mask terms are staged by the first BK threads");
   constexpr float NEG_INF = -__builtin_inff();
+  constexpr float RESCALE_TH = 8.f; // log2 units
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  float *ldsMask = (float *)(lds + 4 * TILEB);
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -90,6 +120,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
   const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
   const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+  const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
   // ---- Q operand registers
   v8 qreg[QB][KS];
@@ -115,6 +146,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
   // ---- tile staging: global -> registers -> LDS
   u32x4 kst[CPT], vst[CPT];
+  float mst = 0.f;
   auto gload = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
@@ -129,6 +161,13 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       kst[i] = kk;
       vst[i] = vv;
     }
+    if (MASK == kMaskPerKey && tid < BK) {
+      // additive term of key k0+tid, divided by the score scale so that it can seed the
+      // accumulator of K.Q^T (the product then comes out as score + term/scale and one fma
+      // finishes it); keys past the end get -inf, which also covers the ragged last tile
+      const int kr = k0 + tid;
+      mst = kr < a.sk ? fmaf((float)mkey[kr], a.mask_a, a.mask_b) * a.inv_scale_l2 : NEG_INF;
+    }
   };
   auto lstore = [&](int stage) {
     char *kd = lds + stage * 2 * TILEB;
@@ -140,9 +179,10 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       *(u32x4 *)(kd + row * ROWB + col * 16) = kst[i];
       *(u32x4 *)(vd + row * ROWB + col * 16) = vst[i];
     }
+    if (MASK == kMaskPerKey && tid < BK) ldsMask[stage * BK + tid] = mst;
   };
 
-  // ---- per-row mask / drop-mask base pointers
+  // ---- per-row base pointers of [.., sk]-shaped tensors
   const T *mrow[QB];
   const T *drow[QB];
   size_t srow[QB];
@@ -152,20 +192,22 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     if (q > a.sq - 1) q = a.sq - 1;
     mrow[qb] = nullptr;
     drow[qb] = nullptr;
-    if (MASK) mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
+    if (MASK == kMaskFull)
+      mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
     srow[qb] = ((size_t)bh * a.sq + q) * a.sk;
     if (DROP == 2 && a.drop_mask) drow[qb] = (const T *)a.drop_mask + srow[qb];
   }
 
-  // four consecutive elements of a [.., sk] row starting at key kk (kk % 4 == 0), as floats
-  auto load4 = [&](const T *row, int kk, float dflt, float out[4]) {
-    if (a.mask_vec && kk + 3 < a.sk) {
+  // four consecutive elements of a [.., sk] row starting at key kk (kk % 4 == 0), as floats.
+  // SAFE = the whole group is known to be in range and 8-byte aligned.
+  auto load4 = [&](const T *row, int kk, bool safe, float out[4]) {
+    if (safe) {
       v4 t = as_v4<T>(*(const u32x2 *)(row + kk));
 #pragma unroll
       for (int i = 0; i < 4; ++i) out[i] = (float)t[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = (kk + i < a.sk) ? (float)row[kk + i] : dflt;
+      for (int i = 0; i < 4; ++i) out[i] = (kk + i < a.sk) ? (float)row[kk + i] : 0.f;
     }
   };
   auto store4 = [&](T *row, int kk, const float in[4]) {
@@ -183,10 +225,10 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
   // ---- running state
   f32x16 o[QB][DB];
-  float m[QB], lsum[QB];
+  float mref[QB], lsum[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    m[qb] = NEG_INF;
+    mref[qb] = NEG_INF;
     lsum[qb] = 0.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -217,6 +259,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
       const char *ldsK = lds + cur * 2 * TILEB;
       const char *ldsV = ldsK + TILEB;
+      const float *ldsM = ldsMask + cur * BK;
 
       const bool active = !CAUSAL || (k0 <= q0w + QB * 32 - 1);
       if (active) {
@@ -225,9 +268,20 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb) {
 #pragma unroll
-          for (int qb = 0; qb < QB; ++qb)
+          for (int qb = 0; qb < QB; ++qb) {
+            if (MASK == kMaskPerKey) {
+              // row r of the accumulator is key 8*(r/4) + 4h + r%4: seed it with that key's term
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[qb][sb][r] = 0.f;
+              for (int g = 0; g < 4; ++g) {
+                const f32x4 t4 = *(const f32x4 *)(ldsM + sb * 32 + 8 * g + 4 * h);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) s[qb][sb][4 * g + t] = t4[t];
+              }
+            } else {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) s[qb][sb][r] = 0.f;
+            }
+          }
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
             const v8 ka = as_v8<T>(*(const u32x4 *)(ldsK + (sb * 32 + ql) * ROWB + ks * 32 + h * 16));
@@ -236,63 +290,75 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
           }
         }
 
-        const bool pred = (k0 + BK > a.sk) || (CAUSAL && (k0 + BK - 1 > q0w));
+        // Tiles that need a per-element bounds / causal test take the guarded path; the
+        // per-key mask path encodes the ragged tail in its -inf terms and needs none.
+        const bool ragged = (MASK != kMaskPerKey) && (k0 + BK > a.sk);
+        const bool diag = CAUSAL && (k0 + BK - 1 > q0w);
+        const bool vec_ok = a.mask_vec && !ragged;
         v8 pfrag[QB][NSB][2];
 
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
+        auto softmax_block = [&](int qb, auto guarded_tag) {
+          constexpr bool GUARDED = decltype(guarded_tag)::value;
           const int q = q0w + qb * 32 + ql;
-          // scores in log2 units, mask, bounds
+          // ---- raw scores (per-key mask term already inside), bounds, running max.
+          // With a full mask tensor the scaled+masked score x is formed here; otherwise the
+          // scale is folded into the exponent's fma below (scale > 0 keeps the max monotone).
           float mx = NEG_INF;
 #pragma unroll
           for (int sb = 0; sb < NSB; ++sb) {
+            if (MASK == kMaskFull || GUARDED) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const int kk = k0 + sb * 32 + 8 * g + 4 * h;
-              float mv[4] = {0.f, 0.f, 0.f, 0.f};
-              if (MASK) {
-                load4(mrow[qb], kk, 0.f, mv);
+              for (int g = 0; g < 4; ++g) {
+                const int kk = k0 + sb * 32 + 8 * g + 4 * h;
+                float mv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (MASK == kMaskFull) {
+                  load4(mrow[qb], kk, vec_ok, mv);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) mv[t] = fmaf(mv[t], a.mask_a, a.mask_b);
-              }
-#pragma unroll
-              for (int t = 0; t < 4; ++t) {
-                float x = fmaf(s[qb][sb][4 * g + t], a.scale_l2, mv[t]);
-                if (pred) {
-                  const int k = kk + t;
-                  const bool ok = (k < a.sk) && (!CAUSAL || k <= q);
-                  x = ok ? x : NEG_INF;
+                  for (int t = 0; t < 4; ++t) mv[t] = fmaf(mv[t], a.mask_a, a.mask_b);
                 }
-                s[qb][sb][4 * g + t] = x;
-                mx = fmaxf(mx, x);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                  float x = s[qb][sb][4 * g + t];
+                  if (MASK == kMaskFull) x = fmaf(x, a.scale_l2, mv[t]);
+                  if (GUARDED) {
+                    const int k = kk + t;
+                    const bool ok = (k < a.sk) && (!CAUSAL || k <= q);
+                    x = ok ? x : NEG_INF;
+                  }
+                  s[qb][sb][4 * g + t] = x;
+                }
               }
             }
+            mx = max3(mx, s[qb][sb][0], s[qb][sb][1]);
+#pragma unroll
+            for (int r = 2; r < 16; r += 2) mx = max3(mx, s[qb][sb][r], s[qb][sb][r + 1]);
           }
-          float msafe;
+          constexpr bool PRESCALED = (MASK == kMaskFull);
+          const float cs = PRESCALED ? 1.f : a.scale_l2;
+
           if (pass == 0) {
-            mx = xhalf_max(mx);
-            const float mnew = fmaxf(m[qb], mx);
-            msafe = (mnew == NEG_INF) ? 0.f : mnew;
-            const float alpha = fast_exp2(m[qb] - msafe);
-            m[qb] = mnew;
-            lsum[qb] *= alpha;
+            mx = xhalf_max(mx) * cs;
+            // raise the reference exponent only when this tile would overflow the 2^8 headroom
+            // (with mref = -inf the test reads mx > -inf: the first finite maximum always raises it)
+            if (__builtin_amdgcn_ballot_w64(mx > mref[qb] + RESCALE_TH) != 0ull) {
+              const float mnew = fmaxf(mref[qb], mx);
+              const float ms = (mnew == NEG_INF) ? 0.f : mnew;
+              const float alpha = fast_exp2(mref[qb] - ms);
+              mref[qb] = mnew;
+              lsum[qb] *= alpha;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+              for (int db = 0; db < DB; ++db)
 #pragma unroll
-              for (int r = 0; r < 16; ++r) o[qb][db][r] *= alpha;
-          } else {
-            msafe = (m[qb] == NEG_INF) ? 0.f : m[qb];
+                for (int r = 0; r < 16; ++r) o[qb][db][r] *= alpha;
+            }
           }
-          float rs = 0.f;
+          const float nmsafe = (mref[qb] == NEG_INF) ? 0.f : -mref[qb];
+
 #pragma unroll
           for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const float p = fast_exp2(s[qb][sb][r] - msafe);
-              s[qb][sb][r] = p;
-              rs += p;
-            }
-          if (pass == 0) lsum[qb] += rs;
+            for (int r = 0; r < 16; ++r)
+              s[qb][sb][r] = fast_exp2(PRESCALED ? s[qb][sb][r] + nmsafe : fmaf(s[qb][sb][r], cs, nmsafe));
 
           if (pass == 1) {
             // save-intermediates pass: normalised softmax and its dropped/scaled version
@@ -310,17 +376,31 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
                   for (int t = 0; t < 4; ++t) pv[t] = s[qb][sb][4 * g + t] * inv_l[qb];
                   if (ssm) store4(ssm, kk, pv);
                   if (sdr) {
-                    if (drow[qb]) load4(drow[qb], kk, 0.f, dm);
+                    if (drow[qb]) load4(drow[qb], kk, vec_ok, dm);
 #pragma unroll
                     for (int t = 0; t < 4; ++t) pv[t] = pv[t] * (dm[t] * a.drop_scale);
                     store4(sdr, kk, pv);
                   }
                 }
             }
-            continue;
+            return;
           }
 
-          // ---- dropout on the (unnormalised) probabilities
+          // ---- round to the element type, sum the rounded values (softmax denominator)
+          float rs = 0.f;
+          v8 pk[NSB][2];
+#pragma unroll
+          for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) pk[sb][c][j] = (T)s[qb][sb][8 * c + j];
+#pragma unroll
+              for (int j = 0; j < 4; ++j) rs = dot2_ones<T>(pk[sb][c], j, rs);
+            }
+          lsum[qb] += rs;
+
+          // ---- dropout acts on the numerator only
           if (DROP == 1) {
 #pragma unroll
             for (int sb = 0; sb < NSB; ++sb)
@@ -330,7 +410,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
                 const uint32_t wd = drop_word(a.drop, (uint32_t)bh, (uint32_t)q, (uint32_t)(kk >> 2));
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                  if (!drop_keep_byte(wd, t, a.drop.thr)) s[qb][sb][4 * g + t] = 0.f;
+                  if (!drop_keep_byte(wd, t, a.drop.thr)) pk[sb][g >> 1][4 * (g & 1) + t] = (T)0.f;
               }
           } else if (DROP == 2) {
             if (drow[qb]) {
@@ -340,19 +420,25 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
                 for (int g = 0; g < 4; ++g) {
                   const int kk = k0 + sb * 32 + 8 * g + 4 * h;
                   float dm[4];
-                  load4(drow[qb], kk, 0.f, dm);
+                  load4(drow[qb], kk, vec_ok, dm);
 #pragma unroll
-                  for (int t = 0; t < 4; ++t) s[qb][sb][4 * g + t] *= dm[t];
+                  for (int t = 0; t < 4; ++t)
+                    pk[sb][g >> 1][4 * (g & 1) + t] = (T)((float)pk[sb][g >> 1][4 * (g & 1) + t] * dm[t]);
                 }
             }
           }
-          // ---- round to the element type: B operand of the second product
 #pragma unroll
           for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-            for (int c = 0; c < 2; ++c)
+            for (int c = 0; c < 2; ++c) pfrag[qb][sb][c] = pk[sb][c];
+        };
+
+        if (ragged || diag) {
 #pragma unroll
-              for (int j = 0; j < 8; ++j) pfrag[qb][sb][c][j] = (T)s[qb][sb][8 * c + j];
+          for (int qb = 0; qb < QB; ++qb) softmax_block(qb, std::true_type{});
+        } else {
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) softmax_block(qb, std::false_type{});
         }
 
         if (pass == 0) {
@@ -363,21 +449,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
             for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
               for (int c = 0; c < 2; ++c) {
-                v8 va;
-                const int key0 = sb * 32 + 4 * h + 16 * c;
-                if (a.flags & 1) {
-#pragma unroll
-                  for (int j = 0; j < 8; ++j)
-                    va[j] = *(const T *)(ldsV + (key0 + 8 * (j >> 2) + (j & 3)) * ROWB + (db * 32 + ql) * 2);
-                } else {
-                  const int i16 = l & 15;
-                  const int d0 = db * 32 + (ql & 16);
-                  const char *p0 = ldsV + (key0 + (i16 >> 2)) * ROWB + (d0 + 4 * (i16 & 3)) * 2;
-                  const u32x2 lo = lds_read_tr16(p0);
-                  const u32x2 hi = lds_read_tr16(p0 + 8 * ROWB);
-                  u32x4 both = {lo.x, lo.y, hi.x, hi.y};
-                  va = as_v8<T>(both);
-                }
+                const v8 va = lds_load_a_transposed<T, ROWB>(ldsV, sb * 32, db * 32, c, l);
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) o[qb][db] = E::mfma(va, pfrag[qb][sb][c], o[qb][db]);
               }
@@ -407,7 +479,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
           *(v4 *)(Ob + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
         }
       if (a.lse && h == 0)
-        a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (m[qb] + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
+        a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
     }
   }
 }

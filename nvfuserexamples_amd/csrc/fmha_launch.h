@@ -11,7 +11,7 @@ namespace fmha {
 
 struct FwdVariant {
   int qb;       // 32-query blocks per wave (1 or 2)
-  bool mask;    // a mask tensor is read
+  int mask;     // kMaskNone / kMaskPerKey (constant along queries) / kMaskFull
   bool causal;
   int drop;     // 0 none, 1 Philox, 2 tensor / save-intermediates
 };

@@ -16,6 +16,10 @@ from conftest import make_qkv, pad_mask, f32
 pytestmark = pytest.mark.gpu
 
 TOL = {"fp16": 2e-3, "bf16": 2e-2}
+# The kernel's softmax denominator sums the probabilities AFTER rounding to the element type (so the
+# weights of the second product sum to one exactly); the saved LSE carries that rounding: up to
+# 2^-11 relative (fp16) / 2^-9 (bf16) on rows with a handful of visible keys.
+LSE_TOL = {"fp16": 1e-3, "bf16": 5e-3}
 TDT = {"fp16": torch.float16, "bf16": torch.bfloat16}
 
 
@@ -65,7 +69,7 @@ def test_forward_matches_oracle(bh, sq, sk, d, dtype, mask, causal, qb, monkeypa
                            mask_kind="keep01" if mk == capi.MASK_KEEP01 else "additive", causal=causal,
                            want=("o", "lse"))
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= TOL[dtype]
-    assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= 1e-3
+    assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= LSE_TOL[dtype]
 
 
 @pytest.mark.parametrize("bh,sq,sk,d,causal", [(3, 128, 192, 64, False), (2, 257, 257, 64, True),
