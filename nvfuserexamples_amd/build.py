@@ -9,6 +9,7 @@ Everything is compiled for gfx950 only.  Run as ``python -m nvfuserexamples_amd.
 """
 import concurrent.futures as cf
 import os
+import re
 import subprocess
 import sys
 import sysconfig
@@ -19,6 +20,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 OBJDIR = os.path.join(ROOT, "build", "obj")
 HIP_LIB = os.path.join(LIBDIR, "libfmha_hip.so")
+EXTRA = os.environ.get("FMHA_EXTRA_HIPFLAGS", "").split()  # experiments only
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
@@ -59,10 +61,13 @@ def build_hip(jobs=None, verbose=True):
     os.makedirs(OBJDIR, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     cmds, objs = [], []
+    only = os.environ.get("FMHA_BUILD_ONLY")  # development aid: regex of objects to recompile
     for src, obj, defs in _tus():
         o = os.path.join(OBJDIR, obj)
         objs.append(o)
-        cmds.append([HIPCC, *HIP_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", o])
+        if only and os.path.exists(o) and not re.search(only, obj):
+            continue
+        cmds.append([HIPCC, *HIP_FLAGS, *EXTRA, *defs, "-c", os.path.join(CSRC, src), "-o", o])
     with cf.ThreadPoolExecutor(jobs) as ex:
         for out in ex.map(_run, cmds):
             if verbose and out.strip():

@@ -1,6 +1,7 @@
 // Instantiates the forward kernel for one (element type, head dim) pair, chosen with
 // -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128}, and exports its dispatcher.
 #include "fmha_launch.h"
+#include "fmha_fwd_pipe.h"
 
 #if FMHA_TU_BF16
 #define FMHA_TU_T __bf16
@@ -19,7 +20,11 @@ constexpr int kNW = 4;
 
 template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
   using Cfg = FwdCfg<FMHA_TU_D>;
-  auto kern = fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+  // tensor dropout and the save pass run on the plain loop; everything else is software-pipelined
+  auto kern = [] {
+    if constexpr (DROP == 2) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+    else return fmha_fwd_pipe_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+  }();
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
   if (attr != hipSuccess) return 2;
@@ -41,15 +46,28 @@ template <int QB, int MASK> int by_causal(FwdArgs &a, const FwdVariant &v, hipSt
   return v.causal ? by_drop<QB, MASK, true>(a, v.drop, s) : by_drop<QB, MASK, false>(a, v.drop, s);
 }
 
+#ifdef FMHA_DEV_MINIMAL
+// development builds: only the variants the headline benchmark uses
+template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
+  if (QB != 1 || v.causal || v.drop) return 1;
+  if (v.mask == kMaskPerKey) return launch<1, kMaskPerKey, false, 0>(a, s);
+  if (v.mask == kMaskNone) return launch<1, kMaskNone, false, 0>(a, s);
+  return 1;
+}
+#else
 template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
   if (v.mask == kMaskPerKey) return by_causal<QB, kMaskPerKey>(a, v, s);
   if (v.mask == kMaskFull) return by_causal<QB, kMaskFull>(a, v, s);
   return by_causal<QB, kMaskNone>(a, v, s);
 }
+#endif
 
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
+#ifdef FMHA_DEV_MINIMAL
+  if (v.drop == 2) return 1;
+#endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;
     if (v.mask == kMaskPerKey) return launch<1, kMaskPerKey, false, 2>(a, s);

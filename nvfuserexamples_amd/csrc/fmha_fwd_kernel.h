@@ -4,28 +4,39 @@
 // (fmha/fmha_manual.cpp:20-409, :411-807, :809-1214).  Where the reference keeps a
 // whole key row of 128 in one CTA (fmha_manual.cpp:107-111) and moves the score
 // tile through shared memory twice (:160,165,274,322), this kernel walks the keys
-// in LDS tiles of 64 with an online (running max / running sum) softmax and keeps
-// scores and probabilities in registers from the first product to the second.
+// in LDS tiles of 64 with an online softmax and keeps scores and probabilities in
+// registers from the first product to the second.
 //
 // Work decomposition
 //   workgroup = NW waves, one (bh, query tile of NW*QB*32 rows); wave = QB blocks of
 //   32 queries.  K and V tiles of 64 keys are staged in LDS (double buffered, padded
 //   rows); Q lives in registers as the B operand for the whole kernel.
 // Products are computed transposed so that every lane owns one query column:
-//   S^T[key][q] = K . Q^T       A = K rows from LDS (ds_read_b128), B = Q registers
+//   X^T[key][q] = K . Q'^T      A = K rows from LDS (ds_read_b128), B = Q' registers
 //   O^T[d][q]   = V^T . P^T     A = V^T via the LDS transpose read, B = P registers
-// The accumulator layout of S^T (lane = query, registers = keys) is exactly the B
+// The accumulator layout of X^T (lane = query, registers = keys) is exactly the B
 // operand layout of the second product under a fixed permutation of the key index,
 // and V is fetched with that same permutation, so P never leaves registers.
 //
-// Softmax bookkeeping per lane (one query): a reference exponent m, a partial sum l
-// of the ROUNDED probabilities (accumulated with v_dot2 on the packed pairs, so the
-// denominator matches what the second product actually sums) and the unnormalised
-// accumulator O^T.  The reference m is raised -- and l, O rescaled -- only when a
-// tile's maximum exceeds it by more than 2^8, which keeps every probability below
-// 256 (exact in fp16/bf16 range) and removes the rescale from almost every tile.
-// Row max needs one exchange between lane l and l^32 per tile; the two half-wave
-// partial sums are combined once in the epilogue.
+// The softmax is VALU-bound at head dim 64 (one v_exp per score against ~16 MFMA
+// flops per score), so everything except the exponential and the rounding is pushed
+// into the matrix pipe:
+//   * Q' = Q * scale * log2(e), rounded once to the element type, so the product is
+//     already in log2 units;
+//   * the product gets one extra contraction step whose A rows are
+//     (1, mask_hi[key], mask_lo[key], 1, 0, ...) and whose B columns are
+//     (-m[q], 1, 1, c, 0, ...): the accumulator comes out as
+//         x = score + mask[key] - m[q]
+//     i.e. the per-key additive mask (split hi+lo so it keeps 2x the element type's
+//     precision; -inf for keys past the end) and the per-query reference exponent m are
+//     applied by the MFMA, and P = exp2(x) needs no further arithmetic;
+//   * m is kept representable in the element type so the subtraction is exact, and it
+//     is NOT the running maximum: it is only raised when a tile's probabilities would
+//     leave a 2^14 window (detected from the tile's row sum, which is needed anyway),
+//     so the common tile computes no maximum and rescales nothing;
+//   * the row sum is taken over the ROUNDED probabilities with v_dot2 on the packed
+//     pairs, so the denominator matches what the second product sums.
+// The two half-wave partial sums are combined once in the epilogue.
 #pragma once
 #include <type_traits>
 
@@ -63,7 +74,8 @@ template <int D> struct FwdCfg {
   static constexpr int DB = D / 32;       // 32-row blocks of O^T
   static constexpr int ROWB = D * 2 + 16; // LDS row pitch in bytes (16 B pad: conflict-free b128 reads)
   static constexpr int TILEB = BK * ROWB;
-  static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * 4; // {K,V} x 2 stages + per-key mask terms x 2 stages
+  static constexpr int XROWB = 32;        // pitch of the extra-contraction-step rows (16 elements)
+  static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * XROWB; // {K,V} x 2 stages + extra rows x 2 stages
 };
 
 template <typename T> FMHA_DEV float dot2_ones(typename Elem<T>::v8 v, int pair, float acc);
@@ -86,19 +98,19 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = FwdCfg<D>;
-  constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB;
+  constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, XROWB = C::XROWB;
   constexpr int TILEB = C::TILEB;
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
   constexpr int CPR = D / 8;                 // 16-byte chunks per row
   constexpr int CPT = BK * CPR / NT;         // chunks per thread per tile
   static_assert(BK * CPR % NT == 0, "tile must divide evenly over the workgroup");
-  static_assert(NT >= BK, "per-key mask terms are staged by the first BK threads");
+  static_assert(NT >= BK, "the extra rows are staged by the first BK threads");
   constexpr float NEG_INF = -__builtin_inff();
-  constexpr float RESCALE_TH = 8.f; // log2 units
+  constexpr float WINDOW = 16384.f; // a tile whose rounded row sum reaches 2^14 raises the reference
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  float *ldsMask = (float *)(lds + 4 * TILEB);
+  char *ldsX = lds + 4 * TILEB;
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -122,7 +134,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
   const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
-  // ---- Q operand registers
+  // ---- Q' = Q * scale * log2(e) as B-operand registers
   v8 qreg[QB][KS];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
@@ -131,7 +143,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 t = {0u, 0u, 0u, 0u};
       if (q < a.sq) t = *(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8);
-      qreg[qb][ks] = as_v8<T>(t);
+      const v8 raw = as_v8<T>(t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
     }
   }
 
@@ -146,7 +160,8 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
   // ---- tile staging: global -> registers -> LDS
   u32x4 kst[CPT], vst[CPT];
-  float mst = 0.f;
+  T mraw = (T)0.f;     // raw per-key mask element in flight (converted when it is written to LDS,
+  bool mvalid = false; // so that the conversion does not wait on the loads issued with it)
   auto gload = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
@@ -161,12 +176,10 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       kst[i] = kk;
       vst[i] = vv;
     }
-    if (MASK == kMaskPerKey && tid < BK) {
-      // additive term of key k0+tid, divided by the score scale so that it can seed the
-      // accumulator of K.Q^T (the product then comes out as score + term/scale and one fma
-      // finishes it); keys past the end get -inf, which also covers the ragged last tile
+    if (tid < BK) {
       const int kr = k0 + tid;
-      mst = kr < a.sk ? fmaf((float)mkey[kr], a.mask_a, a.mask_b) * a.inv_scale_l2 : NEG_INF;
+      mvalid = kr < a.sk;
+      if (MASK == kMaskPerKey && mvalid) mraw = mkey[kr];
     }
   };
   auto lstore = [&](int stage) {
@@ -179,7 +192,28 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       *(u32x4 *)(kd + row * ROWB + col * 16) = kst[i];
       *(u32x4 *)(vd + row * ROWB + col * 16) = vst[i];
     }
-    if (MASK == kMaskPerKey && tid < BK) ldsMask[stage * BK + tid] = mst;
+    if (tid < BK) {
+      // extra contraction step, A side: (1, mask_hi, mask_lo, 1, 0 ...); keys past the end get
+      // mask = -inf, which is all the ragged last tile needs
+      float mk = 0.f;
+      if (MASK == kMaskPerKey) mk = fmaf((float)mraw, a.mask_a, a.mask_b);
+      if (!mvalid) mk = NEG_INF;
+      const T hi = (T)mk;
+      const T lo = mvalid ? (T)(mk - (float)hi) : (T)0.f;
+      v8 x0, x1;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        x0[j] = (T)0.f;
+        x1[j] = (T)0.f;
+      }
+      x0[0] = (T)1.f;
+      x0[1] = hi;
+      x0[2] = (hi == hi && (float)hi != NEG_INF) ? lo : (T)0.f;
+      x0[3] = (T)1.f;
+      v8 *dst = (v8 *)(ldsX + stage * BK * XROWB + tid * XROWB);
+      dst[0] = x0;
+      dst[1] = x1;
+    }
   };
 
   // ---- per-row base pointers of [.., sk]-shaped tensors
@@ -199,7 +233,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   }
 
   // four consecutive elements of a [.., sk] row starting at key kk (kk % 4 == 0), as floats.
-  // SAFE = the whole group is known to be in range and 8-byte aligned.
+  // safe = the whole group is known to be in range and 8-byte aligned.
   auto load4 = [&](const T *row, int kk, bool safe, float out[4]) {
     if (safe) {
       v4 t = as_v4<T>(*(const u32x2 *)(row + kk));
@@ -223,17 +257,28 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     }
   };
 
-  // ---- running state
+  // ---- running state.  mref: reference exponent (log2 units, representable in T); seen: a
+  // finite score has set it; lsum: this lane's part of the denominator; o: unnormalised O^T.
   f32x16 o[QB][DB];
   float mref[QB], lsum[QB];
+  bool seen[QB];
+  v8 bx[QB]; // extra contraction step, B side: (-mref, 1, 1, c, 0 ...) on the lower half-wave
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    mref[qb] = NEG_INF;
+    mref[qb] = 0.f;
+    seen[qb] = false;
     lsum[qb] = 0.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[qb][db][r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bx[qb][j] = (T)0.f;
+    if (h == 0) {
+      bx[qb][1] = (T)1.f;
+      bx[qb][2] = (T)1.f;
+      if (MASK == kMaskFull) bx[qb][3] = (T)a.mask_b; // constant part of a full mask's term
+    }
   }
   float inv_l[QB]; // used by the save pass
 
@@ -259,106 +304,76 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
       const char *ldsK = lds + cur * 2 * TILEB;
       const char *ldsV = ldsK + TILEB;
-      const float *ldsM = ldsMask + cur * BK;
+      const char *ldsXc = ldsX + cur * BK * XROWB;
 
       const bool active = !CAUSAL || (k0 <= q0w + QB * 32 - 1);
       if (active) {
-        // ---- S^T = K . Q^T
-        f32x16 s[QB][NSB];
+        // ---- x^T = K . Q'^T  + (mask[key] - mref[q]) through the extra step
+        f32x16 x[QB][NSB];
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb) {
 #pragma unroll
-          for (int qb = 0; qb < QB; ++qb) {
-            if (MASK == kMaskPerKey) {
-              // row r of the accumulator is key 8*(r/4) + 4h + r%4: seed it with that key's term
+          for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-              for (int g = 0; g < 4; ++g) {
-                const f32x4 t4 = *(const f32x4 *)(ldsM + sb * 32 + 8 * g + 4 * h);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) s[qb][sb][4 * g + t] = t4[t];
-              }
-            } else {
-#pragma unroll
-              for (int r = 0; r < 16; ++r) s[qb][sb][r] = 0.f;
-            }
-          }
+            for (int r = 0; r < 16; ++r) x[qb][sb][r] = 0.f;
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
             const v8 ka = as_v8<T>(*(const u32x4 *)(ldsK + (sb * 32 + ql) * ROWB + ks * 32 + h * 16));
 #pragma unroll
-            for (int qb = 0; qb < QB; ++qb) s[qb][sb] = E::mfma(ka, qreg[qb][ks], s[qb][sb]);
+            for (int qb = 0; qb < QB; ++qb) x[qb][sb] = E::mfma(ka, qreg[qb][ks], x[qb][sb]);
           }
+          const v8 xa = as_v8<T>(*(const u32x4 *)(ldsXc + (sb * 32 + ql) * XROWB + h * 16));
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) x[qb][sb] = E::mfma(xa, bx[qb], x[qb][sb]);
         }
 
-        // Tiles that need a per-element bounds / causal test take the guarded path; the
-        // per-key mask path encodes the ragged tail in its -inf terms and needs none.
-        const bool ragged = (MASK != kMaskPerKey) && (k0 + BK > a.sk);
+        // Only tiles crossing the causal diagonal need a per-element test (the ragged tail is
+        // handled by the -inf mask terms of the extra step).
         const bool diag = CAUSAL && (k0 + BK - 1 > q0w);
-        const bool vec_ok = a.mask_vec && !ragged;
+        const bool vec_ok = a.mask_vec && (k0 + BK <= a.sk);
         v8 pfrag[QB][NSB][2];
 
         auto softmax_block = [&](int qb, auto guarded_tag) {
           constexpr bool GUARDED = decltype(guarded_tag)::value;
           const int q = q0w + qb * 32 + ql;
-          // ---- raw scores (per-key mask term already inside), bounds, running max.
-          // With a full mask tensor the scaled+masked score x is formed here; otherwise the
-          // scale is folded into the exponent's fma below (scale > 0 keeps the max monotone).
-          float mx = NEG_INF;
+          if (MASK == kMaskFull || GUARDED) {
 #pragma unroll
-          for (int sb = 0; sb < NSB; ++sb) {
-            if (MASK == kMaskFull || GUARDED) {
+            for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
               for (int g = 0; g < 4; ++g) {
                 const int kk = k0 + sb * 32 + 8 * g + 4 * h;
                 float mv[4] = {0.f, 0.f, 0.f, 0.f};
-                if (MASK == kMaskFull) {
-                  load4(mrow[qb], kk, vec_ok, mv);
-#pragma unroll
-                  for (int t = 0; t < 4; ++t) mv[t] = fmaf(mv[t], a.mask_a, a.mask_b);
-                }
+                if (MASK == kMaskFull) load4(mrow[qb], kk, vec_ok, mv);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                  float x = s[qb][sb][4 * g + t];
-                  if (MASK == kMaskFull) x = fmaf(x, a.scale_l2, mv[t]);
-                  if (GUARDED) {
-                    const int k = kk + t;
-                    const bool ok = (k < a.sk) && (!CAUSAL || k <= q);
-                    x = ok ? x : NEG_INF;
-                  }
-                  s[qb][sb][4 * g + t] = x;
+                  float xv = x[qb][sb][4 * g + t];
+                  if (MASK == kMaskFull) xv = fmaf(mv[t], a.mask_a, xv);
+                  if (GUARDED) xv = (kk + t <= q) ? xv : NEG_INF;
+                  x[qb][sb][4 * g + t] = xv;
                 }
               }
-            }
-            mx = max3(mx, s[qb][sb][0], s[qb][sb][1]);
-#pragma unroll
-            for (int r = 2; r < 16; r += 2) mx = max3(mx, s[qb][sb][r], s[qb][sb][r + 1]);
           }
-          constexpr bool PRESCALED = (MASK == kMaskFull);
-          const float cs = PRESCALED ? 1.f : a.scale_l2;
 
-          if (pass == 0) {
-            mx = xhalf_max(mx) * cs;
-            // raise the reference exponent only when this tile would overflow the 2^8 headroom
-            // (with mref = -inf the test reads mx > -inf: the first finite maximum always raises it)
-            if (__builtin_amdgcn_ballot_w64(mx > mref[qb] + RESCALE_TH) != 0ull) {
-              const float mnew = fmaxf(mref[qb], mx);
-              const float ms = (mnew == NEG_INF) ? 0.f : mnew;
-              const float alpha = fast_exp2(mref[qb] - ms);
-              mref[qb] = mnew;
-              lsum[qb] *= alpha;
+          // ---- P = exp2(x), rounded to the element type; row sum of the rounded values
+          float p[NSB][16];
+          v8 pk[NSB][2];
+          float rs = 0.f;
+          auto exp_pack = [&](float shift) {
+            rs = 0.f;
 #pragma unroll
-              for (int db = 0; db < DB; ++db)
+            for (int sb = 0; sb < NSB; ++sb) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o[qb][db][r] *= alpha;
+              for (int r = 0; r < 16; ++r) p[sb][r] = fast_exp2(x[qb][sb][r] + shift);
+#pragma unroll
+              for (int c = 0; c < 2; ++c) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) pk[sb][c][j] = (T)p[sb][8 * c + j];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) rs = dot2_ones<T>(pk[sb][c], j, rs);
+              }
             }
-          }
-          const float nmsafe = (mref[qb] == NEG_INF) ? 0.f : -mref[qb];
-
-#pragma unroll
-          for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-              s[qb][sb][r] = fast_exp2(PRESCALED ? s[qb][sb][r] + nmsafe : fmaf(s[qb][sb][r], cs, nmsafe));
+          };
+          exp_pack(0.f);
 
           if (pass == 1) {
             // save-intermediates pass: normalised softmax and its dropped/scaled version
@@ -373,7 +388,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
                   if (kk >= a.sk) continue;
                   float pv[4], dm[4] = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
-                  for (int t = 0; t < 4; ++t) pv[t] = s[qb][sb][4 * g + t] * inv_l[qb];
+                  for (int t = 0; t < 4; ++t) pv[t] = p[sb][4 * g + t] * inv_l[qb];
                   if (ssm) store4(ssm, kk, pv);
                   if (sdr) {
                     if (drow[qb]) load4(drow[qb], kk, vec_ok, dm);
@@ -386,18 +401,36 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
             return;
           }
 
-          // ---- round to the element type, sum the rounded values (softmax denominator)
-          float rs = 0.f;
-          v8 pk[NSB][2];
+          // ---- rare path: the reference exponent is unset or this tile left the window.
+          // Take the tile maximum, move the reference there (kept representable in T),
+          // rescale the running sums and redo the exponentials.
+          const bool unfit = !(rs < WINDOW) || !seen[qb];
+          if (__builtin_amdgcn_ballot_w64(unfit) != 0ull) {
+            float mx = NEG_INF;
 #pragma unroll
-          for (int sb = 0; sb < NSB; ++sb)
+            for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-#pragma unroll
-              for (int j = 0; j < 8; ++j) pk[sb][c][j] = (T)s[qb][sb][8 * c + j];
-#pragma unroll
-              for (int j = 0; j < 4; ++j) rs = dot2_ones<T>(pk[sb][c], j, rs);
+              for (int r = 0; r < 16; r += 2) mx = max3(mx, x[qb][sb][r], x[qb][sb][r + 1]);
+            mx = xhalf_max(mx);
+            float mnew = mref[qb];
+            if (mx != NEG_INF) {
+              const float cand = (float)(T)(mref[qb] + mx);
+              mnew = seen[qb] ? fmaxf(mref[qb], cand) : cand;
+              seen[qb] = true;
             }
+            const float shift = mref[qb] - mnew;
+            if (shift != 0.f) {
+              const float alpha = fast_exp2(shift);
+              lsum[qb] *= alpha;
+#pragma unroll
+              for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[qb][db][r] *= alpha;
+            }
+            mref[qb] = mnew;
+            if (h == 0) bx[qb][0] = (T)(-mnew);
+            exp_pack(shift);
+          }
           lsum[qb] += rs;
 
           // ---- dropout acts on the numerator only
@@ -433,7 +466,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
             for (int c = 0; c < 2; ++c) pfrag[qb][sb][c] = pk[sb][c];
         };
 
-        if (ragged || diag) {
+        if (diag) {
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) softmax_block(qb, std::true_type{});
         } else {
@@ -478,8 +511,11 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
           for (int i = 0; i < 4; ++i) t[i] = (T)(o[qb][db][4 * g + i] * inv);
           *(v4 *)(Ob + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
         }
+      // the constant part of a full mask's term entered the product rounded to T; the
+      // difference cancels in O but belongs in the log-sum-exp
+      const float cfix = (MASK == kMaskFull) ? a.mask_b - (float)(T)a.mask_b : 0.f;
       if (a.lse && h == 0)
-        a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
+        a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + cfix + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
     }
   }
 }
