@@ -24,7 +24,7 @@ template <typename K> int set_lds(K kern, int bytes) {
                              bytes) == hipSuccess ? 0 : 2;
 }
 
-template <bool MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s) {
+template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s) {
   using Cfg = BwdCfg<FMHA_TU_D>;
   auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP>;
   auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP>;
@@ -44,7 +44,7 @@ template <bool MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
-template <bool MASK, bool CAUSAL> int by_drop(BwdArgs &a, int drop, hipStream_t s) {
+template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<MASK, CAUSAL, 0>(a, s);
   if (drop == 1) return launch<MASK, CAUSAL, 1>(a, s);
   return 1;
@@ -53,8 +53,11 @@ template <bool MASK, bool CAUSAL> int by_drop(BwdArgs &a, int drop, hipStream_t 
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
-  if (v.mask) return v.causal ? by_drop<true, true>(a, v.drop, s) : by_drop<true, false>(a, v.drop, s);
-  return v.causal ? by_drop<false, true>(a, v.drop, s) : by_drop<false, false>(a, v.drop, s);
+  if (v.mask == kMaskPerKey)
+    return v.causal ? by_drop<kMaskPerKey, true>(a, v.drop, s) : by_drop<kMaskPerKey, false>(a, v.drop, s);
+  if (v.mask == kMaskFull)
+    return v.causal ? by_drop<kMaskFull, true>(a, v.drop, s) : by_drop<kMaskFull, false>(a, v.drop, s);
+  return v.causal ? by_drop<kMaskNone, true>(a, v.drop, s) : by_drop<kMaskNone, false>(a, v.drop, s);
 }
 
 } // namespace fmha

@@ -7,17 +7,26 @@
 //
 // Two kernels, no atomics, deterministic:
 //   fmha_bwd_dq_kernel    one workgroup per (bh, query tile), walks the key tiles;
-//                         lane = query, like the forward: S^T = K.Q^T, dP^T = V.dO^T,
+//                         lane = query, like the forward: x^T = K.Q'^T, g^T = V.dO^T,
 //                         dQ^T += K^T.dS^T (K^T through the LDS transpose read).  Also
 //                         computes delta for its rows and writes it out.
 //   fmha_bwd_dkdv_kernel  one workgroup per (bh, key tile), walks the query tiles with
 //                         dK^T / dV^T accumulators resident in registers; lane = key:
-//                         S = Q.K^T, dP = dO.V^T, dV^T += dO^T.(P o Z), dK^T += Q^T.dS
+//                         x = Q.K'^T, g = dO.V^T, dV^T += dO^T.(P o Z), dK^T += Q^T.dS
 //                         (dO^T and Q^T through the LDS transpose read).
 // In both, the 32x32 accumulator tile of the score product is converted in registers
 // into the B operand of the next product (see fmha_common.h), so P and dS never travel
 // through LDS.  The price of avoiding atomics and LDS transposes of dS is that the score
 // and dP products are formed in both kernels (7 tile products instead of 5).
+//
+// As in the forward, the per-element VALU work is what bounds these kernels at head dim
+// 64, so everything that is a rank-one term rides in one extra contraction step:
+//   x = score*scale*log2e + mask[key] - LSE[q]*log2e     (K' or Q' pre-scaled; mask and LSE
+//                                                         split hi+lo in the element type)
+//   g = dO.V^T - delta[q] / drop_scale
+// leaving  P = exp2(x)  and  dS = P * (kept ? drop_scale*g : -delta)  (= P*g without dropout).
+// "Minus infinity" terms are entered as a large finite negative number, because the same
+// extra rows also meet zeros in the other operand of the second product.
 #pragma once
 #include "fmha_common.h"
 #include "fmha_fwd_kernel.h"
@@ -36,7 +45,7 @@ struct BwdArgs {
   float mask_a, mask_b;
   int32_t bh, sq, sk;
   int32_t ntile; // tiles per head of the kernel being launched
-  float scale_l2, scale, drop_scale;
+  float scale_l2, scale, drop_scale, inv_drop_scale;
   DropCtx drop;
   int32_t flags;
 };
@@ -48,25 +57,38 @@ template <int D> struct BwdCfg {
   static constexpr int DB = D / 32;
   static constexpr int ROWB = D * 2 + 16;
   static constexpr int TILEB = BT * ROWB;
-  static constexpr int LDS_BYTES = 4 * TILEB + 2 * 2 * BT * 4; // two tiles x 2 stages + {lse, delta} x 2 stages
+  static constexpr int XROWB = 32;        // extra-step rows: 16 elements
+  // two tiles x 2 stages + two sets of extra rows x 2 stages + {delta} x 2 stages
+  static constexpr int LDS_BYTES = 4 * TILEB + 2 * 2 * BT * XROWB + 2 * BT * 4;
 };
 
+// A value as hi + lo in the element type (|error| ~ 2^-2p relative), clamped to a large finite
+// negative number so that it may be multiplied by zero.
+template <typename T> FMHA_DEV void split_hi_lo(float v, T &hi, T &lo) {
+  constexpr float BIG = sizeof(T) == 2 && std::is_same<T, _Float16>::value ? -60000.f : -1.0e30f;
+  v = v > BIG ? v : BIG;
+  hi = (T)v;
+  lo = (T)(v - (float)hi);
+}
+
 // ------------------------------------------------------------------------------ dQ
-template <typename T, int D, int QB, int NW, bool MASK, bool CAUSAL, int DROP>
+template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
 __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = BwdCfg<D>;
   constexpr int BK = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, TILEB = C::TILEB;
+  constexpr int XROWB = C::XROWB;
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
   constexpr int CPR = D / 8;
   constexpr int CPT = BK * CPR / NT;
   constexpr float NEG_INF = -__builtin_inff();
-  constexpr float POS_INF = __builtin_inff();
+  constexpr float BIGNEG = -60000.f;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  char *ldsXb = lds + 4 * TILEB; // extra rows per key: (1, 1, mask_hi, mask_lo, 1, 1, 0 ...)
 
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, ql = l & 31, h = l >> 5;
@@ -84,10 +106,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
   const T *dOb = (const T *)a.dout + (size_t)bh * a.sq * D;
   const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
   const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+  const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
-  // ---- per-row operands: Q and dO as B operands, delta, LSE
+  // ---- per-row operands: Q' and dO as B operands, the extra-step columns, delta
   v8 qreg[QB][KS], doreg[QB][KS];
-  float delta[QB], lse2[QB];
+  v8 bxs[QB], bxd[QB]; // (-L_hi, -L_lo, 1, 1, c_hi, c_lo, 0, 0) and (-d_hi, -d_lo, 0 ...) on the lower half-wave
+  float delta[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int q = q0w + qb * 32 + ql;
@@ -101,21 +125,44 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
         td = *(const u32x4 *)(dOb + off);
         to = *(const u32x4 *)(Ob + off);
       }
-      qreg[qb][ks] = as_v8<T>(tq);
+      const v8 qraw = as_v8<T>(tq);
       doreg[qb][ks] = as_v8<T>(td);
       const v8 ov = as_v8<T>(to);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dsum = fmaf((float)doreg[qb][ks][j], (float)ov[j], dsum);
+      for (int j = 0; j < 8; ++j) {
+        qreg[qb][ks][j] = (T)((float)qraw[j] * a.scale_l2);
+        dsum = fmaf((float)doreg[qb][ks][j], (float)ov[j], dsum);
+      }
     }
     dsum = xhalf_sum(dsum);
     delta[qb] = dsum;
-    float ls = POS_INF; // rows past the end and fully masked rows get P = 0
+    float nl = BIGNEG; // rows past the end and fully masked rows get P = 0
     if (q < a.sq) {
       const float v = a.lse[(size_t)bh * a.sq + q];
-      if (v != NEG_INF) ls = v * FMHA_LOG2E;
+      if (v != NEG_INF) nl = -v * FMHA_LOG2E;
       if (h == 0) a.delta[(size_t)bh * a.sq + q] = dsum;
     }
-    lse2[qb] = ls;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      bxs[qb][j] = (T)0.f;
+      bxd[qb][j] = (T)0.f;
+    }
+    if (h == 0) {
+      T hi, lo;
+      split_hi_lo<T>(nl, hi, lo);
+      bxs[qb][0] = hi;
+      bxs[qb][1] = lo;
+      bxs[qb][2] = (T)1.f;
+      bxs[qb][3] = (T)1.f;
+      if (MASK == kMaskFull) { // constant part of a full mask's term
+        split_hi_lo<T>(a.mask_b, hi, lo);
+        bxs[qb][4] = hi;
+        bxs[qb][5] = lo;
+      }
+      split_hi_lo<T>(-dsum * a.inv_drop_scale, hi, lo);
+      bxd[qb][0] = hi;
+      bxd[qb][1] = lo;
+    }
   }
 
   int nkt = (a.sk + BK - 1) / BK;
@@ -125,22 +172,26 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
     const int need = qmax / BK + 1;
     if (need < nkt) nkt = need;
   }
+  const int kend = nkt * BK < a.sk ? nkt * BK : a.sk;
 
+  // ---- staging (unconditional loads: rows past the end re-read the last valid row; their
+  // scores are pushed to -60000 by the extra step, so P = dS = 0 for them)
   u32x4 kst[CPT], vst[CPT];
+  T mraw = (T)0.f;
+  bool mvalid = false;
   auto gload = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * NT;
       const int row = c / CPR, col = c % CPR;
-      const int kr = k0 + row;
-      u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-      if (kr < a.sk) {
-        kk = *(const u32x4 *)(Kb + (size_t)kr * D + col * 8);
-        vv = *(const u32x4 *)(Vb + (size_t)kr * D + col * 8);
-      }
-      kst[i] = kk;
-      vst[i] = vv;
+      int kr = k0 + row;
+      kr = kr < kend ? kr : kend - 1;
+      kst[i] = *(const u32x4 *)(Kb + (size_t)kr * D + col * 8);
+      vst[i] = *(const u32x4 *)(Vb + (size_t)kr * D + col * 8);
     }
+    const int kr = k0 + (tid & (BK - 1));
+    mvalid = kr < kend;
+    if (MASK == kMaskPerKey) mraw = mkey[mvalid ? kr : kend - 1];
   };
   auto lstore = [&](int stage) {
     char *kd = lds + stage * 2 * TILEB;
@@ -152,6 +203,28 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
       *(u32x4 *)(kd + row * ROWB + col * 16) = kst[i];
       *(u32x4 *)(vd + row * ROWB + col * 16) = vst[i];
     }
+    if (tid < BK) {
+      float mk = 0.f;
+      if (MASK == kMaskPerKey) mk = fmaf((float)mraw, a.mask_a, a.mask_b);
+      if (!mvalid) mk = BIGNEG;
+      T hi, lo;
+      split_hi_lo<T>(mk, hi, lo);
+      v8 x0, x1;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        x0[j] = (T)0.f;
+        x1[j] = (T)0.f;
+      }
+      x0[0] = (T)1.f;
+      x0[1] = (T)1.f;
+      x0[2] = hi;
+      x0[3] = lo;
+      x0[4] = (T)1.f;
+      x0[5] = (T)1.f;
+      v8 *dst = (v8 *)(ldsXb + stage * BK * XROWB + tid * XROWB);
+      dst[0] = x0;
+      dst[1] = x1;
+    }
   };
 
   const T *mrow[QB];
@@ -160,10 +233,11 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
     int q = q0w + qb * 32 + ql;
     if (q > a.sq - 1) q = a.sq - 1;
     mrow[qb] = nullptr;
-    if (MASK) mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
+    if (MASK == kMaskFull)
+      mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
   }
-  auto load4 = [&](const T *row, int kk, float out[4]) {
-    if (a.mask_vec && kk + 3 < a.sk) {
+  auto load4 = [&](const T *row, int kk, bool safe, float out[4]) {
+    if (safe) {
       v4 t = as_v4<T>(*(const u32x2 *)(row + kk));
 #pragma unroll
       for (int i = 0; i < 4; ++i) out[i] = (float)t[i];
@@ -191,85 +265,87 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
     if (kt + 1 < nkt) gload(k0 + BK);
     const char *ldsK = lds + cur * 2 * TILEB;
     const char *ldsV = ldsK + TILEB;
+    const char *ldsX = ldsXb + cur * BK * XROWB;
 
-    const bool active = !CAUSAL || (k0 <= q0w + QB * 32 - 1);
-    if (active) {
-      f32x16 s[QB][NSB], dp[QB][NSB];
+    // x^T = K.Q'^T + (mask - LSE) ; g^T = V.dO^T - delta/drop_scale   (accumulators visited round-robin)
+    f32x16 x[QB][NSB], g[QB][NSB];
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          x[qb][sb][r] = 0.f;
+          g[qb][sb][r] = 0.f;
+        }
+#pragma unroll
+    for (int ks = 0; ks <= KS; ++ks)
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            s[qb][sb][r] = 0.f;
-            dp[qb][sb][r] = 0.f;
-          }
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+        if (ks < KS) {
           const int off = (sb * 32 + ql) * ROWB + ks * 32 + h * 16;
           const v8 ka = as_v8<T>(*(const u32x4 *)(ldsK + off));
           const v8 va = as_v8<T>(*(const u32x4 *)(ldsV + off));
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) {
-            s[qb][sb] = E::mfma(ka, qreg[qb][ks], s[qb][sb]);
-            dp[qb][sb] = E::mfma(va, doreg[qb][ks], dp[qb][sb]);
+            x[qb][sb] = E::mfma(ka, qreg[qb][ks], x[qb][sb]);
+            g[qb][sb] = E::mfma(va, doreg[qb][ks], g[qb][sb]);
+          }
+        } else {
+          const v8 xa = as_v8<T>(*(const u32x4 *)(ldsX + (sb * 32 + ql) * XROWB + h * 16));
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            x[qb][sb] = E::mfma(xa, bxs[qb], x[qb][sb]);
+            g[qb][sb] = E::mfma(xa, bxd[qb], g[qb][sb]);
           }
         }
       }
 
-      const bool pred = (k0 + BK > a.sk) || (CAUSAL && (k0 + BK - 1 > q0w));
-      v8 dsfrag[QB][NSB][2];
+    const bool diag = CAUSAL && (k0 + BK - 1 > q0w);
+    const bool vec_ok = a.mask_vec && (k0 + BK <= a.sk);
+    v8 dsfrag[QB][NSB][2];
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        const int q = q0w + qb * 32 + ql;
+    for (int qb = 0; qb < QB; ++qb) {
+      const int q = q0w + qb * 32 + ql;
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb) {
+      for (int sb = 0; sb < NSB; ++sb) {
+        uint32_t wd[4] = {0u, 0u, 0u, 0u};
+        if (DROP == 1) drop_words_q(a.drop, (uint32_t)bh, (uint32_t)q, (uint32_t)(k0 + sb * 32), h, l, wd);
+        float ds[16];
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int kk = k0 + sb * 32 + 8 * g + 4 * h;
-            float mv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (MASK) {
-              load4(mrow[qb], kk, mv);
+        for (int gq = 0; gq < 4; ++gq) {
+          const int kk = k0 + sb * 32 + 8 * gq + 4 * h;
+          float mv[4] = {0.f, 0.f, 0.f, 0.f};
+          if (MASK == kMaskFull) load4(mrow[qb], kk, vec_ok, mv);
 #pragma unroll
-              for (int t = 0; t < 4; ++t) mv[t] = fmaf(mv[t], a.mask_a, a.mask_b);
-            }
-            uint32_t wd = 0;
-            if (DROP == 1) wd = drop_word(a.drop, (uint32_t)bh, (uint32_t)q, (uint32_t)(kk >> 2));
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              float x = fmaf(s[qb][sb][4 * g + t], a.scale_l2, mv[t]);
-              if (pred) {
-                const int k = kk + t;
-                const bool ok = (k < a.sk) && (!CAUSAL || k <= q);
-                x = ok ? x : NEG_INF;
-              }
-              const float p = fast_exp2(x - lse2[qb]);
-              float dpe = dp[qb][sb][4 * g + t];
-              if (DROP == 1) dpe = drop_keep_byte(wd, t, a.drop.thr) ? dpe * a.drop_scale : 0.f;
-              s[qb][sb][4 * g + t] = p * (dpe - delta[qb]);
-            }
+          for (int t = 0; t < 4; ++t) {
+            float xv = x[qb][sb][4 * gq + t];
+            if (MASK == kMaskFull) xv = fmaf(mv[t], a.mask_a, xv);
+            if (diag) xv = (kk + t <= q) ? xv : BIGNEG;
+            const float p = fast_exp2(xv);
+            float gv = g[qb][sb][4 * gq + t];
+            if (DROP == 1) gv = drop_keep_byte(wd[gq], t, a.drop.thr) ? gv * a.drop_scale : -delta[qb];
+            ds[4 * gq + t] = p * gv;
           }
         }
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb)
+        for (int c = 0; c < 2; ++c)
 #pragma unroll
-          for (int c = 0; c < 2; ++c)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) dsfrag[qb][sb][c][j] = (T)s[qb][sb][8 * c + j];
+          for (int j = 0; j < 8; ++j) dsfrag[qb][sb][c][j] = (T)ds[8 * c + j];
       }
-
-      // dQ^T += K^T . dS^T
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            const v8 kt_a = lds_load_a_transposed<T, ROWB>(ldsK, sb * 32, db * 32, c, l);
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) dq[qb][db] = E::mfma(kt_a, dsfrag[qb][sb][c], dq[qb][db]);
-          }
     }
+
+    // dQ^T += K^T . dS^T
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const v8 kt_a = lds_load_a_transposed<T, ROWB>(ldsK, sb * 32, db * 32, c, l);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) dq[qb][db] = E::mfma(kt_a, dsfrag[qb][sb][c], dq[qb][db]);
+        }
 
     if (kt + 1 < nkt) lstore(cur ^ 1);
     __syncthreads();
@@ -283,34 +359,37 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
+        for (int gq = 0; gq < 4; ++gq) {
           v4 t;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) t[i] = (T)(dq[qb][db][4 * g + i] * a.scale);
-          *(v4 *)(dQb + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
+          for (int i = 0; i < 4; ++i) t[i] = (T)(dq[qb][db][4 * gq + i] * a.scale);
+          *(v4 *)(dQb + (size_t)q * D + db * 32 + 8 * gq + 4 * h) = t;
         }
     }
   }
 }
 
 // --------------------------------------------------------------------------- dK, dV
-template <typename T, int D, int KB, int NW, bool MASK, bool CAUSAL, int DROP>
+template <typename T, int D, int KB, int NW, int MASK, bool CAUSAL, int DROP>
 __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = BwdCfg<D>;
   constexpr int BQ = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, TILEB = C::TILEB;
+  constexpr int XROWB = C::XROWB;
   constexpr int NT = NW * 64;
   constexpr int KT = NW * KB * 32;
   constexpr int CPR = D / 8;
   constexpr int CPT = BQ * CPR / NT;
   constexpr float NEG_INF = -__builtin_inff();
-  constexpr float POS_INF = __builtin_inff();
-  static_assert(NT >= 2 * BQ, "row statistics are staged by the first 2*BQ threads");
+  constexpr float BIGNEG = -60000.f;
+  static_assert(NT >= BQ, "row statistics are staged by the first BQ threads");
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  float *ldsStat = (float *)(lds + 4 * TILEB); // [stage][{lse2, delta}][BQ]
+  // extra rows per query: [stage][{score row (-L_hi,-L_lo,1,1,1,1,0..), dP row (-d_hi,-d_lo,0..)}][BQ]
+  char *ldsXb = lds + 4 * TILEB;
+  float *ldsDl = (float *)(ldsXb + 2 * 2 * BQ * XROWB); // [stage][BQ] delta (dropout path)
 
   const int tid = threadIdx.x;
   const int w = tid >> 6, l = tid & 63, kl = l & 31, h = l >> 5;
@@ -329,9 +408,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
   const float *lseb = a.lse + (size_t)bh * a.sq;
   const float *delb = a.delta + (size_t)bh * a.sq;
 
-  // ---- per-key operands: K and V rows as B operands
+  // ---- per-key operands: K' and V rows as B operands, the extra-step columns
   v8 kreg[KB][KS], vreg[KB][KS];
-  float mcol[KB];
+  v8 bxs[KB], bxd[KB]; // (1, 1, mask_hi, mask_lo, c_hi, c_lo, 0, 0) and (1, 1, 0 ...) on the lower half-wave
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     const int key = k0w + kb * 32 + kl;
@@ -343,46 +422,59 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
         tk = *(const u32x4 *)(Kb + off);
         tv = *(const u32x4 *)(Vb + off);
       }
-      kreg[kb][ks] = as_v8<T>(tk);
+      const v8 kraw = as_v8<T>(tk);
       vreg[kb][ks] = as_v8<T>(tv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) kreg[kb][ks][j] = (T)((float)kraw[j] * a.scale_l2);
     }
-    mcol[kb] = 0.f;
-    if (MASK && a.mask_sq == 0 && key < a.sk) // mask constant along queries: one value per lane
-      mcol[kb] = fmaf((float)((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + key], a.mask_a, a.mask_b);
+    float mk = 0.f;
+    if (MASK == kMaskPerKey && key < a.sk)
+      mk = fmaf((float)((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + key], a.mask_a, a.mask_b);
+    if (key >= a.sk) mk = BIGNEG;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      bxs[kb][j] = (T)0.f;
+      bxd[kb][j] = (T)0.f;
+    }
+    if (h == 0) {
+      T hi, lo;
+      bxs[kb][0] = (T)1.f;
+      bxs[kb][1] = (T)1.f;
+      split_hi_lo<T>(mk, hi, lo);
+      bxs[kb][2] = hi;
+      bxs[kb][3] = lo;
+      if (MASK == kMaskFull) {
+        split_hi_lo<T>(a.mask_b, hi, lo);
+        bxs[kb][4] = hi;
+        bxs[kb][5] = lo;
+      }
+      bxd[kb][0] = (T)1.f;
+      bxd[kb][1] = (T)1.f;
+    }
   }
-  const T *mbase = MASK ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
+  const T *mbase = (MASK == kMaskFull) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
   const int nqt = (a.sq + BQ - 1) / BQ;
   const int qt0 = CAUSAL ? (ktile * KT) / BQ : 0; // first query tile that sees any of these keys
 
   u32x4 qst[CPT], dst[CPT];
-  float stat = 0.f;
+  float lraw = 0.f, draw = 0.f;
+  bool qvalid = false;
   auto gload = [&](int q0) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * NT;
       const int row = c / CPR, col = c % CPR;
-      const int qr = q0 + row;
-      u32x4 qq = {0u, 0u, 0u, 0u}, dd = {0u, 0u, 0u, 0u};
-      if (qr < a.sq) {
-        qq = *(const u32x4 *)(Qb + (size_t)qr * D + col * 8);
-        dd = *(const u32x4 *)(dOb + (size_t)qr * D + col * 8);
-      }
-      qst[i] = qq;
-      dst[i] = dd;
+      int qr = q0 + row;
+      qr = qr < a.sq ? qr : a.sq - 1;
+      qst[i] = *(const u32x4 *)(Qb + (size_t)qr * D + col * 8);
+      dst[i] = *(const u32x4 *)(dOb + (size_t)qr * D + col * 8);
     }
-    if (tid < BQ) {
-      const int qr = q0 + tid;
-      float v = POS_INF;
-      if (qr < a.sq) {
-        const float t = lseb[qr];
-        if (t != NEG_INF) v = t * FMHA_LOG2E;
-      }
-      stat = v;
-    } else if (tid < 2 * BQ) {
-      const int qr = q0 + tid - BQ;
-      stat = qr < a.sq ? delb[qr] : 0.f;
-    }
+    int qr = q0 + (tid & (BQ - 1));
+    qvalid = qr < a.sq;
+    qr = qvalid ? qr : a.sq - 1;
+    lraw = lseb[qr];
+    draw = delb[qr];
   };
   auto lstore = [&](int stage) {
     char *qd = lds + stage * 2 * TILEB;
@@ -394,7 +486,39 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
       *(u32x4 *)(qd + row * ROWB + col * 16) = qst[i];
       *(u32x4 *)(dd + row * ROWB + col * 16) = dst[i];
     }
-    if (tid < 2 * BQ) ldsStat[stage * 2 * BQ + tid] = stat;
+    if (tid < BQ) {
+      // rows past the end (whose Q/dO rows repeat the last valid row) and fully masked rows: P = 0
+      float nl = BIGNEG, dl = 0.f;
+      if (qvalid && lraw != NEG_INF) {
+        nl = -lraw * FMHA_LOG2E;
+        dl = draw;
+      }
+      v8 xs, xd, z;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        xs[j] = (T)0.f;
+        xd[j] = (T)0.f;
+        z[j] = (T)0.f;
+      }
+      T hi, lo;
+      split_hi_lo<T>(nl, hi, lo);
+      xs[0] = hi;
+      xs[1] = lo;
+      xs[2] = (T)1.f;
+      xs[3] = (T)1.f;
+      xs[4] = (T)1.f;
+      xs[5] = (T)1.f;
+      split_hi_lo<T>(-dl * a.inv_drop_scale, hi, lo);
+      xd[0] = hi;
+      xd[1] = lo;
+      v8 *ds_ = (v8 *)(ldsXb + (stage * 2 + 0) * BQ * XROWB + tid * XROWB);
+      v8 *dd_ = (v8 *)(ldsXb + (stage * 2 + 1) * BQ * XROWB + tid * XROWB);
+      ds_[0] = xs;
+      ds_[1] = z;
+      dd_[0] = xd;
+      dd_[1] = z;
+      ldsDl[stage * BQ + tid] = dl;
+    }
   };
 
   f32x16 dk[KB][DB], dv[KB][DB];
@@ -420,102 +544,108 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
     if (qt + 1 < nqt) gload(q0 + BQ);
     const char *ldsQ = lds + cur * 2 * TILEB;
     const char *ldsDO = ldsQ + TILEB;
-    const float *ldsL = ldsStat + cur * 2 * BQ;
-    const float *ldsDl = ldsL + BQ;
+    const char *ldsXs = ldsXb + (cur * 2 + 0) * BQ * XROWB;
+    const char *ldsXd = ldsXb + (cur * 2 + 1) * BQ * XROWB;
+    const float *ldsD = ldsDl + cur * BQ;
 
-    // queries of this tile all precede this wave's keys: nothing visible under the causal mask
-    const bool active = !CAUSAL || (q0 + BQ - 1 >= k0w);
-    if (active) {
-      f32x16 s[KB][NSB], dp[KB][NSB];
+    // x = Q.K'^T + (mask - LSE) ; g = dO.V^T - delta/drop_scale
+    f32x16 x[KB][NSB], g[KB][NSB];
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          x[kb][sb][r] = 0.f;
+          g[kb][sb][r] = 0.f;
+        }
+#pragma unroll
+    for (int ks = 0; ks <= KS; ++ks)
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            s[kb][sb][r] = 0.f;
-            dp[kb][sb][r] = 0.f;
-          }
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+        if (ks < KS) {
           const int off = (sb * 32 + kl) * ROWB + ks * 32 + h * 16;
           const v8 qa = as_v8<T>(*(const u32x4 *)(ldsQ + off));
           const v8 da = as_v8<T>(*(const u32x4 *)(ldsDO + off));
 #pragma unroll
           for (int kb = 0; kb < KB; ++kb) {
-            s[kb][sb] = E::mfma(qa, kreg[kb][ks], s[kb][sb]);
-            dp[kb][sb] = E::mfma(da, vreg[kb][ks], dp[kb][sb]);
+            x[kb][sb] = E::mfma(qa, kreg[kb][ks], x[kb][sb]);
+            g[kb][sb] = E::mfma(da, vreg[kb][ks], g[kb][sb]);
+          }
+        } else {
+          const int off = (sb * 32 + kl) * XROWB + h * 16;
+          const v8 xsa = as_v8<T>(*(const u32x4 *)(ldsXs + off));
+          const v8 xda = as_v8<T>(*(const u32x4 *)(ldsXd + off));
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+            x[kb][sb] = E::mfma(xsa, bxs[kb], x[kb][sb]);
+            g[kb][sb] = E::mfma(xda, bxd[kb], g[kb][sb]);
           }
         }
       }
 
-      const bool pred = (q0 + BQ > a.sq) || (k0w + KB * 32 > a.sk) || (CAUSAL && (k0w + KB * 32 - 1 > q0));
-      v8 pfrag[KB][NSB][2], dsfrag[KB][NSB][2];
+    const bool diag = CAUSAL && (k0w + KB * 32 - 1 > q0);
+    v8 pfrag[KB][NSB][2], dsfrag[KB][NSB][2];
 #pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        const int key = k0w + kb * 32 + kl;
+    for (int kb = 0; kb < KB; ++kb) {
+      const int key = k0w + kb * 32 + kl;
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb) {
-          f32x16 pd;
+      for (int sb = 0; sb < NSB; ++sb) {
+        uint32_t wd[4][4];
+        if (DROP == 1) drop_words_k(a.drop, (uint32_t)bh, (uint32_t)(q0 + sb * 32), (uint32_t)key, h, l, wd);
+        float pz[16], ds[16];
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int qq = sb * 32 + 8 * g + 4 * h; // row in tile of t = 0
-            const f32x4 L = *(const f32x4 *)(ldsL + qq);
-            const f32x4 Dl = *(const f32x4 *)(ldsDl + qq);
-            uint32_t o4[4] = {0u, 0u, 0u, 0u};
-            if (DROP == 1) drop_block(a.drop, (uint32_t)bh, (uint32_t)((q0 + qq) >> 2), (uint32_t)(key >> 2), o4);
+        for (int gq = 0; gq < 4; ++gq) {
+          const int qq = sb * 32 + 8 * gq + 4 * h; // row in tile of t = 0
+          f32x4 Dl = {0.f, 0.f, 0.f, 0.f};
+          if (DROP == 1) Dl = *(const f32x4 *)(ldsD + qq);
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              const int q = q0 + qq + t;
-              float mv = mcol[kb];
-              if (MASK && a.mask_sq != 0) {
-                const int qc = q < a.sq ? q : a.sq - 1;
-                const int kc = key < a.sk ? key : a.sk - 1;
-                mv = fmaf((float)mbase[(size_t)qc * a.mask_sq + kc], a.mask_a, a.mask_b);
-              }
-              float x = fmaf(s[kb][sb][4 * g + t], a.scale_l2, mv);
-              if (pred) {
-                const bool ok = (q < a.sq) && (key < a.sk) && (!CAUSAL || key <= q);
-                x = ok ? x : NEG_INF;
-              }
-              const float p = fast_exp2(x - L[t]);
-              float dpe = dp[kb][sb][4 * g + t];
-              float pz = p;
-              if (DROP == 1) {
-                const bool keep = drop_keep_byte(o4[t], key & 3, a.drop.thr);
-                dpe = keep ? dpe * a.drop_scale : 0.f;
-                pz = keep ? p * a.drop_scale : 0.f;
-              }
-              pd[4 * g + t] = pz;
-              s[kb][sb][4 * g + t] = p * (dpe - Dl[t]);
+          for (int t = 0; t < 4; ++t) {
+            const int q = q0 + qq + t;
+            float xv = x[kb][sb][4 * gq + t];
+            if (MASK == kMaskFull) {
+              const int qc = q < a.sq ? q : a.sq - 1;
+              const int kc = key < a.sk ? key : a.sk - 1;
+              xv = fmaf((float)mbase[(size_t)qc * a.mask_sq + kc], a.mask_a, xv);
             }
+            if (diag) xv = (key <= q) ? xv : BIGNEG;
+            const float p = fast_exp2(xv);
+            float gv = g[kb][sb][4 * gq + t];
+            float pzv = p;
+            if (DROP == 1) {
+              const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
+              gv = keep ? gv * a.drop_scale : -Dl[t];
+              pzv = keep ? p * a.drop_scale : 0.f;
+            }
+            pz[4 * gq + t] = pzv;
+            ds[4 * gq + t] = p * gv;
           }
-#pragma unroll
-          for (int c = 0; c < 2; ++c)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              pfrag[kb][sb][c][j] = (T)pd[8 * c + j];
-              dsfrag[kb][sb][c][j] = (T)s[kb][sb][8 * c + j];
-            }
         }
-      }
-
-      // dV^T += dO^T . (P o Z) ;  dK^T += Q^T . dS
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            const v8 dot = lds_load_a_transposed<T, ROWB>(ldsDO, sb * 32, db * 32, c, l);
-            const v8 qtr = lds_load_a_transposed<T, ROWB>(ldsQ, sb * 32, db * 32, c, l);
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-              dv[kb][db] = E::mfma(dot, pfrag[kb][sb][c], dv[kb][db]);
-              dk[kb][db] = E::mfma(qtr, dsfrag[kb][sb][c], dk[kb][db]);
-            }
+          for (int j = 0; j < 8; ++j) {
+            pfrag[kb][sb][c][j] = (T)pz[8 * c + j];
+            dsfrag[kb][sb][c][j] = (T)ds[8 * c + j];
           }
+      }
     }
+
+    // dV^T += dO^T . (P o Z) ;  dK^T += Q^T . dS
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const v8 dot = lds_load_a_transposed<T, ROWB>(ldsDO, sb * 32, db * 32, c, l);
+          const v8 qtr = lds_load_a_transposed<T, ROWB>(ldsQ, sb * 32, db * 32, c, l);
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+            dv[kb][db] = E::mfma(dot, pfrag[kb][sb][c], dv[kb][db]);
+            dk[kb][db] = E::mfma(qtr, dsfrag[kb][sb][c], dk[kb][db]);
+          }
+        }
 
     if (qt + 1 < nqt) lstore(cur ^ 1);
     __syncthreads();
@@ -530,14 +660,14 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
+        for (int gq = 0; gq < 4; ++gq) {
           v4 tk, tv;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            tk[i] = (T)(dk[kb][db][4 * g + i] * a.scale);
-            tv[i] = (T)dv[kb][db][4 * g + i];
+            tk[i] = (T)(dk[kb][db][4 * gq + i] * a.scale);
+            tv[i] = (T)dv[kb][db][4 * gq + i];
           }
-          const size_t off = (size_t)key * D + db * 32 + 8 * g + 4 * h;
+          const size_t off = (size_t)key * D + db * 32 + 8 * gq + 4 * h;
           *(v4 *)(dKb + off) = tk;
           *(v4 *)(dVb + off) = tv;
         }

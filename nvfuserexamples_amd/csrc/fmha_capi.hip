@@ -201,11 +201,13 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   a.scale = p->scale;
   a.scale_l2 = p->scale * FMHA_LOG2E;
   a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
+  if (!(a.drop_scale > 0.f)) return FMHA_E_ARG;
+  a.inv_drop_scale = 1.f / a.drop_scale;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
 
   BwdVariant v;
-  v.mask = a.mask != nullptr;
+  v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0;
   hipStream_t s = (hipStream_t)hip_stream;

@@ -166,6 +166,60 @@ FMHA_DEV void drop_block(const DropCtx &c, uint32_t bh, uint32_t q4, uint32_t k4
   Philox::run(c.off_lo, c.off_hi, (uint32_t)blk, (uint32_t)(blk >> 32), c.seed_lo, c.seed_hi, o);
 }
 
+// ---- sharing one Philox call per 4x4 block among the four lanes that need it
+// (v_mov_b32 with a DPP quad permutation; lanes 4n..4n+3 form a quad)
+template <int CTRL> FMHA_DEV uint32_t quad_perm(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, false);
+}
+
+// 4x4 transpose inside a quad: on entry lane i holds a[0..3]; on exit a[g] is what lane g held
+// in a[i].  Two butterfly stages (partner lane ^1, then ^2).
+FMHA_DEV void quad_transpose4(uint32_t a[4], int lane) {
+  const bool odd = lane & 1;
+  // stage 1: exchange a[1]<->a[0] and a[3]<->a[2] with the lane ^ 1
+  uint32_t s0 = odd ? a[0] : a[1];
+  uint32_t s1 = odd ? a[2] : a[3];
+  s0 = quad_perm<0xB1>(s0);
+  s1 = quad_perm<0xB1>(s1);
+  if (odd) { a[0] = s0; a[2] = s1; } else { a[1] = s0; a[3] = s1; }
+  // stage 2: exchange the (a[2],a[3]) pair of lanes 0,1 with the (a[0],a[1]) pair of lanes 2,3
+  const bool hi = lane & 2;
+  uint32_t u0 = hi ? a[0] : a[2];
+  uint32_t u1 = hi ? a[1] : a[3];
+  u0 = quad_perm<0x4E>(u0);
+  u1 = quad_perm<0x4E>(u1);
+  if (hi) { a[0] = u0; a[1] = u1; } else { a[2] = u0; a[3] = u1; }
+}
+
+// Lane = query layout.  The lane owns query q and, in one 32-key block starting at key kb32, the
+// keys 4h + 8g + t (g, t = 0..3).  Returns in w[g] the word holding the four random bytes of
+// (q, keys 4h+8g .. +3).  The four lanes of a quad share q/4: each evaluates the block of ONE g
+// and the words are exchanged, instead of every lane evaluating all four.
+FMHA_DEV void drop_words_q(const DropCtx &c, uint32_t bh, uint32_t q, uint32_t kb32, int h, int lane,
+                           uint32_t w[4]) {
+  const uint32_t g = (uint32_t)lane & 3u;
+  drop_block(c, bh, q >> 2, (kb32 >> 2) + (uint32_t)h + 2u * g, w); // w[j] = word of query row 4*(q/4)+j
+  quad_transpose4(w, lane);                                        // w[g] = word of row q in block g
+}
+
+// Lane = key layout.  The lane owns key k and, in one 32-query block starting at qb32, the
+// queries 4h + 8g + t.  Returns in w[g][t] the word of query row (qb32 + 4h + 8g + t) in the
+// block containing key k (the lane's byte is k % 4).  Lanes of a quad share k/4: lane i
+// evaluates the block of g = i and broadcasts its four words.
+FMHA_DEV void drop_words_k(const DropCtx &c, uint32_t bh, uint32_t qb32, uint32_t k, int h, int lane,
+                           uint32_t w[4][4]) {
+  const uint32_t g = (uint32_t)lane & 3u;
+  uint32_t o[4];
+  drop_block(c, bh, (qb32 >> 2) + (uint32_t)h + 2u * g, k >> 2, o);
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    w[0][t] = quad_perm<0x00>(o[t]);
+    w[1][t] = quad_perm<0x55>(o[t]);
+    w[2][t] = quad_perm<0xAA>(o[t]);
+    w[3][t] = quad_perm<0xFF>(o[t]);
+  }
+}
+
 FMHA_DEV bool drop_keep_byte(uint32_t word, int t, uint32_t thr) {
   return ((word >> (8 * t)) & 0xffu) >= thr;
 }

@@ -412,15 +412,15 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
     if (DROP == 1) {
       const int q = q0w + qb * 32 + ql;
 #pragma unroll
-      for (int sb = 0; sb < NSB; ++sb)
+      for (int sb = 0; sb < NSB; ++sb) {
+        uint32_t wd[4];
+        drop_words_q(a.drop, (uint32_t)bh, (uint32_t)q, (uint32_t)(tile * BK + sb * 32), h, l, wd);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int kk = tile * BK + sb * 32 + 8 * g + 4 * h;
-          const uint32_t wd = drop_word(a.drop, (uint32_t)bh, (uint32_t)q, (uint32_t)(kk >> 2));
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            if (!drop_keep_byte(wd, t, a.drop.thr)) pk[sb][g >> 1][4 * (g & 1) + t] = (T)0.f;
-        }
+            if (!drop_keep_byte(wd[g], t, a.drop.thr)) pk[sb][g >> 1][4 * (g & 1) + t] = (T)0.f;
+      }
     }
   };
 

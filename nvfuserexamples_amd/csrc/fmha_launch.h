@@ -23,7 +23,7 @@ int fwd_dispatch_bf16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 
 struct BwdVariant {
-  bool mask;
+  int mask;  // kMaskNone / kMaskPerKey / kMaskFull
   bool causal;
   int drop; // 0 none, 1 Philox
 };
