@@ -130,6 +130,9 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="input sets rotated to defeat the last-level cache")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-bwd", action="store_true", help="skip the train-step (fwd+bwd) leg")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times: under `rocprofv3 --pmc FETCH_SIZE` "
+                         "(or WRITE_SIZE) its known traffic calibrates the counter for the attention kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; attention shards over batch*heads without "
@@ -144,6 +147,14 @@ def main():
         return 2
     L = capi.lib()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    if args.traffic_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)   # reads 256 MiB, writes 256 MiB per launch
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- forward (headline)
     sets = make_inputs(torch, capi, args.sets)

@@ -143,9 +143,9 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
-  // Two query blocks per wave halve the LDS traffic per MFMA; use them once there is
-  // enough work to fill the chip with 256-row tiles.
-  v.qb = (p->sq >= 256 && (long long)p->bh * ((p->sq + 255) / 256) >= 512) ? 2 : 1;
+  // One 32-query block per wave keeps two waves per SIMD resident (two blocks need > 256 VGPRs);
+  // measured faster at every shape tried.  The two-block variants stay selectable for tuning.
+  v.qb = 1;
   const int force = env_int("FMHA_FWD_QB", 0);
   if (force == 1 || force == 2) v.qb = force;
 

@@ -67,18 +67,17 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
   const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
-  v8 qreg[QB][KS];
+  // Q rows are loaded unconditionally (rows past the end repeat the last valid row and are
+  // never stored) and converted only after the first K/V tiles have been requested, so that
+  // the whole prologue costs one global round trip instead of three.
+  u32x4 qraw[QB][KS];
+  v8 qreg[QB][KS]; // filled in the prologue
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const int q = q0w + qb * 32 + ql;
+    int q = q0w + qb * 32 + ql;
+    q = q < a.sq ? q : a.sq - 1;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      u32x4 t = {0u, 0u, 0u, 0u};
-      if (q < a.sq) t = *(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8);
-      const v8 raw = as_v8<T>(t);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
-    }
+    for (int ks = 0; ks < KS; ++ks) qraw[qb][ks] = *(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8);
   }
 
   // ---- key range: tiles [0, nkt), keys [0, kend); the count is padded to even with an
@@ -495,10 +494,19 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   // ---- prologue: K(0), K(1) into LDS, first product of tile 0
   gloadK(0, st0);
   gloadK(1, st1);
+  gloadV(0, st1);
+  // Q' = Q * scale * log2(e) as B-operand registers
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const v8 raw = as_v8<T>(qraw[qb][ks]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
+    }
   lstoreK(0, st0);
   lstoreK(1, st1);
-  gloadK(2, st1);
-  gloadV(0, st1);
+  gloadK(2, st1); // K(2) joins V(0) in the set that the first iteration writes to LDS
   __syncthreads();
   g1(0, xA, bkA);
   __syncthreads(); // tile 0's K stage is refilled during the first iteration
