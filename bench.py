@@ -26,6 +26,8 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
+# rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) of the headline forward kernel, bytes per launch
+MEASURED_TRAFFIC_BYTES = int((98511 + 32768) * 1024)
 
 B, H, S, D = 32, 16, 512, 64
 
@@ -91,6 +93,22 @@ def time_steps(torch, step, steps, warmup):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3
     return e0.elapsed_time(e1) / steps, wall / steps
+
+
+def time_launches(torch, step, steps, warmup):
+    """Average duration of ONE launch: a HIP event pair around every launch of the timed region
+    (same stream as the kernels).  Excludes the idle gap between back-to-back launches, so it is
+    the figure comparable with rocprofv3's per-kernel average."""
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for i, (a, b) in enumerate(ev):
+        a.record()
+        step(i)
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in ev) / steps
 
 
 def cpu_baseline(torch, budget_s=12.0):
@@ -173,6 +191,8 @@ def main():
     def fwd_warm(i):
         L.fmha_fwd_launch(C.byref(fps[0]), stream)
     ms_warm, _ = time_steps(torch, fwd_warm, args.steps, args.warmup)
+    ms_launch = time_launches(torch, fwd_step, args.steps, args.warmup)
+    tflops_launch = flops / (ms_launch * 1e-3) / 1e12
     del sets, fps
 
     out = {
@@ -183,13 +203,18 @@ def main():
         "config": {"workload": "BERT-large attention forward: B32 H16 S512 D64 fp16, additive [B,1,1,S] "
                                "padding mask (valid length U{256..512}), scale 1/8, no dropout",
                    "layout": "[B*H,S,D] contiguous", "input_sets_rotated": args.sets},
-        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_MFMA_TFLOPS, 4), "traffic": None,
+        # achieved = algorithmic flops of one launch / mean launch duration (event pair per launch);
+        # traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
+        # counter reads for a 256 MiB copy (profiles/fmha_fwd_pipe_kernel_B32H16S512D64_f16.md)
+        "roofline": {"bound": "mfma", "achieved": round(tflops_launch, 2), "peak": PEAK_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tflops_launch / PEAK_MFMA_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "fmha_fwd_pipe_kernel<f16,D64,per-key mask>", "flops_per_launch": flops,
                      "algorithmic_bytes_per_launch": bytes_,
                      "hbm_achieved_GBps": round(bytes_ / (ms * 1e-3) / 1e9, 1),
                      "hbm_frac": round(bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                     "launch_us": round(ms * 1e3, 2)},
+                     "hbm_achieved_GBps_launch": round(bytes_ / (ms_launch * 1e-3) / 1e9, 1),
+                     "launch_us": round(ms_launch * 1e3, 2)},
         "fwd_warm_cache": {"ms_per_step": round(ms_warm, 5),
                            "tflops": round(flops / (ms_warm * 1e-3) / 1e12, 2)},
         "host_wall_ms_per_step": round(wall_ms, 5),

@@ -6,6 +6,7 @@
 """
 import importlib.util
 import os
+import sys
 
 __all__ = ["load_ops"]
 
@@ -14,6 +15,9 @@ def load_ops():
     """Import the in-tree ``mha_manual`` extension (registers torch.ops.mha_manual.*).
 
     Raises if it has not been built; there is no fallback implementation."""
+    import torch
+    if "mha_manual" in sys.modules:  # already imported (by this function or by `import mha_manual`)
+        return torch.ops.mha_manual
     from . import build
     path = build.ext_path()
     if not os.path.exists(path):
@@ -21,5 +25,5 @@ def load_ops():
     spec = importlib.util.spec_from_file_location("mha_manual", path)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
-    import torch
+    sys.modules["mha_manual"] = mod
     return torch.ops.mha_manual

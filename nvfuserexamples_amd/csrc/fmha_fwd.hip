@@ -16,7 +16,10 @@
 namespace fmha {
 namespace {
 
-constexpr int kNW = 4;
+#ifndef FMHA_FWD_NW
+#define FMHA_FWD_NW 4
+#endif
+constexpr int kNW = FMHA_FWD_NW;
 
 template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
   using Cfg = FwdCfg<FMHA_TU_D>;
