@@ -143,11 +143,24 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
-  // One 32-query block per wave keeps two waves per SIMD resident (two blocks need > 256 VGPRs);
-  // measured faster at every shape tried.  The two-block variants stay selectable for tuning.
+  // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
+  // flop.  That pays (3-5 % measured) for the plain variants at head dim 64 when there is
+  // enough work for every resident workgroup to get several 256-query items; with dropout, a
+  // causal or a full mask the per-element work dominates and one block per wave is faster.
   v.qb = 1;
-  const int force = env_int("FMHA_FWD_QB", 0);
-  if (force == 1 || force == 2) v.qb = force;
+  if (p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull) {
+    static const int cus = [] {
+      int dev = 0, n = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        n = 0;
+      return n;
+    }();
+    const long long items2 = (long long)p->bh * ((p->sq + 255) / 256);
+    if (cus > 0 && items2 >= 4LL * cus) v.qb = 2;
+  }
+  const int force = env_int("FMHA_FWD_QB", 0); // tuning override: 1 or 2
+  if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;
 
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;

@@ -22,20 +22,36 @@ namespace {
 constexpr int kNW = FMHA_FWD_NW;
 
 template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
-  using Cfg = FwdCfg<FMHA_TU_D>;
+  constexpr bool kPipe = DROP != 2;
+  constexpr int kLds = kPipe ? PipeCfg<FMHA_TU_D, QB>::lds_bytes(kNW) : FwdCfg<FMHA_TU_D>::LDS_BYTES;
   // tensor dropout and the save pass run on the plain loop; everything else is software-pipelined
   auto kern = [] {
     if constexpr (DROP == 2) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
     else return fmha_fwd_pipe_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
   }();
-  static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-  if (attr != hipSuccess) return 2;
+  // once per kernel: allow the dynamic LDS size, and for the persistent kernel find how many
+  // workgroups the device keeps resident (that is its grid size)
+  static const int resident = [&]() -> int {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds) !=
+        hipSuccess)
+      return -1;
+    if (!kPipe) return 0;
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kern), kNW * 64, kLds) !=
+            hipSuccess ||
+        cus <= 0 || per_cu <= 0)
+      return -1;
+    return cus * per_cu;
+  }();
+  if (resident < 0) return 2;
   constexpr int QT = kNW * QB * 32;
   a.nqt = (a.sq + QT - 1) / QT;
-  const long long nblk = (long long)a.bh * a.nqt;
+  long long nblk = (long long)a.bh * a.nqt;
   if (nblk > 0x7fffffffLL) return 2;
-  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(kNW * 64), Cfg::LDS_BYTES, s, a);
+  if (kPipe && nblk > resident) nblk = resident;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(kNW * 64), kLds, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
@@ -52,7 +68,7 @@ template <int QB, int MASK> int by_causal(FwdArgs &a, const FwdVariant &v, hipSt
 #ifdef FMHA_DEV_MINIMAL
 // development builds: only the variants the headline benchmark uses
 template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
-  if (QB != 1 || v.causal || v.drop) return 1;
+  if (v.causal || v.drop) return 1;
   if (v.mask == kMaskPerKey) return launch<1, kMaskPerKey, false, 0>(a, s);
   if (v.mask == kMaskNone) return launch<1, kMaskNone, false, 0>(a, s);
   return 1;
@@ -78,8 +94,12 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
     return launch<1, kMaskNone, false, 2>(a, s);
   }
 #if FMHA_TU_D == 64
-  // two query blocks per wave only where their accumulators fit the register file
-  if (v.qb == 2) return by_mask<2>(a, v, s);
+  // two query blocks per wave: only where their accumulators fit the register file and only
+  // for the variants the host ever selects them for
+  if (v.qb == 2) {
+    if (v.causal || v.drop != 0 || v.mask == kMaskFull) return 1;
+    return v.mask == kMaskPerKey ? launch<2, kMaskPerKey, false, 0>(a, s) : launch<2, kMaskNone, false, 0>(a, s);
+  }
 #endif
   return by_mask<1>(a, v, s);
 }

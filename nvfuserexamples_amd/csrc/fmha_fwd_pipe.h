@@ -14,6 +14,24 @@
 // LDS and fetches K(t+2) and V(t); both still fit two stages each because the stage a
 // fetch overwrites was last read one iteration earlier.
 //
+// K and V tiles go from global memory straight into LDS (global_load_lds_dwordx4: every
+// lane names a 16-byte global chunk and the wave's 64 chunks land in 1 KiB of consecutive
+// LDS), issued at the top of an iteration and awaited at its end, so no registers and no
+// VALU/LDS-write issue slots are spent on staging.  Consecutive placement rules out row
+// padding, so a tile is kept as D/64 panels of 64 columns, each panel [key][8 chunks of 16
+// bytes] with a 128-byte pitch, and chunk c of row r sits at position c ^ ((r >> 1) & 7):
+// sixteen consecutive rows then spread one logical chunk over all sixteen 16-byte bank
+// groups, which is what a conflict-free ds_read_b128 needs.  The lane simply fetches the
+// chunk that belongs at its position.  The loads are written as inline assembly with
+// hand-placed s_waitcnt: the compiler would otherwise wait for all of them before any
+// later LDS read.
+//
+// Workgroups are persistent: the grid holds as many workgroups as the chip keeps resident
+// and each walks a strided list of (head, query tile) items.  The K and extra-row streams
+// simply run on into the next item's first tiles, and the next item's Q rows are copied
+// into an LDS buffer of their own as soon as the current Q has been read, so that only the
+// first item of a workgroup waits for global memory before it can start computing.
+//
 // x(t+1) is started before the softmax of tile t may raise the reference exponent, so
 // each x buffer remembers the reference that was baked into it; a mismatch sends that
 // tile through the (rare) correction path, which re-bases the exponentials.
@@ -24,14 +42,43 @@
 
 namespace fmha {
 
+template <int D, int QB> struct PipeCfg {
+  // keys per LDS tile: the two in-flight score buffers of a wave hold QB x BK/32 accumulator
+  // tiles each, which is what the register file can carry
+  static constexpr int BK = 64 / QB;
+  static constexpr int NSB = BK / 32; // 32-key sub-blocks per tile
+  static constexpr int KS = D / 16;   // contraction steps of K.Q^T
+  static constexpr int DB = D / 32;   // 32-row blocks of O^T
+  static constexpr int ROWB = 128;    // LDS row pitch in bytes of one 64-column panel (unpadded, swizzled)
+  static constexpr int PANELB = BK * ROWB;
+  static constexpr int TILEB = (D / 64) * PANELB;
+  static constexpr int XROWB = 32;    // pitch of the extra-contraction-step rows (16 elements)
+  // The next item's Q rows are prefetched into LDS where that still leaves room for two
+  // workgroups per CU; otherwise Q is loaded from global memory when the item starts.
+  static constexpr bool QLDS = (D == 64);
+  static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * XROWB; // {K,V} x 2 stages + extra rows x 2 stages
+  static constexpr int lds_bytes(int nw) { return LDS_BYTES + (QLDS ? nw * QB * 32 * D * 2 : 0); }
+};
+
+// One wave-wide 16-byte-per-lane copy from global memory into LDS: lane i's chunk lands at
+// LDS byte address lds_wave_base + 16*i.  lds_wave_base must be wave-uniform.
+FMHA_DEV void dma_global_to_lds_b128(const void *gptr, uint32_t lds_wave_base) {
+  // the readfirstlane is free when the compiler already knows the value to be uniform
+  lds_wave_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr)
+               : "memory");
+}
+// Wait until every copy issued with dma_global_to_lds_b128 by this wave has landed.
+FMHA_DEV void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
 __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  using C = FwdCfg<D>;
+  using C = PipeCfg<D, QB>;
   constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, XROWB = C::XROWB;
-  constexpr int TILEB = C::TILEB;
+  constexpr int TILEB = C::TILEB, PANELB = C::PANELB;
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
   constexpr int CPR = D / 8;
@@ -39,6 +86,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   static_assert(BK * CPR % NT == 0, "tile must divide evenly over the workgroup");
   static_assert(NT >= BK, "the extra rows are staged by the first BK threads");
   static_assert(DROP == 0 || DROP == 1, "tensor dropout and the save pass use fmha_fwd_kernel");
+  static_assert(D % 64 == 0, "tiles are stored as panels of 64 columns");
   constexpr float NEG_INF = -__builtin_inff();
   constexpr float WINDOW = 16384.f;
 
@@ -54,94 +102,130 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   const int ql = l & 31;
   const int h = l >> 5;
 
-  int bid = blockIdx.x;
-  const int nb = gridDim.x;
-  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3); // one XCD (one L2) per run of tiles
-  const int bh = bid / a.nqt;
-  int qt = bid - bh * a.nqt;
-  if (CAUSAL) qt = a.nqt - 1 - qt;
-  const int q0w = qt * QT + w * (QB * 32);
+  // ---- persistent schedule: this workgroup handles items lb, lb + G, lb + 2G, ...
+  // Workgroups are dealt round-robin to the 8 XCDs; lb is chosen so that one XCD (one L2)
+  // works on a contiguous run of items at any time, i.e. on the query tiles of few heads.
+  const int G = gridDim.x;
+  const int nitems = a.bh * a.nqt;
+  int lb = blockIdx.x;
+  if ((G & 7) == 0) lb = (lb & 7) * (G >> 3) + (lb >> 3);
 
-  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
-  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
-  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
-  const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
-
-  // Q rows are loaded unconditionally (rows past the end repeat the last valid row and are
-  // never stored) and converted only after the first K/V tiles have been requested, so that
-  // the whole prologue costs one global round trip instead of three.
-  u32x4 qraw[QB][KS];
-  v8 qreg[QB][KS]; // filled in the prologue
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    int q = q0w + qb * 32 + ql;
-    q = q < a.sq ? q : a.sq - 1;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qraw[qb][ks] = *(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8);
-  }
-
-  // ---- key range: tiles [0, nkt), keys [0, kend); the count is padded to even with an
-  // all-masked phantom tile so that the two x / P buffers alternate with fixed roles
-  int nkt = (a.sk + BK - 1) / BK;
-  if (CAUSAL) {
-    int qmax = qt * QT + QT - 1;
-    if (qmax > a.sq - 1) qmax = a.sq - 1;
-    const int need = qmax / BK + 1;
-    if (need < nkt) nkt = need;
-  }
-  const int kend = nkt * BK < a.sk ? nkt * BK : a.sk;
-  const int nkt2 = (nkt + 1) & ~1;
+  // Everything that depends on the item.  Keys: tiles [0, nkt), keys [0, kend); the tile count
+  // is padded to even (nkt2) with an all-masked phantom tile so that the two x / P buffers and
+  // the two LDS stages alternate with fixed roles across items as well.
+  struct Item {
+    int bh, qt, nkt2, kend;
+    const T *Kb, *Vb, *mkey;
+  };
+  auto make_item = [&](int idx) {
+    Item it;
+    it.bh = idx / a.nqt;
+    it.qt = idx - it.bh * a.nqt;
+    // Causal items grow with the query tile.  A workgroup's items are G apart, which is often a
+    // multiple of the tiles per head, so the order of the tiles is reversed in every other
+    // round: long and short items then alternate within each workgroup.  (Within a round the
+    // map stays one-to-one, so every item is still visited exactly once.)
+    if (CAUSAL && ((idx / G) & 1) == 0) it.qt = a.nqt - 1 - it.qt;
+    int nkt = (a.sk + BK - 1) / BK;
+    if (CAUSAL) {
+      int qmax = it.qt * QT + QT - 1;
+      if (qmax > a.sq - 1) qmax = a.sq - 1;
+      const int need = qmax / BK + 1;
+      if (need < nkt) nkt = need;
+    }
+    it.kend = nkt * BK < a.sk ? nkt * BK : a.sk;
+    it.nkt2 = (nkt + 1) & ~1;
+    it.Kb = (const T *)a.k + (size_t)it.bh * a.sk * D;
+    it.Vb = (const T *)a.v + (size_t)it.bh * a.sk * D;
+    it.mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(it.bh / a.mask_div) * a.mask_sb : nullptr;
+    return it;
+  };
+  Item cur = make_item(lb);
+  Item nxt = make_item(lb + G < nitems ? lb + G : lb); // without a successor the streams harmlessly re-read the item
+  int bh = cur.bh, q0w = cur.qt * QT + w * (QB * 32); // of the current item
 
   // ---- staging
-  // Two register sets: a tile's global loads are issued two iterations before its data is
-  // written to LDS, so that their latency (of the order of an iteration) stays hidden.
-  struct Stage {
-    u32x4 k[CPT], v[CPT];
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
+  const uint32_t wave_dst = (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u;
+  // Copy tile `tile` of `base` (K or V of this head) into stage (tile & 1) of the LDS area at
+  // byte offset area_off.  Chunk slot c = tid + i*NT of the tile (panel c / (8*BK), row
+  // (c / 8) % BK, position c % 8) receives chunk position ^ ((row >> 1) & 7) of that panel.
+  // Rows past the end re-read the last valid row: their scores get -inf through the extra
+  // step, and finite garbage in V is multiplied by P = 0.
+  auto dma_tile = [&](const T *base, int kend, int tile, uint32_t area_off) {
+    const int k0 = tile * BK;
+    const uint32_t dst = lds_base + area_off + (uint32_t)(tile & 1) * TILEB + wave_dst;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = tid + i * NT;
+      const int panel = c / (8 * BK), row = (c / 8) % BK, pos = c % 8;
+      const int col = panel * 8 + (pos ^ ((row >> 1) & 7));
+      int kr = k0 + row;
+      kr = kr < kend ? kr : kend - 1;
+      dma_global_to_lds_b128(base + (size_t)kr * D + col * 8, dst + (uint32_t)(i * NT * 16));
+    }
+  };
+  // K tile u of the stream that runs from the current item on into the next one (u may reach
+  // past the current item's last tile; nkt2 is even, so the stage parity carries over)
+  auto dmaK = [&](int u) {
+    const bool here = u < cur.nkt2;
+    dma_tile(here ? cur.Kb : nxt.Kb, here ? cur.kend : nxt.kend, here ? u : u - cur.nkt2, 0u);
+  };
+  auto dmaV = [&](int tile) { dma_tile(cur.Vb, cur.kend, tile, 2u * TILEB); };
+
+  // Q rows of an item: lane (ql, h) of wave w owns chunks [16*ks + 8*h, +8) of row q0 + 32*qb + ql.
+  // Each wave copies its own rows into its own part of the Q buffer, exactly where its lanes
+  // read them back, so the buffer needs no synchronisation beyond the wave's own wait.
+  char *ldsQb = lds + C::LDS_BYTES;
+  auto q_row = [&](const Item &it, int qb) {
+    int q = it.qt * QT + w * (QB * 32) + qb * 32 + ql;
+    q = q < a.sq ? q : a.sq - 1; // rows past the end repeat the last valid row and are never stored
+    return (const T *)a.q + ((size_t)it.bh * a.sq + q) * D + h * 8;
+  };
+  auto dmaQ = [&](const Item &it) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const T *row = q_row(it, qb);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        dma_global_to_lds_b128(row + ks * 16, lds_base + C::LDS_BYTES + (uint32_t)((qb * KS + ks) * NT * 16) + wave_dst);
+    }
+  };
+
+  // The extra-step rows (validity and per-key mask of each key) take the register path.
+  struct XStage {
     T mraw;      // raw per-key mask element (converted when it is written to LDS, so that the
-    bool mvalid; // conversion does not wait on the loads issued with it)
+    bool mvalid; // conversion does not wait on the load)
   };
-  Stage st0, st1;
-  st0.mraw = (T)0.f; st0.mvalid = false;
-  st1.mraw = (T)0.f; st1.mvalid = false;
-  auto gloadK = [&](int tile, Stage &st) {
-    const int k0 = tile * BK;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      // Loads are unconditional (rows past the end re-read the last valid row) so that the
-      // number of loads in flight is known at compile time and the wait before the LDS write
-      // can leave the younger set outstanding.  Rows past the end need no zeroing: their scores
-      // get -inf through the extra step, and finite garbage in V is multiplied by P = 0.
-      int kr = k0 + row;
-      kr = kr < kend ? kr : kend - 1;
-      st.k[i] = *(const u32x4 *)(Kb + (size_t)kr * D + col * 8);
-    }
-    {
-      const int kr = k0 + (tid & (BK - 1));
-      st.mvalid = kr < kend;
-      if (MASK == kMaskPerKey) st.mraw = mkey[st.mvalid ? kr : kend - 1];
-    }
+  XStage xs; // extra rows of the tile after next, in flight across iterations
+  int nn_kend = cur.kend;      // key range and per-key mask of the item after next
+  const T *nn_mkey = cur.mkey;
+  auto set_after_next = [&](int idx) {
+    const Item it = make_item(idx + 2 * G < nitems ? idx + 2 * G : idx);
+    nn_kend = it.kend;
+    nn_mkey = it.mkey;
   };
-  auto gloadV = [&](int tile, Stage &st) {
-    const int k0 = tile * BK;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      int kr = k0 + row;
-      kr = kr < kend ? kr : kend - 1;
-      st.v[i] = *(const u32x4 *)(Vb + (size_t)kr * D + col * 8);
+  // u: position in the tile stream, as for dmaK; it runs up to three tiles ahead, which can
+  // reach the first tile of the item after next when the next item has only two tiles
+  auto gloadX = [&](int u, XStage &st) {
+    int tile = u, kend = cur.kend;
+    const T *mk = cur.mkey;
+    if (tile >= cur.nkt2) {
+      tile -= cur.nkt2;
+      kend = nxt.kend;
+      mk = nxt.mkey;
+      if (tile >= nxt.nkt2) {
+        tile -= nxt.nkt2;
+        kend = nn_kend;
+        mk = nn_mkey;
+      }
     }
+    const int kr = tile * BK + (tid & (BK - 1));
+    st.mvalid = kr < kend;
+    st.mraw = (T)0.f;
+    if (MASK == kMaskPerKey) st.mraw = mk[st.mvalid ? kr : kend - 1];
   };
-  auto lstoreK = [&](int tile, const Stage &st) {
-    char *kd = ldsKb + (tile & 1) * TILEB;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      *(u32x4 *)(kd + row * ROWB + col * 16) = st.k[i];
-    }
+  auto lstoreX = [&](int tile, const XStage &st) {
     if (tid < BK) {
       float mk = 0.f;
       if (MASK == kMaskPerKey) mk = fmaf((float)st.mraw, a.mask_a, a.mask_b);
@@ -164,25 +248,37 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
       dst[1] = x1;
     }
   };
-  auto lstoreV = [&](int tile, const Stage &st) {
-    char *vd = ldsVb + (tile & 1) * TILEB;
+
+  // Per-lane LDS offsets of the swizzled operand reads.
+  // K (A operand of the first product): row ql of a 32-key sub-block, logical chunk 2*ks + h of
+  // panel ks / 4, which sits at position (2*(ks%4)) ^ (h ^ ((ql >> 1) & 7)).
+  uint32_t kofs[4];
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      *(u32x4 *)(vd + row * ROWB + col * 16) = st.v[i];
-    }
+  for (int j = 0; j < 4; ++j) kofs[j] = (uint32_t)(ql * ROWB + (((2 * j) ^ (h ^ ((ql >> 1) & 7))) << 4));
+  // V (A operand of the second product, read transposed): lane l addresses row
+  // r = 4h + (l%16)/4 (+ multiples of 8) and the 8 bytes at logical byte column
+  // 64*db + 32*((l/16)%2) + 8*(l%4), i.e. chunk 4*(db%2) + lp of panel db/2.  Adding 8 to the
+  // row flips bit 2 of the swizzle, which exchanges the two 64-byte halves of the panel row.
+  uint32_t vofs;
+  {
+    const int i16 = l & 15;
+    const int row_l = 4 * h + (i16 >> 2);
+    const int lp = 2 * ((l >> 4) & 1) + ((i16 & 3) >> 1);
+    vofs = (uint32_t)(row_l * ROWB + ((lp ^ (row_l >> 1)) << 4) + 8 * (i16 & 1));
+  }
+  auto readK = [&](const char *ldsK, int sb, int ks) -> v8 {
+    return as_v8<T>(*(const u32x4 *)(ldsK + kofs[ks & 3] + sb * 32 * ROWB + (ks >> 2) * PANELB));
+  };
+  // rows row0 + 4h + 16c + {0,1,2,3, 8,9,10,11} of column block db, as lds_load_a_transposed
+  auto readV = [&](const char *ldsV, int sb, int db, int c) -> v8 {
+    const char *p0 = ldsV + vofs + (sb * 32 + 16 * c) * ROWB + (db >> 1) * PANELB;
+    const u32x2 lo = lds_read_tr16(p0 + (db & 1) * 64);
+    const u32x2 hi = lds_read_tr16(p0 + 8 * ROWB + ((db & 1) ^ 1) * 64);
+    const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
+    return as_v8<T>(both);
   };
 
-  const T *mrow[QB];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    int q = q0w + qb * 32 + ql;
-    if (q > a.sq - 1) q = a.sq - 1;
-    mrow[qb] = nullptr;
-    if (MASK == kMaskFull)
-      mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
-  }
+  const T *mrow[QB]; // this lane's rows of a full mask tensor, set when an item starts
   auto load4 = [&](const T *row, int kk, bool safe, float out[4]) {
     if (safe) {
       v4 t = as_v4<T>(*(const u32x2 *)(row + kk));
@@ -199,23 +295,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   float mref[QB], lsum[QB];
   bool seen[QB];
   v8 bx[QB];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    mref[qb] = 0.f;
-    seen[qb] = false;
-    lsum[qb] = 0.f;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[qb][db][r] = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) bx[qb][j] = (T)0.f;
-    if (h == 0) {
-      bx[qb][1] = (T)1.f;
-      bx[qb][2] = (T)1.f;
-      if (MASK == kMaskFull) bx[qb][3] = (T)a.mask_b;
-    }
-  }
+  v8 qreg[QB][KS]; // Q' = Q * scale * log2(e) as B-operand registers
 
   // x buffers (accumulators of the first product) with the reference baked into each,
   // and the rounded probabilities of the previous / current tile
@@ -239,7 +319,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
-        const v8 ka = as_v8<T>(*(const u32x4 *)(ldsK + (sb * 32 + ql) * ROWB + ks * 32 + h * 16));
+        const v8 ka = readK(ldsK, sb, ks);
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) x[qb][sb] = E::mfma(ka, qreg[qb][ks], x[qb][sb]);
       }
@@ -259,7 +339,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const v8 va = lds_load_a_transposed<T, ROWB>(ldsV, sb * 32, db * 32, c, l);
+          const v8 va = readV(ldsV, sb, db, c);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) o[qb][db] = E::mfma(va, p[qb][sb][c], o[qb][db]);
         }
@@ -290,7 +370,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
         const int sb = i / 2, c = i % 2;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const v8 va = lds_load_a_transposed<T, ROWB>(ldsV, sb * 32, db * 32, c, l);
+          const v8 va = readV(ldsV, sb, db, c);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) o[qb][db] = E::mfma(va, p[qb][sb][c], o[qb][db]);
         }
@@ -299,7 +379,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb) {
           if (i < KS) {
-            const v8 ka = as_v8<T>(*(const u32x4 *)(ldsK + (sb * 32 + ql) * ROWB + i * 32 + h * 16));
+            const v8 ka = readK(ldsK, sb, i);
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) x[qb][sb] = E::mfma(ka, qreg[qb][i], x[qb][sb]);
           } else {
@@ -426,17 +506,20 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   // One iteration.  FIRST: tile t is the first tile (no previous second product; the
   // reference is set from this tile before the next first product bakes it).
   // LAST: there is no next tile.
-  // stl: register set to load into (K(t+3), V(t+1)); sts: set loaded one iteration ago,
-  // written to LDS at the end (K(t+2), V(t)).
+  // K(t+2) and V(t) are requested at the top and awaited by tile_sync() after the body; past
+  // the item's last tile, "K(t+2)" is one of the first two tiles of the next item.
+  // The extra rows of tile t+2 are written first, from the registers `xs` that the previous
+  // iteration loaded (so the load has certainly landed: tile_sync() waited for it), and `xs`
+  // is refilled for tile t+3 -- all before the copies are issued, because the compiler's own
+  // wait for a load it knows about also waits for every copy issued ahead of it.
   auto body = [&](int t, auto first_tag, auto last_tag, auto guarded_tag, f32x16 (&xc)[QB][NSB], float (&bkc)[QB],
-                  f32x16 (&xn)[QB][NSB], float (&bkn)[QB], const v8 (&pprev)[QB][NSB][2], v8 (&pcur)[QB][NSB][2],
-                  Stage &stl, const Stage &sts) {
+                  f32x16 (&xn)[QB][NSB], float (&bkn)[QB], const v8 (&pprev)[QB][NSB][2], v8 (&pcur)[QB][NSB][2]) {
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr bool LAST = decltype(last_tag)::value;
-    if (!LAST) {
-      gloadK(t + 3, stl);
-      gloadV(t + 1, stl);
-    }
+    lstoreX(t + 2, xs);
+    gloadX(t + 3, xs);
+    dmaK(t + 2);
+    dmaV(t);
     adjust(t, xc, guarded_tag);
     if (FIRST) {
       float shift[QB];
@@ -487,78 +570,142 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
         dropout(t, qb, pcur[qb]);
       }
     }
-    if (!LAST) lstoreK(t + 2, sts);
-    lstoreV(t, sts);
   };
-
-  // ---- prologue: K(0), K(1) into LDS, first product of tile 0
-  gloadK(0, st0);
-  gloadK(1, st1);
-  gloadV(0, st1);
-  // Q' = Q * scale * log2(e) as B-operand registers
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const v8 raw = as_v8<T>(qraw[qb][ks]);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
-    }
-  lstoreK(0, st0);
-  lstoreK(1, st1);
-  gloadK(2, st1); // K(2) joins V(0) in the set that the first iteration writes to LDS
-  __syncthreads();
-  g1(0, xA, bkA);
-  __syncthreads(); // tile 0's K stage is refilled during the first iteration
+  auto tile_sync = [&]() {
+    dma_wait_all();
+    __syncthreads();
+  };
 
   using Yes = std::true_type;
   using No = std::false_type;
   // A tile crosses the causal diagonal of this wave iff its last key exceeds the wave's first query.
   auto diag = [&](int t) { return CAUSAL && (t * BK + BK - 1 > q0w); };
 
-  // t = 0
-  if (diag(0)) body(0, Yes{}, No{}, Yes{}, xA, bkA, xB, bkB, pB, pA, st0, st1);
-  else body(0, Yes{}, No{}, No{}, xA, bkA, xB, bkB, pB, pA, st0, st1);
-  __syncthreads();
-  // steady state, two tiles per trip so that the buffers keep fixed roles
-  for (int t = 1; t < nkt2 - 1; t += 2) {
-    if (diag(t)) body(t, No{}, No{}, Yes{}, xB, bkB, xA, bkA, pA, pB, st1, st0);
-    else body(t, No{}, No{}, No{}, xB, bkB, xA, bkA, pA, pB, st1, st0);
-    __syncthreads();
-    if (diag(t + 1)) body(t + 1, No{}, No{}, Yes{}, xA, bkA, xB, bkB, pB, pA, st0, st1);
-    else body(t + 1, No{}, No{}, No{}, xA, bkA, xB, bkB, pB, pA, st0, st1);
-    __syncthreads();
-  }
-  // last tile (odd index) and the second product that is still owed
+  // ---- workgroup prologue: the first item's Q, K(0), K(1) and extra rows
+  set_after_next(lb);
+  if (C::QLDS) dmaQ(cur);
+  dmaK(0);
+  dmaK(1);
   {
-    const int t = nkt2 - 1;
-    if (diag(t)) body(t, No{}, Yes{}, Yes{}, xB, bkB, xA, bkA, pA, pB, st1, st0);
-    else body(t, No{}, Yes{}, No{}, xB, bkB, xA, bkA, pA, pB, st1, st0);
-    __syncthreads();
-    g2(t, pB);
+    XStage x0, x1;
+    gloadX(0, x0);
+    gloadX(1, x1);
+    gloadX(2, xs);
+    lstoreX(0, x0);
+    lstoreX(1, x1);
   }
 
-  // ---- epilogue
-  T *Ob = (T *)a.o + (size_t)bh * a.sq * D;
+  for (int idx = lb;;) {
+    const int nidx = idx + G;
+    const bool more = nidx < nitems;
+    nxt = make_item(more ? nidx : idx);
+    set_after_next(idx);
+    bh = cur.bh;
+    q0w = cur.qt * QT + w * (QB * 32);
+
+    // ---- item prologue: Q' registers, state, first product of tile 0
+    // Only the first item has copies in flight here (Q, K(0), K(1)) and extra rows that other
+    // waves have not seen yet.  For later items all of that was awaited inside the previous
+    // item, and waiting again would only stall on the output stores just issued.
+    if (idx == lb) tile_sync();
+    if (C::QLDS) {
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    const int q = q0w + qb * 32 + ql;
-    const float lt = xhalf_sum(lsum[qb]);
-    const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
-    if (q < a.sq) {
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const v8 raw = as_v8<T>(*(const u32x4 *)(ldsQb + ((qb * KS + ks) * NT + tid) * 16));
+#pragma unroll
+          for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
+        }
+    } else {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        const T *row = q_row(cur, qb);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const v8 raw = as_v8<T>(*(const u32x4 *)(row + ks * 16));
+#pragma unroll
+          for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
+        }
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      mref[qb] = 0.f;
+      seen[qb] = false;
+      lsum[qb] = 0.f;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          v4 t;
+        for (int r = 0; r < 16; ++r) o[qb][db][r] = 0.f;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) t[i] = (T)(o[qb][db][4 * g + i] * inv);
-          *(v4 *)(Ob + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
-        }
-      const float cfix = (MASK == kMaskFull) ? a.mask_b - (float)(T)a.mask_b : 0.f;
-      if (a.lse && h == 0)
-        a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + cfix + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
+      for (int j = 0; j < 8; ++j) bx[qb][j] = (T)0.f;
+      if (h == 0) {
+        bx[qb][1] = (T)1.f;
+        bx[qb][2] = (T)1.f;
+        if (MASK == kMaskFull) bx[qb][3] = (T)a.mask_b;
+      }
+      int q = q0w + qb * 32 + ql;
+      if (q > a.sq - 1) q = a.sq - 1;
+      mrow[qb] = nullptr;
+      if (MASK == kMaskFull)
+        mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
     }
+    g1(0, xA, bkA);
+    __syncthreads(); // tile 0's K stage is refilled during the first iteration
+    // The next item's Q rows are requested here rather than earlier so that the wait they end
+    // up in is the one at the end of the first iteration.  The Q buffer has been read (the
+    // first product used the registers made from it).
+    if (C::QLDS && more) dmaQ(nxt);
+
+    const int nkt2 = cur.nkt2;
+    // t = 0
+    if (diag(0)) body(0, Yes{}, No{}, Yes{}, xA, bkA, xB, bkB, pB, pA);
+    else body(0, Yes{}, No{}, No{}, xA, bkA, xB, bkB, pB, pA);
+    tile_sync();
+    // steady state, two tiles per trip so that the buffers keep fixed roles
+    for (int t = 1; t < nkt2 - 1; t += 2) {
+      if (diag(t)) body(t, No{}, No{}, Yes{}, xB, bkB, xA, bkA, pA, pB);
+      else body(t, No{}, No{}, No{}, xB, bkB, xA, bkA, pA, pB);
+      tile_sync();
+      if (diag(t + 1)) body(t + 1, No{}, No{}, Yes{}, xA, bkA, xB, bkB, pB, pA);
+      else body(t + 1, No{}, No{}, No{}, xA, bkA, xB, bkB, pB, pA);
+      tile_sync();
+    }
+    // last tile (odd index) and the second product that is still owed
+    {
+      const int t = nkt2 - 1;
+      if (diag(t)) body(t, No{}, Yes{}, Yes{}, xB, bkB, xA, bkA, pA, pB);
+      else body(t, No{}, Yes{}, No{}, xB, bkB, xA, bkA, pA, pB);
+      tile_sync();
+      g2(t, pB);
+    }
+
+    // ---- item epilogue
+    T *Ob = (T *)a.o + (size_t)bh * a.sq * D;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const int q = q0w + qb * 32 + ql;
+      const float lt = xhalf_sum(lsum[qb]);
+      const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
+      if (q < a.sq) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            v4 t;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[i] = (T)(o[qb][db][4 * g + i] * inv);
+            *(v4 *)(Ob + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
+          }
+        const float cfix = (MASK == kMaskFull) ? a.mask_b - (float)(T)a.mask_b : 0.f;
+        if (a.lse && h == 0)
+          a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + cfix + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
+      }
+    }
+    if (!more) break;
+    idx = nidx;
+    cur = nxt;
   }
 }
 
