@@ -156,8 +156,10 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
         n = 0;
       return n;
     }();
-    const long long items2 = (long long)p->bh * ((p->sq + 255) / 256);
-    if (cus > 0 && items2 >= 4LL * cus) v.qb = 2;
+    const int tiles2 = (p->sq + 255) / 256;
+    const long long items2 = (long long)p->bh * tiles2;
+    const bool little_padding = tiles2 * 256 - p->sq <= p->sq / 8;
+    if (cus > 0 && items2 >= 4LL * cus && little_padding) v.qb = 2;
   }
   const int force = env_int("FMHA_FWD_QB", 0); // tuning override: 1 or 2
   if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;

@@ -20,6 +20,10 @@ TOL = {"fp16": 2e-3, "bf16": 2e-2}
 # weights of the second product sum to one exactly); the saved LSE carries that rounding: up to
 # 2^-11 relative (fp16) / 2^-9 (bf16) on rows with a handful of visible keys.
 LSE_TOL = {"fp16": 1e-3, "bf16": 5e-3}
+# Q is pre-multiplied by scale * log2(e) and rounded ONCE to the element type before the first
+# product, so every score carries that rounding (2^-11 / 2^-8 relative).  A row with one or two
+# visible keys shows it in full in its LSE, hence the term proportional to |LSE| where such rows occur.
+LSE_REL = {"fp16": 2.0 ** -11, "bf16": 2.0 ** -8}
 TDT = {"fp16": torch.float16, "bf16": torch.bfloat16}
 
 
@@ -70,6 +74,37 @@ def test_forward_matches_oracle(bh, sq, sk, d, dtype, mask, causal, qb, monkeypa
                            want=("o", "lse"))
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= TOL[dtype]
     assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= LSE_TOL[dtype]
+
+
+# The forward kernel is persistent: the grid is capped at the number of workgroups the device
+# keeps resident (two per CU: 512 on a 256-CU part) and each workgroup walks several (head,
+# query tile) items, prefetching the next item's Q rows and first K tiles while it works.
+# These shapes have more items than any such grid, few key tiles per item (so the prefetch
+# stream crosses item boundaries every other tile, and with two tiles per item reaches the
+# item after next), and masks that differ from head to head.
+MANY_ITEMS = [
+    # bh, sq, sk, d, dtype, mask, causal, qb
+    (600, 128, 128, 64, "fp16", "pad", False, 1),    # 600 items of two key tiles
+    (600, 128, 100, 64, "fp16", "pad", False, 1),    # ... of one key tile and a phantom tile
+    (560, 192, 192, 64, "fp16", "pad", True, 1),     # causal: 1120 items of unequal length
+    (520, 128, 200, 128, "bf16", None, False, 1),    # head dim 128: Q comes from global memory per item
+    (1040, 256, 64, 64, "fp16", "pad", False, 2),    # two query blocks per wave: 32-key tiles, 1040 items
+    (1040, 256, 200, 64, "fp16", None, False, 2),
+]
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,mask,causal,qb", MANY_ITEMS)
+def test_forward_many_items_per_workgroup(bh, sq, sk, d, dtype, mask, causal, qb, monkeypatch):
+    monkeypatch.setenv("FMHA_FWD_QB", str(qb))
+    q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype)
+    m = None
+    if mask == "pad":
+        m = pad_mask(bh // 2, sk, 1, sk).to(TDT[dtype])  # one row per pair of heads, valid lengths in [1, sk]
+    o, lse, _, _ = _run(q, k, v, mask=None if m is None else m.cuda(), causal=causal, want_lse=True)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=None if m is None else f32(m), causal=causal,
+                           want=("o", "lse"))
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= TOL[dtype]
+    assert (np.abs(lse.cpu().numpy() - ref["lse"]) <= LSE_TOL[dtype] + LSE_REL[dtype] * np.abs(ref["lse"])).all()
 
 
 @pytest.mark.parametrize("bh,sq,sk,d,causal", [(3, 128, 192, 64, False), (2, 257, 257, 64, True),
