@@ -55,8 +55,7 @@ template <int D> struct BwdCfg {
   static constexpr int NSB = BT / 32;
   static constexpr int KS = D / 16;
   static constexpr int DB = D / 32;
-  static constexpr int ROWB = D * 2 + 16;
-  static constexpr int TILEB = BT * ROWB;
+  static constexpr int TILEB = BT * D * 2; // swizzled panel layout of fmha_common.h, no padding
   static constexpr int XROWB = 32;        // extra-step rows: 16 elements
   // two tiles x 2 stages + two sets of extra rows x 2 stages + {delta} x 2 stages
   static constexpr int LDS_BYTES = 4 * TILEB + 2 * 2 * BT * XROWB + 2 * BT * 4;
@@ -78,12 +77,10 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = BwdCfg<D>;
-  constexpr int BK = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, TILEB = C::TILEB;
+  constexpr int BK = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, TILEB = C::TILEB;
   constexpr int XROWB = C::XROWB;
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
-  constexpr int CPR = D / 8;
-  constexpr int CPT = BK * CPR / NT;
   constexpr float NEG_INF = -__builtin_inff();
   constexpr float BIGNEG = -60000.f;
 
@@ -174,35 +171,27 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
   }
   const int kend = nkt * BK < a.sk ? nkt * BK : a.sk;
 
-  // ---- staging (unconditional loads: rows past the end re-read the last valid row; their
-  // scores are pushed to -60000 by the extra step, so P = dS = 0 for them)
-  u32x4 kst[CPT], vst[CPT];
+  // ---- staging.  K and V tiles are copied from global memory straight into LDS (rows past the
+  // end re-read the last valid row; their scores are pushed to -60000 by the extra step, so
+  // P = dS = 0 for them).  The extra rows take the register path, one tile further ahead, so
+  // that their load has long landed when it is used: the compiler's wait for a load it knows
+  // about also waits for every copy issued before it.
+  const uint32_t lds_base = lds_address(lds);
+  PanelLane pl;
+  pl.init(l);
+  auto dma_kv = [&](int kt) {
+    const uint32_t dst = lds_base + (uint32_t)(kt & 1) * 2 * TILEB;
+    dma_tile_rows<T, D, BK, NT>(Kb, kt * BK, kend, dst, tid);
+    dma_tile_rows<T, D, BK, NT>(Vb, kt * BK, kend, dst + TILEB, tid);
+  };
   T mraw = (T)0.f;
   bool mvalid = false;
-  auto gload = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      int kr = k0 + row;
-      kr = kr < kend ? kr : kend - 1;
-      kst[i] = *(const u32x4 *)(Kb + (size_t)kr * D + col * 8);
-      vst[i] = *(const u32x4 *)(Vb + (size_t)kr * D + col * 8);
-    }
-    const int kr = k0 + (tid & (BK - 1));
+  auto gloadX = [&](int kt) {
+    const int kr = kt * BK + (tid & (BK - 1));
     mvalid = kr < kend;
     if (MASK == kMaskPerKey) mraw = mkey[mvalid ? kr : kend - 1];
   };
-  auto lstore = [&](int stage) {
-    char *kd = lds + stage * 2 * TILEB;
-    char *vd = kd + TILEB;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      *(u32x4 *)(kd + row * ROWB + col * 16) = kst[i];
-      *(u32x4 *)(vd + row * ROWB + col * 16) = vst[i];
-    }
+  auto lstoreX = [&](int stage) {
     if (tid < BK) {
       float mk = 0.f;
       if (MASK == kMaskPerKey) mk = fmaf((float)mraw, a.mask_a, a.mask_b);
@@ -255,14 +244,21 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) dq[qb][db][r] = 0.f;
 
-  gload(0);
-  lstore(0);
+  dma_kv(0);
+  gloadX(0);
+  lstoreX(0);
+  gloadX(1);
+  dma_wait_all();
   __syncthreads();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int cur = kt & 1;
     const int k0 = kt * BK;
-    if (kt + 1 < nkt) gload(k0 + BK);
+    if (kt + 1 < nkt) {
+      lstoreX(cur ^ 1); // rows of tile kt+1, loaded one iteration ago
+      gloadX(kt + 2);
+      dma_kv(kt + 1);
+    }
     const char *ldsK = lds + cur * 2 * TILEB;
     const char *ldsV = ldsK + TILEB;
     const char *ldsX = ldsXb + cur * BK * XROWB;
@@ -283,9 +279,8 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
         if (ks < KS) {
-          const int off = (sb * 32 + ql) * ROWB + ks * 32 + h * 16;
-          const v8 ka = as_v8<T>(*(const u32x4 *)(ldsK + off));
-          const v8 va = as_v8<T>(*(const u32x4 *)(ldsV + off));
+          const v8 ka = panel_read_rows<T, BK>(ldsK, pl, sb, ks);
+          const v8 va = panel_read_rows<T, BK>(ldsV, pl, sb, ks);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) {
             x[qb][sb] = E::mfma(ka, qreg[qb][ks], x[qb][sb]);
@@ -342,12 +337,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const v8 kt_a = lds_load_a_transposed<T, ROWB>(ldsK, sb * 32, db * 32, c, l);
+          const v8 kt_a = panel_read_transposed<T, BK>(ldsK, pl, sb, db, c);
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb) dq[qb][db] = E::mfma(kt_a, dsfrag[qb][sb][c], dq[qb][db]);
         }
 
-    if (kt + 1 < nkt) lstore(cur ^ 1);
+    dma_wait_all();
     __syncthreads();
   }
 
@@ -376,12 +371,10 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = BwdCfg<D>;
-  constexpr int BQ = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, TILEB = C::TILEB;
+  constexpr int BQ = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, TILEB = C::TILEB;
   constexpr int XROWB = C::XROWB;
   constexpr int NT = NW * 64;
   constexpr int KT = NW * KB * 32;
-  constexpr int CPR = D / 8;
-  constexpr int CPT = BQ * CPR / NT;
   constexpr float NEG_INF = -__builtin_inff();
   constexpr float BIGNEG = -60000.f;
   static_assert(NT >= BQ, "row statistics are staged by the first BQ threads");
@@ -457,35 +450,27 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
   const int nqt = (a.sq + BQ - 1) / BQ;
   const int qt0 = CAUSAL ? (ktile * KT) / BQ : 0; // first query tile that sees any of these keys
 
-  u32x4 qst[CPT], dst[CPT];
+  // ---- staging: Q and dO tiles copied straight into LDS (rows past the end repeat the last
+  // valid row); the per-query extra rows take the register path one tile further ahead, as in
+  // the dQ kernel.
+  const uint32_t lds_base = lds_address(lds);
+  PanelLane pl;
+  pl.init(l);
+  auto dma_qdo = [&](int qt) {
+    const uint32_t dst = lds_base + (uint32_t)(qt & 1) * 2 * TILEB;
+    dma_tile_rows<T, D, BQ, NT>(Qb, qt * BQ, a.sq, dst, tid);
+    dma_tile_rows<T, D, BQ, NT>(dOb, qt * BQ, a.sq, dst + TILEB, tid);
+  };
   float lraw = 0.f, draw = 0.f;
   bool qvalid = false;
-  auto gload = [&](int q0) {
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      int qr = q0 + row;
-      qr = qr < a.sq ? qr : a.sq - 1;
-      qst[i] = *(const u32x4 *)(Qb + (size_t)qr * D + col * 8);
-      dst[i] = *(const u32x4 *)(dOb + (size_t)qr * D + col * 8);
-    }
-    int qr = q0 + (tid & (BQ - 1));
+  auto gloadX = [&](int qt) {
+    int qr = qt * BQ + (tid & (BQ - 1));
     qvalid = qr < a.sq;
     qr = qvalid ? qr : a.sq - 1;
     lraw = lseb[qr];
     draw = delb[qr];
   };
-  auto lstore = [&](int stage) {
-    char *qd = lds + stage * 2 * TILEB;
-    char *dd = qd + TILEB;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int row = c / CPR, col = c % CPR;
-      *(u32x4 *)(qd + row * ROWB + col * 16) = qst[i];
-      *(u32x4 *)(dd + row * ROWB + col * 16) = dst[i];
-    }
+  auto lstoreX = [&](int stage) {
     if (tid < BQ) {
       // rows past the end (whose Q/dO rows repeat the last valid row) and fully masked rows: P = 0
       float nl = BIGNEG, dl = 0.f;
@@ -533,15 +518,22 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
       }
 
   if (qt0 < nqt) {
-    gload(qt0 * BQ);
-    lstore(qt0 & 1);
+    dma_qdo(qt0);
+    gloadX(qt0);
+    lstoreX(qt0 & 1);
+    gloadX(qt0 + 1); // row indices are clamped, so looking past the last tile is harmless
   }
+  dma_wait_all();
   __syncthreads();
 
   for (int qt = qt0; qt < nqt; ++qt) {
     const int cur = qt & 1;
     const int q0 = qt * BQ;
-    if (qt + 1 < nqt) gload(q0 + BQ);
+    if (qt + 1 < nqt) {
+      lstoreX(cur ^ 1); // rows of tile qt+1, loaded one iteration ago
+      gloadX(qt + 2);
+      dma_qdo(qt + 1);
+    }
     const char *ldsQ = lds + cur * 2 * TILEB;
     const char *ldsDO = ldsQ + TILEB;
     const char *ldsXs = ldsXb + (cur * 2 + 0) * BQ * XROWB;
@@ -564,9 +556,8 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
         if (ks < KS) {
-          const int off = (sb * 32 + kl) * ROWB + ks * 32 + h * 16;
-          const v8 qa = as_v8<T>(*(const u32x4 *)(ldsQ + off));
-          const v8 da = as_v8<T>(*(const u32x4 *)(ldsDO + off));
+          const v8 qa = panel_read_rows<T, BQ>(ldsQ, pl, sb, ks);
+          const v8 da = panel_read_rows<T, BQ>(ldsDO, pl, sb, ks);
 #pragma unroll
           for (int kb = 0; kb < KB; ++kb) {
             x[kb][sb] = E::mfma(qa, kreg[kb][ks], x[kb][sb]);
@@ -638,8 +629,8 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
       for (int c = 0; c < 2; ++c)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const v8 dot = lds_load_a_transposed<T, ROWB>(ldsDO, sb * 32, db * 32, c, l);
-          const v8 qtr = lds_load_a_transposed<T, ROWB>(ldsQ, sb * 32, db * 32, c, l);
+          const v8 dot = panel_read_transposed<T, BQ>(ldsDO, pl, sb, db, c);
+          const v8 qtr = panel_read_transposed<T, BQ>(ldsQ, pl, sb, db, c);
 #pragma unroll
           for (int kb = 0; kb < KB; ++kb) {
             dv[kb][db] = E::mfma(dot, pfrag[kb][sb][c], dv[kb][db]);
@@ -647,7 +638,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
           }
         }
 
-    if (qt + 1 < nqt) lstore(cur ^ 1);
+    dma_wait_all();
     __syncthreads();
   }
 

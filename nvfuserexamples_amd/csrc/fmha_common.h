@@ -99,6 +99,89 @@ FMHA_DEV typename Elem<T>::v8 lds_load_a_transposed(const char *tile, int row0, 
   return as_v8<T>(both);
 }
 
+// ---------------------------------------------------------------- swizzled LDS tiles
+// Operand tiles that are copied from global memory straight into LDS
+// (global_load_lds_dwordx4: every lane names a 16-byte global chunk and the wave's 64
+// chunks land in 1 KiB of consecutive LDS) cannot pad their rows.  They are kept as D/64
+// panels of 64 columns, each panel [row][8 chunks of 16 bytes] with a 128-byte pitch, and
+// chunk c of row r sits at position c ^ ((r >> 1) & 7): sixteen consecutive rows then spread
+// one logical chunk over all sixteen 16-byte bank groups, which is what a conflict-free
+// ds_read_b128 needs.  The copying lane simply fetches the chunk that belongs at its slot.
+constexpr int kPanelRowB = 128;
+
+// One wave-wide 16-byte-per-lane copy from global memory into LDS: lane i's chunk lands at
+// LDS byte address lds_wave_base + 16*i.  Written as inline assembly with hand-placed waits
+// (dma_wait_all) because the compiler, which cannot tell which LDS reads a copy may alias,
+// would otherwise wait for all copies before any later LDS read.
+FMHA_DEV void dma_global_to_lds_b128(const void *gptr, uint32_t lds_wave_base) {
+  // the readfirstlane is free when the compiler already knows the value to be uniform
+  lds_wave_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr)
+               : "memory");
+}
+// Wait until every copy issued with dma_global_to_lds_b128 by this wave has landed (this
+// also waits for the wave's other outstanding vector loads and stores).
+FMHA_DEV void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// LDS byte address of a __shared__ object.
+FMHA_DEV uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
+}
+
+// Copies rows [row0, row0 + BT) of a row-major [rows][D] matrix into a swizzled tile whose
+// LDS byte address is lds_tile; NT threads take part, tid is the caller's index among them.
+// Rows >= rend re-read row rend - 1 (callers neutralise them through their extra-step rows).
+template <typename T, int D, int BT, int NT>
+FMHA_DEV void dma_tile_rows(const T *base, int row0, int rend, uint32_t lds_tile, int tid) {
+  constexpr int CHUNKS = BT * D / 8;
+  static_assert(D % 64 == 0 && CHUNKS % NT == 0, "tile must divide evenly over the workgroup");
+  const uint32_t wave_dst = lds_tile + (uint32_t)(tid >> 6) * 1024u;
+#pragma unroll
+  for (int i = 0; i < CHUNKS / NT; ++i) {
+    const int c = tid + i * NT; // chunk slot: panel c / (8*BT), row (c / 8) % BT, position c % 8
+    const int panel = c / (8 * BT), row = (c / 8) % BT, pos = c % 8;
+    const int col = panel * 8 + (pos ^ ((row >> 1) & 7));
+    int r = row0 + row;
+    r = r < rend ? r : rend - 1;
+    dma_global_to_lds_b128(base + (size_t)r * D + col * 8, wave_dst + (uint32_t)(i * NT * 16));
+  }
+}
+
+// Per-lane offsets of the two kinds of operand read from a swizzled tile.
+struct PanelLane {
+  uint32_t rowofs[4]; // row (l % 32) of a 32-row block, logical chunk pair j: chunks 2j + l/32
+  uint32_t trofs;     // transposed read, see panel_read_transposed
+  FMHA_DEV void init(int l) {
+    const int ql = l & 31, h = l >> 5;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rowofs[j] = (uint32_t)(ql * kPanelRowB + (((2 * j) ^ (h ^ ((ql >> 1) & 7))) << 4));
+    const int i16 = l & 15;
+    const int row_l = 4 * h + (i16 >> 2);
+    const int lp = 2 * ((l >> 4) & 1) + ((i16 & 3) >> 1);
+    trofs = (uint32_t)(row_l * kPanelRowB + ((lp ^ (row_l >> 1)) << 4) + 8 * (i16 & 1));
+  }
+};
+
+// A operand whose rows are tile rows: row 32*sb + l%32, contraction indices 16*ks + 8*(l/32) .. +7.
+template <typename T, int BT>
+FMHA_DEV typename Elem<T>::v8 panel_read_rows(const char *tile, const PanelLane &pl, int sb, int ks) {
+  return as_v8<T>(*(const u32x4 *)(tile + pl.rowofs[ks & 3] + sb * 32 * kPanelRowB + (ks >> 2) * (BT * kPanelRowB)));
+}
+
+// A operand of a product that consumes the tile transposed (contraction over tile rows), with the
+// row order of lds_load_a_transposed: rows 32*sb + 4h + 16c + {0,1,2,3, 8,9,10,11}, column 32*db + l%32.
+// Lane l addresses row 4h + (l%16)/4 (+ multiples of 8) and the 8 bytes at logical byte column
+// 64*db + 32*((l/16)%2) + 8*(l%4); adding 8 to the row flips bit 2 of the swizzle, which exchanges
+// the two 64-byte halves of the panel row.
+template <typename T, int BT>
+FMHA_DEV typename Elem<T>::v8 panel_read_transposed(const char *tile, const PanelLane &pl, int sb, int db, int c) {
+  const char *p0 = tile + pl.trofs + (sb * 32 + 16 * c) * kPanelRowB + (db >> 1) * (BT * kPanelRowB);
+  const u32x2 lo = lds_read_tr16(p0 + (db & 1) * 64);
+  const u32x2 hi = lds_read_tr16(p0 + 8 * kPanelRowB + ((db & 1) ^ 1) * 64);
+  const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
+  return as_v8<T>(both);
+}
+
 // Exchange between lane l and lane l^32 (v_permlane32_swap), reduced with max / add.
 FMHA_DEV float xhalf_max(float x) {
   int v = __float_as_int(x);

@@ -17,14 +17,8 @@
 // K and V tiles go from global memory straight into LDS (global_load_lds_dwordx4: every
 // lane names a 16-byte global chunk and the wave's 64 chunks land in 1 KiB of consecutive
 // LDS), issued at the top of an iteration and awaited at its end, so no registers and no
-// VALU/LDS-write issue slots are spent on staging.  Consecutive placement rules out row
-// padding, so a tile is kept as D/64 panels of 64 columns, each panel [key][8 chunks of 16
-// bytes] with a 128-byte pitch, and chunk c of row r sits at position c ^ ((r >> 1) & 7):
-// sixteen consecutive rows then spread one logical chunk over all sixteen 16-byte bank
-// groups, which is what a conflict-free ds_read_b128 needs.  The lane simply fetches the
-// chunk that belongs at its position.  The loads are written as inline assembly with
-// hand-placed s_waitcnt: the compiler would otherwise wait for all of them before any
-// later LDS read.
+// VALU/LDS-write issue slots are spent on staging; the tiles use the swizzled panel layout
+// of fmha_common.h.
 //
 // Workgroups are persistent: the grid holds as many workgroups as the chip keeps resident
 // and each walks a strided list of (head, query tile) items.  The K and extra-row streams
@@ -49,9 +43,7 @@ template <int D, int QB> struct PipeCfg {
   static constexpr int NSB = BK / 32; // 32-key sub-blocks per tile
   static constexpr int KS = D / 16;   // contraction steps of K.Q^T
   static constexpr int DB = D / 32;   // 32-row blocks of O^T
-  static constexpr int ROWB = 128;    // LDS row pitch in bytes of one 64-column panel (unpadded, swizzled)
-  static constexpr int PANELB = BK * ROWB;
-  static constexpr int TILEB = (D / 64) * PANELB;
+  static constexpr int TILEB = BK * D * 2; // swizzled panel layout, no padding
   static constexpr int XROWB = 32;    // pitch of the extra-contraction-step rows (16 elements)
   // The next item's Q rows are prefetched into LDS where that still leaves room for two
   // workgroups per CU; otherwise Q is loaded from global memory when the item starts.
@@ -60,30 +52,16 @@ template <int D, int QB> struct PipeCfg {
   static constexpr int lds_bytes(int nw) { return LDS_BYTES + (QLDS ? nw * QB * 32 * D * 2 : 0); }
 };
 
-// One wave-wide 16-byte-per-lane copy from global memory into LDS: lane i's chunk lands at
-// LDS byte address lds_wave_base + 16*i.  lds_wave_base must be wave-uniform.
-FMHA_DEV void dma_global_to_lds_b128(const void *gptr, uint32_t lds_wave_base) {
-  // the readfirstlane is free when the compiler already knows the value to be uniform
-  lds_wave_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_wave_base);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(gptr)
-               : "memory");
-}
-// Wait until every copy issued with dma_global_to_lds_b128 by this wave has landed.
-FMHA_DEV void dma_wait_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
 __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = PipeCfg<D, QB>;
-  constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, XROWB = C::XROWB;
-  constexpr int TILEB = C::TILEB, PANELB = C::PANELB;
+  constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, XROWB = C::XROWB;
+  constexpr int TILEB = C::TILEB;
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
-  constexpr int CPR = D / 8;
-  constexpr int CPT = BK * CPR / NT;
-  static_assert(BK * CPR % NT == 0, "tile must divide evenly over the workgroup");
   static_assert(NT >= BK, "the extra rows are staged by the first BK threads");
   static_assert(DROP == 0 || DROP == 1, "tensor dropout and the save pass use fmha_fwd_kernel");
   static_assert(D % 64 == 0, "tiles are stored as panels of 64 columns");
@@ -145,25 +123,13 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
   int bh = cur.bh, q0w = cur.qt * QT + w * (QB * 32); // of the current item
 
   // ---- staging
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;
+  const uint32_t lds_base = lds_address(lds);
   const uint32_t wave_dst = (uint32_t)__builtin_amdgcn_readfirstlane(w) * 1024u;
-  // Copy tile `tile` of `base` (K or V of this head) into stage (tile & 1) of the LDS area at
-  // byte offset area_off.  Chunk slot c = tid + i*NT of the tile (panel c / (8*BK), row
-  // (c / 8) % BK, position c % 8) receives chunk position ^ ((row >> 1) & 7) of that panel.
-  // Rows past the end re-read the last valid row: their scores get -inf through the extra
-  // step, and finite garbage in V is multiplied by P = 0.
+  // Copy tile `tile` of `base` (K or V of a head) into stage (tile & 1) of the LDS area at byte
+  // offset area_off.  Rows past kend re-read the last valid row: their scores get -inf through
+  // the extra step, and finite garbage in V is multiplied by P = 0.
   auto dma_tile = [&](const T *base, int kend, int tile, uint32_t area_off) {
-    const int k0 = tile * BK;
-    const uint32_t dst = lds_base + area_off + (uint32_t)(tile & 1) * TILEB + wave_dst;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = tid + i * NT;
-      const int panel = c / (8 * BK), row = (c / 8) % BK, pos = c % 8;
-      const int col = panel * 8 + (pos ^ ((row >> 1) & 7));
-      int kr = k0 + row;
-      kr = kr < kend ? kr : kend - 1;
-      dma_global_to_lds_b128(base + (size_t)kr * D + col * 8, dst + (uint32_t)(i * NT * 16));
-    }
+    dma_tile_rows<T, D, BK, NT>(base, tile * BK, kend, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
   };
   // K tile u of the stream that runs from the current item on into the next one (u may reach
   // past the current item's last tile; nkt2 is even, so the stage parity carries over)
@@ -249,33 +215,11 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
     }
   };
 
-  // Per-lane LDS offsets of the swizzled operand reads.
-  // K (A operand of the first product): row ql of a 32-key sub-block, logical chunk 2*ks + h of
-  // panel ks / 4, which sits at position (2*(ks%4)) ^ (h ^ ((ql >> 1) & 7)).
-  uint32_t kofs[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) kofs[j] = (uint32_t)(ql * ROWB + (((2 * j) ^ (h ^ ((ql >> 1) & 7))) << 4));
-  // V (A operand of the second product, read transposed): lane l addresses row
-  // r = 4h + (l%16)/4 (+ multiples of 8) and the 8 bytes at logical byte column
-  // 64*db + 32*((l/16)%2) + 8*(l%4), i.e. chunk 4*(db%2) + lp of panel db/2.  Adding 8 to the
-  // row flips bit 2 of the swizzle, which exchanges the two 64-byte halves of the panel row.
-  uint32_t vofs;
-  {
-    const int i16 = l & 15;
-    const int row_l = 4 * h + (i16 >> 2);
-    const int lp = 2 * ((l >> 4) & 1) + ((i16 & 3) >> 1);
-    vofs = (uint32_t)(row_l * ROWB + ((lp ^ (row_l >> 1)) << 4) + 8 * (i16 & 1));
-  }
-  auto readK = [&](const char *ldsK, int sb, int ks) -> v8 {
-    return as_v8<T>(*(const u32x4 *)(ldsK + kofs[ks & 3] + sb * 32 * ROWB + (ks >> 2) * PANELB));
-  };
-  // rows row0 + 4h + 16c + {0,1,2,3, 8,9,10,11} of column block db, as lds_load_a_transposed
+  PanelLane pl;
+  pl.init(l);
+  auto readK = [&](const char *ldsK, int sb, int ks) -> v8 { return panel_read_rows<T, BK>(ldsK, pl, sb, ks); };
   auto readV = [&](const char *ldsV, int sb, int db, int c) -> v8 {
-    const char *p0 = ldsV + vofs + (sb * 32 + 16 * c) * ROWB + (db >> 1) * PANELB;
-    const u32x2 lo = lds_read_tr16(p0 + (db & 1) * 64);
-    const u32x2 hi = lds_read_tr16(p0 + 8 * ROWB + ((db & 1) ^ 1) * 64);
-    const u32x4 both = {lo.x, lo.y, hi.x, hi.y};
-    return as_v8<T>(both);
+    return panel_read_transposed<T, BK>(ldsV, pl, sb, db, c);
   };
 
   const T *mrow[QB]; // this lane's rows of a full mask tensor, set when an item starts
