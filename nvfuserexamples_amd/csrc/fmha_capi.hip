@@ -144,9 +144,10 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
-  // flop.  That pays (3-5 % measured) for the plain variants at head dim 64 when there is
-  // enough work for every resident workgroup to get several 256-query items; with dropout, a
-  // causal or a full mask the per-element work dominates and one block per wave is faster.
+  // flop.  That pays (about 5 % measured) for the plain variants at head dim 64 on long key
+  // ranges when there is enough work for every resident workgroup to get several 256-query
+  // items; with dropout, a causal or a full mask the per-element work dominates, and on short
+  // key ranges the longer per-item prologue does, so one block per wave is faster there.
   v.qb = 1;
   if (p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull) {
     static const int cus = [] {
@@ -159,7 +160,7 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
     const int tiles2 = (p->sq + 255) / 256;
     const long long items2 = (long long)p->bh * tiles2;
     const bool little_padding = tiles2 * 256 - p->sq <= p->sq / 8;
-    if (cus > 0 && items2 >= 4LL * cus && little_padding) v.qb = 2;
+    if (cus > 0 && items2 >= 4LL * cus && little_padding && p->sk >= 1024) v.qb = 2;
   }
   const int force = env_int("FMHA_FWD_QB", 0); // tuning override: 1 or 2
   if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;

@@ -52,8 +52,40 @@ template <int D, int QB> struct PipeCfg {
   static constexpr int lds_bytes(int nw) { return LDS_BYTES + (QLDS ? nw * QB * 32 * D * 2 : 0); }
 };
 
+// The LDS operands of one steady-state iteration in issue order.  kind 0: V^T block of the
+// second product (sb, c, db); kind 1: K rows of contraction step ks for sub-block sb; kind 2: the
+// extra-step rows of sub-block sb.  The two products alternate so that consecutive MFMAs never
+// share an accumulator: a dependent MFMA cannot start until its predecessor has drained the
+// matrix pipe (about twice the issue interval).
+struct FwdOperandList {
+  int n;
+  int kind[48], a0[48], a1[48], a2[48];
+};
+template <int NSB, int KS, int DB, bool WITH_FIRST_PRODUCT> constexpr FwdOperandList fwd_operand_list() {
+  FwdOperandList L{};
+  int n = 0;
+  constexpr int S2 = NSB * 2, S1 = WITH_FIRST_PRODUCT ? KS + 1 : 0, S = S2 > S1 ? S2 : S1;
+  for (int i = 0; i < S; ++i) {
+    if (i < S2)
+      for (int db = 0; db < DB; ++db) {
+        L.kind[n] = 0; L.a0[n] = i / 2; L.a1[n] = i % 2; L.a2[n] = db;
+        ++n;
+      }
+    if (i < S1)
+      for (int sb = 0; sb < NSB; ++sb) {
+        L.kind[n] = i < KS ? 1 : 2; L.a0[n] = i; L.a1[n] = sb; L.a2[n] = 0;
+        ++n;
+      }
+  }
+  L.n = n;
+  return L;
+}
+
+// (Two query blocks per wave, and head dim 128, need more than the 256 registers of a
+// two-waves-per-SIMD budget by a few; the occupancy attribute makes the compiler spill those
+// few instead of settling for one wave per SIMD, which measures 8-30 % faster.)
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
-__global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 2 || D == 128) ? 2 : 1, 2))) void fmha_fwd_pipe_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -289,50 +321,66 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
         }
   };
 
-  // Both products of one iteration, issued so that consecutive MFMAs never share an
-  // accumulator: a dependent MFMA cannot start until its predecessor has drained the
-  // matrix pipe (about twice the issue interval), so the four accumulator chains
-  // o[.][0], o[.][1], x[.][0], x[.][1] are visited round-robin.
-  auto g12 = [&](int tprev, const v8 (&p)[QB][NSB][2], int tnext, f32x16 (&x)[QB][NSB], float (&bk)[QB]) {
+  // One steady-state iteration's matrix work and softmax arithmetic as ONE hand-ordered
+  // instruction stream: second product of tile tprev (probabilities p), first product of tile
+  // tnext into x (skipped when LASTT), and P = exp2(xc) rounded into pc with its row sums rs.
+  // MFMA and VALU work overlap only when they alternate inside one wave, and an LDS operand
+  // must be requested a few MFMAs before its use, so the stream is built as groups of
+  // {request operand j+kAhead, MFMAs of operand j, a slice of the exponentials} and every
+  // group is closed by a scheduling barrier that nothing may cross.
+  auto fused_step = [&](auto last_tag, int tprev, const v8 (&p)[QB][NSB][2], int tnext, f32x16 (&x)[QB][NSB],
+                        float (&bk)[QB], const f32x16 (&xc)[QB][NSB], v8 (&pc)[QB][NSB][2], float (&rs)[QB]) {
+    constexpr bool LASTT = decltype(last_tag)::value;
+    constexpr FwdOperandList ops = fwd_operand_list<NSB, KS, DB, !LASTT>();
+    constexpr int kAhead = QB == 1 ? 3 : 2; // operands in flight; two query blocks leave fewer registers
+    constexpr int NSL = QB * NSB * 8; // slices: two exponentials, one pack, one dot2 each
     const char *ldsV = ldsVb + (tprev & 1) * TILEB;
     const char *ldsK = ldsKb + (tnext & 1) * TILEB;
     const char *ldsX = ldsXb + (tnext & 1) * BK * XROWB;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) bk[qb] = mref[qb];
+    for (int qb = 0; qb < QB; ++qb) {
+      bk[qb] = mref[qb];
+      rs[qb] = 0.f;
+    }
+    auto fetch = [&](int j) -> v8 {
+      if (ops.kind[j] == 0) return readV(ldsV, ops.a0[j], ops.a2[j], ops.a1[j]);
+      if (ops.kind[j] == 1) return readK(ldsK, ops.a1[j], ops.a0[j]);
+      return as_v8<T>(*(const u32x4 *)(ldsX + (ops.a1[j] * 32 + ql) * XROWB + h * 16));
+    };
+    auto slice = [&](int sidx) {
+      const int qb = sidx / (NSB * 8), sb = (sidx / 8) % NSB, pr = sidx % 8;
+      const float e0 = fast_exp2(xc[qb][sb][2 * pr]), e1 = fast_exp2(xc[qb][sb][2 * pr + 1]);
+      const int c = pr / 4, j = pr % 4;
+      pc[qb][sb][c][2 * j] = (T)e0;
+      pc[qb][sb][c][2 * j + 1] = (T)e1;
+      rs[qb] = dot2_ones<T>(pc[qb][sb][c], j, rs[qb]);
+    };
+    v8 opnd[ops.n];
 #pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
+    for (int j = 0; j < kAhead && j < ops.n; ++j) opnd[j] = fetch(j);
+    int done = 0;
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
+    for (int j = 0; j < ops.n; ++j) {
+      if (j + kAhead < ops.n) opnd[j + kAhead] = fetch(j + kAhead);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) x[qb][sb][r] = 0.f;
-    constexpr int STEPS2 = NSB * 2;                    // second product: (sb, c) pairs, DB MFMAs each
-    constexpr int STEPS1 = KS + 1;                     // first product: contraction steps, NSB MFMAs each
-    constexpr int STEPS = STEPS1 > STEPS2 ? STEPS1 : STEPS2;
+      for (int qb = 0; qb < QB; ++qb) {
+        if (ops.kind[j] == 0) {
+          o[qb][ops.a2[j]] = E::mfma(opnd[j], p[qb][ops.a0[j]][ops.a1[j]], o[qb][ops.a2[j]]);
+        } else {
+          f32x16 acc;
+          if (ops.a0[j] == 0) {
 #pragma unroll
-    for (int i = 0; i < STEPS; ++i) {
-      if (i < STEPS2) {
-        const int sb = i / 2, c = i % 2;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const v8 va = readV(ldsV, sb, db, c);
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) o[qb][db] = E::mfma(va, p[qb][sb][c], o[qb][db]);
-        }
-      }
-      if (i < STEPS1) {
-#pragma unroll
-        for (int sb = 0; sb < NSB; ++sb) {
-          if (i < KS) {
-            const v8 ka = readK(ldsK, sb, i);
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) x[qb][sb] = E::mfma(ka, qreg[qb][i], x[qb][sb]);
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
           } else {
-            const v8 xa = as_v8<T>(*(const u32x4 *)(ldsX + (sb * 32 + ql) * XROWB + h * 16));
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) x[qb][sb] = E::mfma(xa, bx[qb], x[qb][sb]);
+            acc = x[qb][ops.a1[j]];
           }
+          x[qb][ops.a1[j]] = E::mfma(opnd[j], ops.kind[j] == 1 ? qreg[qb][ops.a0[j]] : bx[qb], acc);
         }
       }
+      const int upto = (j + 1) * NSL / ops.n;
+#pragma unroll
+      for (; done < upto; ++done) slice(done);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
@@ -382,25 +430,6 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
     }
     return rs;
   };
-  auto exp_pack0 = [&](const f32x16 (&x)[NSB], v8 (&pk)[NSB][2]) -> float {
-    float rs = 0.f;
-#pragma unroll
-    for (int sb = 0; sb < NSB; ++sb) {
-      float p[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) p[r] = fast_exp2(x[sb][r]);
-
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pk[sb][c][j] = (T)p[8 * c + j];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) rs = dot2_ones<T>(pk[sb][c], j, rs);
-      }
-    }
-    return rs;
-  };
-
   // move the reference of query block qb to this tile's maximum (x is relative to bk);
   // returns the shift that re-bases x onto the new reference
   auto rebase = [&](int qb, const f32x16 (&x)[NSB], float bk) -> float {
@@ -476,31 +505,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_pipe_kernel(const FwdArgs a)
         dropout(t, qb, pcur[qb]);
       }
     } else {
-      if (LAST) g2(t - 1, pprev);
-      else g12(t - 1, pprev, t + 1, xn, bkn);
       float rs[QB];
+      fused_step(last_tag, t - 1, pprev, t + 1, xn, bkn, xc, pcur, rs);
       bool unfit = false;
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        rs[qb] = exp_pack0(xc[qb], pcur[qb]);
+      for (int qb = 0; qb < QB; ++qb)
         unfit = unfit | !(rs[qb] < WINDOW) | !seen[qb] | (bkc[qb] != mref[qb]); // no short circuit: keep one basic block
-      }
-      // Shape of this block for the scheduler: operand reads run a few MFMAs ahead of their
-      // use (LDS latency), and every MFMA is followed by a slice of the softmax VALU work.
-      {
-        constexpr int kMfma = QB * (DB * NSB * 2 + (LAST ? 0 : NSB * (KS + 1)));
-        constexpr int kReads = DB * NSB * 2 * 2 + (LAST ? 0 : NSB * (KS + 1));
-        constexpr int kValu = QB * NSB * (16 + 8 + 8) + 8;
-        constexpr int kAhead = 6;
-        constexpr int kValuPer = (kValu + kMfma - 1) / kMfma;
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
-#pragma unroll
-        for (int i = 0; i < kMfma; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (kAhead + 2 * i < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, kValuPer, 0);
-        }
-      }
       if (__builtin_amdgcn_ballot_w64(unfit) != 0ull) {
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
