@@ -179,10 +179,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
   const uint32_t lds_base = lds_address(lds);
   PanelLane pl;
   pl.init(l);
+  TileCopy<T, D, BK, NT> tcopy;
+  tcopy.init(tid);
   auto dma_kv = [&](int kt) {
     const uint32_t dst = lds_base + (uint32_t)(kt & 1) * 2 * TILEB;
-    dma_tile_rows<T, D, BK, NT>(Kb, kt * BK, kend, dst, tid);
-    dma_tile_rows<T, D, BK, NT>(Vb, kt * BK, kend, dst + TILEB, tid);
+    tcopy.issue(Kb, kt * BK, kend, dst, tid);
+    tcopy.issue(Vb, kt * BK, kend, dst + TILEB, tid);
   };
   T mraw = (T)0.f;
   bool mvalid = false;
@@ -456,10 +458,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a)
   const uint32_t lds_base = lds_address(lds);
   PanelLane pl;
   pl.init(l);
+  TileCopy<T, D, BQ, NT> tcopy;
+  tcopy.init(tid);
   auto dma_qdo = [&](int qt) {
     const uint32_t dst = lds_base + (uint32_t)(qt & 1) * 2 * TILEB;
-    dma_tile_rows<T, D, BQ, NT>(Qb, qt * BQ, a.sq, dst, tid);
-    dma_tile_rows<T, D, BQ, NT>(dOb, qt * BQ, a.sq, dst + TILEB, tid);
+    tcopy.issue(Qb, qt * BQ, a.sq, dst, tid);
+    tcopy.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid);
   };
   float lraw = 0.f, draw = 0.f;
   bool qvalid = false;

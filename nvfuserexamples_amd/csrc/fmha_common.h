@@ -128,24 +128,62 @@ FMHA_DEV uint32_t lds_address(const void *p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)p;
 }
 
-// Copies rows [row0, row0 + BT) of a row-major [rows][D] matrix into a swizzled tile whose
-// LDS byte address is lds_tile; NT threads take part, tid is the caller's index among them.
-// Rows >= rend re-read row rend - 1 (callers neutralise them through their extra-step rows).
-template <typename T, int D, int BT, int NT>
-FMHA_DEV void dma_tile_rows(const T *base, int row0, int rend, uint32_t lds_tile, int tid) {
-  constexpr int CHUNKS = BT * D / 8;
-  static_assert(D % 64 == 0 && CHUNKS % NT == 0, "tile must divide evenly over the workgroup");
-  const uint32_t wave_dst = lds_tile + (uint32_t)(tid >> 6) * 1024u;
-#pragma unroll
-  for (int i = 0; i < CHUNKS / NT; ++i) {
-    const int c = tid + i * NT; // chunk slot: panel c / (8*BT), row (c / 8) % BT, position c % 8
-    const int panel = c / (8 * BT), row = (c / 8) % BT, pos = c % 8;
-    const int col = panel * 8 + (pos ^ ((row >> 1) & 7));
-    int r = row0 + row;
-    r = r < rend ? r : rend - 1;
-    dma_global_to_lds_b128(base + (size_t)r * D + col * 8, wave_dst + (uint32_t)(i * NT * 16));
-  }
+// The same copy with the global address given as a wave-uniform base plus a 32-bit per-lane
+// byte offset, so that a lane can keep its offset for the whole kernel and the base advances
+// on the scalar unit.
+FMHA_DEV void dma_global_to_lds_b128(const void *uniform_base, uint32_t lane_offset, uint32_t lds_wave_base) {
+  lds_wave_base = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_wave_base);
+  const uint64_t b = (uint64_t)uniform_base;
+  const uint64_t ub = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b >> 32)) << 32) |
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)b);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_wave_base), "v"(lane_offset),
+               "s"(ub)
+               : "memory");
 }
+
+// Copies rows [row0, row0 + BT) of a row-major [rows][D] matrix into a swizzled tile; NT
+// threads take part.  Rows >= rend re-read row rend - 1 (callers neutralise them through
+// their extra-step rows).  The lane's byte offsets inside a tile are computed once (init).
+template <typename T, int D, int BT, int NT> struct TileCopy {
+  static constexpr int CHUNKS = BT * D / 8;
+  static constexpr int CPT = CHUNKS / NT;
+  static_assert(D % 64 == 0 && CHUNKS % NT == 0, "tile must divide evenly over the workgroup");
+  uint32_t voff[CPT];
+
+  // chunk slot c of a tile: panel c / (8*BT), row (c / 8) % BT, position c % 8, which holds the
+  // row's chunk panel*8 + (position ^ ((row >> 1) & 7))
+  static FMHA_DEV void slot(int c, int &row, int &col) {
+    const int panel = c / (8 * BT), pos = c % 8;
+    row = (c / 8) % BT;
+    col = panel * 8 + (pos ^ ((row >> 1) & 7));
+  }
+  FMHA_DEV void init(int tid) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      int row, col;
+      slot(tid + i * NT, row, col);
+      voff[i] = (uint32_t)(row * D * 2 + col * 16);
+    }
+  }
+  // lds_tile: LDS byte address of the destination tile; tid: the caller's index among the NT threads
+  FMHA_DEV void issue(const T *base, int row0, int rend, uint32_t lds_tile, int tid) const {
+    const uint32_t wave_dst = lds_tile + (uint32_t)(tid >> 6) * 1024u;
+    if (row0 + BT <= rend) { // wave-uniform: a full tile needs no per-lane address arithmetic
+      const T *tb = base + (size_t)row0 * D;
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) dma_global_to_lds_b128(tb, voff[i], wave_dst + (uint32_t)(i * NT * 16));
+    } else {
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) {
+        int row, col;
+        slot(tid + i * NT, row, col);
+        int r = row0 + row;
+        r = r < rend ? r : rend - 1;
+        dma_global_to_lds_b128(base + (size_t)r * D + col * 8, wave_dst + (uint32_t)(i * NT * 16));
+      }
+    }
+  }
+};
 
 // Per-lane offsets of the two kinds of operand read from a swizzled tile.
 struct PanelLane {

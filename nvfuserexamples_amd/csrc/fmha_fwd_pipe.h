@@ -160,8 +160,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // Copy tile `tile` of `base` (K or V of a head) into stage (tile & 1) of the LDS area at byte
   // offset area_off.  Rows past kend re-read the last valid row: their scores get -inf through
   // the extra step, and finite garbage in V is multiplied by P = 0.
+  TileCopy<T, D, BK, NT> tcopy;
+  tcopy.init(tid);
   auto dma_tile = [&](const T *base, int kend, int tile, uint32_t area_off) {
-    dma_tile_rows<T, D, BK, NT>(base, tile * BK, kend, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
+    tcopy.issue(base, tile * BK, kend, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
   };
   // K tile u of the stream that runs from the current item on into the next one (u may reach
   // past the current item's last tile; nkt2 is even, so the stage parity carries over)
@@ -277,14 +279,22 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // and the rounded probabilities of the previous / current tile
   f32x16 xA[QB][NSB], xB[QB][NSB];
   float bkA[QB], bkB[QB];
+  // Row-sum limit that goes with each x buffer: the 2^14 window while the buffer's baked
+  // reference is current, -1 (every sum fails) when the buffer was baked before a reference
+  // existed or has been overtaken by a change of the reference.  lim_now is what a buffer baked
+  // now would get.
+  float limA[QB], limB[QB], lim_now[QB];
   v8 pA[QB][NSB][2], pB[QB][NSB][2];
 
   // first product of `tile` into x, baking the current reference
-  auto g1 = [&](int tile, f32x16 (&x)[QB][NSB], float (&bk)[QB]) {
+  auto g1 = [&](int tile, f32x16 (&x)[QB][NSB], float (&bk)[QB], float (&lim)[QB]) {
     const char *ldsK = ldsKb + (tile & 1) * TILEB;
     const char *ldsX = ldsXb + (tile & 1) * BK * XROWB;
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) bk[qb] = mref[qb];
+    for (int qb = 0; qb < QB; ++qb) {
+      bk[qb] = mref[qb];
+      lim[qb] = lim_now[qb];
+    }
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
@@ -329,7 +339,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // {request operand j+kAhead, MFMAs of operand j, a slice of the exponentials} and every
   // group is closed by a scheduling barrier that nothing may cross.
   auto fused_step = [&](auto last_tag, int tprev, const v8 (&p)[QB][NSB][2], int tnext, f32x16 (&x)[QB][NSB],
-                        float (&bk)[QB], const f32x16 (&xc)[QB][NSB], v8 (&pc)[QB][NSB][2], float (&rs)[QB]) {
+                        float (&bk)[QB], float (&lim)[QB], const f32x16 (&xc)[QB][NSB], v8 (&pc)[QB][NSB][2],
+                        float (&rs)[QB]) {
     constexpr bool LASTT = decltype(last_tag)::value;
     constexpr FwdOperandList ops = fwd_operand_list<NSB, KS, DB, !LASTT>();
     constexpr int kAhead = QB == 1 ? 3 : 2; // operands in flight; two query blocks leave fewer registers
@@ -340,6 +351,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       bk[qb] = mref[qb];
+      lim[qb] = lim_now[qb];
       rs[qb] = 0.f;
     }
     auto fetch = [&](int j) -> v8 {
@@ -445,6 +457,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       const float cand = (float)(T)(bk + mx);
       mnew = seen[qb] ? fmaxf(mref[qb], cand) : cand;
       seen[qb] = true;
+      lim_now[qb] = WINDOW;
     }
     const float up = mref[qb] - mnew;
     if (up != 0.f) {
@@ -486,7 +499,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // is refilled for tile t+3 -- all before the copies are issued, because the compiler's own
   // wait for a load it knows about also waits for every copy issued ahead of it.
   auto body = [&](int t, auto first_tag, auto last_tag, auto guarded_tag, f32x16 (&xc)[QB][NSB], float (&bkc)[QB],
-                  f32x16 (&xn)[QB][NSB], float (&bkn)[QB], const v8 (&pprev)[QB][NSB][2], v8 (&pcur)[QB][NSB][2]) {
+                  float (&limc)[QB], f32x16 (&xn)[QB][NSB], float (&bkn)[QB], float (&limn)[QB],
+                  const v8 (&pprev)[QB][NSB][2], v8 (&pcur)[QB][NSB][2]) {
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr bool LAST = decltype(last_tag)::value;
     lstoreX(t + 2, xs);
@@ -498,7 +512,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       float shift[QB];
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) shift[qb] = rebase(qb, xc[qb], bkc[qb]);
-      if (!LAST) g1(t + 1, xn, bkn);
+      if (!LAST) g1(t + 1, xn, bkn, limn);
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         lsum[qb] += exp_pack(xc[qb], shift[qb], pcur[qb]);
@@ -506,16 +520,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       }
     } else {
       float rs[QB];
-      fused_step(last_tag, t - 1, pprev, t + 1, xn, bkn, xc, pcur, rs);
+      fused_step(last_tag, t - 1, pprev, t + 1, xn, bkn, limn, xc, pcur, rs);
       bool unfit = false;
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
-        unfit = unfit | !(rs[qb] < WINDOW) | !seen[qb] | (bkc[qb] != mref[qb]); // no short circuit: keep one basic block
+      for (int qb = 0; qb < QB; ++qb) unfit = unfit | !(rs[qb] < limc[qb]); // no short circuit: keep one basic block
       if (__builtin_amdgcn_ballot_w64(unfit) != 0ull) {
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
           const float shift = rebase(qb, xc[qb], bkc[qb]);
           rs[qb] = exp_pack(xc[qb], shift, pcur[qb]);
+          if (bkn[qb] != mref[qb]) limn[qb] = -1.f; // the next buffer was baked with the old reference
         }
       }
 #pragma unroll
@@ -587,6 +601,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     for (int qb = 0; qb < QB; ++qb) {
       mref[qb] = 0.f;
       seen[qb] = false;
+      lim_now[qb] = -1.f;
       lsum[qb] = 0.f;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
@@ -605,7 +620,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       if (MASK == kMaskFull)
         mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
     }
-    g1(0, xA, bkA);
+    g1(0, xA, bkA, limA);
     __syncthreads(); // tile 0's K stage is refilled during the first iteration
     // The next item's Q rows are requested here rather than earlier so that the wait they end
     // up in is the one at the end of the first iteration.  The Q buffer has been read (the
@@ -614,23 +629,23 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
 
     const int nkt2 = cur.nkt2;
     // t = 0
-    if (diag(0)) body(0, Yes{}, No{}, Yes{}, xA, bkA, xB, bkB, pB, pA);
-    else body(0, Yes{}, No{}, No{}, xA, bkA, xB, bkB, pB, pA);
+    if (diag(0)) body(0, Yes{}, No{}, Yes{}, xA, bkA, limA, xB, bkB, limB, pB, pA);
+    else body(0, Yes{}, No{}, No{}, xA, bkA, limA, xB, bkB, limB, pB, pA);
     tile_sync();
     // steady state, two tiles per trip so that the buffers keep fixed roles
     for (int t = 1; t < nkt2 - 1; t += 2) {
-      if (diag(t)) body(t, No{}, No{}, Yes{}, xB, bkB, xA, bkA, pA, pB);
-      else body(t, No{}, No{}, No{}, xB, bkB, xA, bkA, pA, pB);
+      if (diag(t)) body(t, No{}, No{}, Yes{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
+      else body(t, No{}, No{}, No{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
       tile_sync();
-      if (diag(t + 1)) body(t + 1, No{}, No{}, Yes{}, xA, bkA, xB, bkB, pB, pA);
-      else body(t + 1, No{}, No{}, No{}, xA, bkA, xB, bkB, pB, pA);
+      if (diag(t + 1)) body(t + 1, No{}, No{}, Yes{}, xA, bkA, limA, xB, bkB, limB, pB, pA);
+      else body(t + 1, No{}, No{}, No{}, xA, bkA, limA, xB, bkB, limB, pB, pA);
       tile_sync();
     }
     // last tile (odd index) and the second product that is still owed
     {
       const int t = nkt2 - 1;
-      if (diag(t)) body(t, No{}, Yes{}, Yes{}, xB, bkB, xA, bkA, pA, pB);
-      else body(t, No{}, Yes{}, No{}, xB, bkB, xA, bkA, pA, pB);
+      if (diag(t)) body(t, No{}, Yes{}, Yes{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
+      else body(t, No{}, Yes{}, No{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
       tile_sync();
       g2(t, pB);
     }
