@@ -25,22 +25,23 @@ template <typename K> int set_lds(K kern, int bytes) {
 }
 
 template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s) {
-  using Cfg = BwdCfg<FMHA_TU_D>;
+  constexpr int kLdsQ = BwdCfg<FMHA_TU_D, bwd_dq_tile_rows<FMHA_TU_D>()>::LDS_BYTES;
+  constexpr int kLdsK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>::LDS_BYTES;
   auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP>;
   auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP>;
-  static const int attr = set_lds(kq, Cfg::LDS_BYTES) | set_lds(kk, Cfg::LDS_BYTES);
+  static const int attr = set_lds(kq, kLdsQ) | set_lds(kk, kLdsK);
   if (attr) return 2;
   constexpr int QT = kNW * kQB * 32, KT = kNW * kKB * 32;
   // dQ first: it also writes delta, which the dK/dV kernel reads (same stream => ordered)
   a.ntile = (a.sq + QT - 1) / QT;
   long long nblk = (long long)a.bh * a.ntile;
   if (nblk > 0x7fffffffLL) return 2;
-  hipLaunchKernelGGL(kq, dim3((unsigned)nblk), dim3(kNW * 64), Cfg::LDS_BYTES, s, a);
+  hipLaunchKernelGGL(kq, dim3((unsigned)nblk), dim3(kNW * 64), kLdsQ, s, a);
   if (hipGetLastError() != hipSuccess) return 2;
   a.ntile = (a.sk + KT - 1) / KT;
   nblk = (long long)a.bh * a.ntile;
   if (nblk > 0x7fffffffLL) return 2;
-  hipLaunchKernelGGL(kk, dim3((unsigned)nblk), dim3(kNW * 64), Cfg::LDS_BYTES, s, a);
+  hipLaunchKernelGGL(kk, dim3((unsigned)nblk), dim3(kNW * 64), kLdsK, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -50,8 +50,20 @@ struct BwdArgs {
   int32_t flags;
 };
 
-template <int D> struct BwdCfg {
-  static constexpr int BT = 64;           // rows per LDS tile
+// BT: rows per LDS tile (keys in the dQ kernel, queries in the dK/dV kernel).  The dK/dV kernel
+// at head dim 128 holds 128 accumulator registers; walking the queries 32 at a time brings its
+// score / dP tiles and their fragments close enough to a two-waves-per-SIMD register budget
+// that forcing that occupancy pays (+11 % measured) -- for the plain variant only: with a causal
+// mask the shorter tiles lose more to the uneven tile counts, and the dropout variant spills
+// too much, so those keep 64-row tiles at one wave per SIMD.
+template <int D> constexpr int bwd_dq_tile_rows() { return 64; }
+template <int D, bool CAUSAL, int DROP> constexpr bool bwd_dkdv_small_tiles() { return D == 128 && !CAUSAL && DROP == 0; }
+template <int D, bool CAUSAL, int DROP> constexpr int bwd_dkdv_tile_rows() {
+  return bwd_dkdv_small_tiles<D, CAUSAL, DROP>() ? 32 : 64;
+}
+
+template <int D, int BT_> struct BwdCfg {
+  static constexpr int BT = BT_;          // rows per LDS tile
   static constexpr int NSB = BT / 32;
   static constexpr int KS = D / 16;
   static constexpr int DB = D / 32;
@@ -71,12 +83,15 @@ template <typename T> FMHA_DEV void split_hi_lo(float v, T &hi, T &lo) {
 }
 
 // ------------------------------------------------------------------------------ dQ
+// (At head dim 128 some variants need a few registers more than a two-waves-per-SIMD budget:
+// spill those few rather than drop to one wave per SIMD, +10 % measured.)
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
-__global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64)
+    __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 1, 2))) void fmha_bwd_dq_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  using C = BwdCfg<D>;
+  using C = BwdCfg<D, bwd_dq_tile_rows<D>()>;
   constexpr int BK = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, TILEB = C::TILEB;
   constexpr int XROWB = C::XROWB;
   constexpr int NT = NW * 64;
@@ -368,11 +383,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_bwd_dq_kernel(const BwdArgs a) {
 
 // --------------------------------------------------------------------------- dK, dV
 template <typename T, int D, int KB, int NW, int MASK, bool CAUSAL, int DROP>
-__global__ __launch_bounds__(NW * 64) void fmha_bwd_dkdv_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(NW * 64)
+    __attribute__((amdgpu_waves_per_eu(bwd_dkdv_small_tiles<D, CAUSAL, DROP>() ? 2 : 1, 2))) void fmha_bwd_dkdv_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
-  using C = BwdCfg<D>;
+  using C = BwdCfg<D, bwd_dkdv_tile_rows<D, CAUSAL, DROP>()>;
   constexpr int BQ = C::BT, NSB = C::NSB, KS = C::KS, DB = C::DB, TILEB = C::TILEB;
   constexpr int XROWB = C::XROWB;
   constexpr int NT = NW * 64;
