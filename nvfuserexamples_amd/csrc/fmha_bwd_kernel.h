@@ -369,14 +369,7 @@ __global__ __launch_bounds__(NW * 64)
     const int q = q0w + qb * 32 + ql;
     if (q < a.sq) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          v4 t;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) t[i] = (T)(dq[qb][db][4 * gq + i] * a.scale);
-          *(v4 *)(dQb + (size_t)q * D + db * 32 + 8 * gq + 4 * h) = t;
-        }
+      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQb + (size_t)q * D + db * 32, dq[qb][db], a.scale, h);
     }
   }
 }
@@ -669,19 +662,10 @@ __global__ __launch_bounds__(NW * 64)
     const int key = k0w + kb * 32 + kl;
     if (key < a.sk) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          v4 tk, tv;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            tk[i] = (T)(dk[kb][db][4 * gq + i] * a.scale);
-            tv[i] = (T)dv[kb][db][4 * gq + i];
-          }
-          const size_t off = (size_t)key * D + db * 32 + 8 * gq + 4 * h;
-          *(v4 *)(dKb + off) = tk;
-          *(v4 *)(dVb + off) = tv;
-        }
+      for (int db = 0; db < DB; ++db) {
+        store_acc_block_row<T>(dKb + (size_t)key * D + db * 32, dk[kb][db], a.scale, h);
+        store_acc_block_row<T>(dVb + (size_t)key * D + db * 32, dv[kb][db], 1.f, h);
+      }
     }
   }
 }

@@ -232,6 +232,38 @@ FMHA_DEV float xhalf_sum(float x) {
   return __int_as_float(r[0]) + __int_as_float(r[1]);
 }
 
+// Store of one 32 (rows = lanes) x 32 (columns) accumulator block, scaled and rounded to T, into a
+// row-major matrix.  In the accumulator layout lane (row, h) holds the column groups
+// 8g + 4h .. +3 (g = 0..3) of its row: four 8-byte pieces 16 bytes apart.  Storing them as they
+// are makes every store instruction write 16-byte fragments of 32 different lines; exchanging
+// pieces between the two half-waves (v_permlane32_swap) gives each lane 16 contiguous bytes --
+// lane h = 0 the first half of a 32-byte group, lane h = 1 the second -- so the same data leaves
+// in half as many, twice as large, writes.  dst: the lane's row; the block starts at column 0.
+template <typename T> FMHA_DEV void store_acc_block_row(T *dst_row, const f32x16 &acc, float scale, int h) {
+#pragma unroll
+  for (int gp = 0; gp < 2; ++gp) {
+    typename Elem<T>::v4 x, y; // pieces g = 2gp and g = 2gp + 1
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = (T)(acc[4 * (2 * gp) + i] * scale);
+      y[i] = (T)(acc[4 * (2 * gp + 1) + i] * scale);
+    }
+    Pack8 px, py;
+    if constexpr (sizeof(T) == 2 && __is_same(T, _Float16)) {
+      px.h = x;
+      py.h = y;
+    } else {
+      px.b = x;
+      py.b = y;
+    }
+    // after the swaps: lanes h = 0 hold (own x, partner's x), lanes h = 1 hold (partner's y, own y)
+    auto r0 = __builtin_amdgcn_permlane32_swap((int)px.u.x, (int)py.u.x, false, false);
+    auto r1 = __builtin_amdgcn_permlane32_swap((int)px.u.y, (int)py.u.y, false, false);
+    const u32x4 both = {(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
+    *(u32x4 *)(dst_row + 16 * gp + 8 * h) = both;
+  }
+}
+
 FMHA_DEV float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 FMHA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 FMHA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

@@ -659,14 +659,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
       if (q < a.sq) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            v4 t;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) t[i] = (T)(o[qb][db][4 * g + i] * inv);
-            *(v4 *)(Ob + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
-          }
+        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * D + db * 32, o[qb][db], inv, h);
         const float cfix = (MASK == kMaskFull) ? a.mask_b - (float)(T)a.mask_b : 0.f;
         if (a.lse && h == 0)
           a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + cfix + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
