@@ -379,6 +379,26 @@ FMHA_DEV void drop_words_k(const DropCtx &c, uint32_t bh, uint32_t qb32, uint32_
   }
 }
 
+// Zeroes the dropped elements of four packed 16-bit values (two registers: elements t = 0,1 and
+// t = 2,3) whose random bytes are the four bytes of `word`.  Packed 16-bit arithmetic instead of a
+// compare and a select per element: the bytes are spread to 16-bit lanes (v_perm_b32), (thr-1) - byte
+// is negative exactly for kept elements, and its sign, smeared over the lane, is the keep mask.
+// thr_m1_x2 = (thr - 1) in both halves.
+FMHA_DEV void drop_apply_pk4(uint32_t word, uint32_t thr_m1_x2, uint32_t &pair01, uint32_t &pair23) {
+  typedef short s16x2 __attribute__((ext_vector_type(2)));
+  union {
+    uint32_t u;
+    s16x2 s;
+  } b01, b23, t, m01, m23;
+  b01.u = __builtin_amdgcn_perm(0u, word, 0x0c010c00u); // (byte0, byte1) zero-extended
+  b23.u = __builtin_amdgcn_perm(0u, word, 0x0c030c02u); // (byte2, byte3)
+  t.u = thr_m1_x2;
+  m01.s = (t.s - b01.s) >> 15;
+  m23.s = (t.s - b23.s) >> 15;
+  pair01 &= m01.u;
+  pair23 &= m23.u;
+}
+
 FMHA_DEV bool drop_keep_byte(uint32_t word, int t, uint32_t thr) {
   return ((word >> (8 * t)) & 0xffu) >= thr;
 }

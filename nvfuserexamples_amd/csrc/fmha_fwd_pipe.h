@@ -480,11 +480,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       for (int sb = 0; sb < NSB; ++sb) {
         uint32_t wd[4];
         drop_words_q(a.drop, (uint32_t)bh, (uint32_t)q, (uint32_t)(tile * BK + sb * 32), h, l, wd);
+        const uint32_t thr2 = ((a.drop.thr - 1u) & 0xffffu) * 0x00010001u; // thr = 0 gives -1: everything kept
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
-#pragma unroll
-          for (int t = 0; t < 4; ++t)
-            if (!drop_keep_byte(wd[g], t, a.drop.thr)) pk[sb][g >> 1][4 * (g & 1) + t] = (T)0.f;
+        for (int c = 0; c < 2; ++c) {
+          Pack16 pp;
+          if constexpr (std::is_same<T, _Float16>::value) pp.h = pk[sb][c];
+          else pp.b = pk[sb][c];
+          uint32_t r0 = pp.u.x, r1 = pp.u.y, r2 = pp.u.z, r3 = pp.u.w;
+          drop_apply_pk4(wd[2 * c], thr2, r0, r1);
+          drop_apply_pk4(wd[2 * c + 1], thr2, r2, r3);
+          pp.u = u32x4{r0, r1, r2, r3};
+          if constexpr (std::is_same<T, _Float16>::value) pk[sb][c] = pp.h;
+          else pk[sb][c] = pp.b;
+        }
       }
     }
   };
