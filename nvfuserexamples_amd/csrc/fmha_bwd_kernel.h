@@ -23,8 +23,9 @@
 // 64, so everything that is a rank-one term rides in one extra contraction step:
 //   x = score*scale*log2e + mask[key] - LSE[q]*log2e     (K' or Q' pre-scaled; mask and LSE
 //                                                         split hi+lo in the element type)
-//   g = dO.V^T - delta[q] / drop_scale
-// leaving  P = exp2(x)  and  dS = P * (kept ? drop_scale*g : -delta)  (= P*g without dropout).
+//   g = drop_scale * dO.V^T - delta[q]                 (the register-resident operand of that
+//                                                        product, dO or V, is pre-multiplied by drop_scale)
+// leaving  P = exp2(x)  and  dS = P * (kept ? g : -delta)  (= P*g without dropout).
 // "Minus infinity" terms are entered as a large finite negative number, because the same
 // extra rows also meet zeros in the other operand of the second product.
 #pragma once
@@ -45,7 +46,7 @@ struct BwdArgs {
   float mask_a, mask_b;
   int32_t bh, sq, sk;
   int32_t ntile; // tiles per head of the kernel being launched
-  float scale_l2, scale, drop_scale, inv_drop_scale;
+  float scale_l2, scale, drop_scale;
   DropCtx drop;
   int32_t flags;
 };
@@ -138,12 +139,13 @@ __global__ __launch_bounds__(NW * 64)
         to = *(const u32x4 *)(Ob + off);
       }
       const v8 qraw = as_v8<T>(tq);
-      doreg[qb][ks] = as_v8<T>(td);
+      const v8 doraw = as_v8<T>(td);
       const v8 ov = as_v8<T>(to);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         qreg[qb][ks][j] = (T)((float)qraw[j] * a.scale_l2);
-        dsum = fmaf((float)doreg[qb][ks][j], (float)ov[j], dsum);
+        doreg[qb][ks][j] = DROP == 1 ? (T)((float)doraw[j] * a.drop_scale) : doraw[j];
+        dsum = fmaf((float)doraw[j], (float)ov[j], dsum);
       }
     }
     dsum = xhalf_sum(dsum);
@@ -171,7 +173,7 @@ __global__ __launch_bounds__(NW * 64)
         bxs[qb][4] = hi;
         bxs[qb][5] = lo;
       }
-      split_hi_lo<T>(-dsum * a.inv_drop_scale, hi, lo);
+      split_hi_lo<T>(-dsum, hi, lo);
       bxd[qb][0] = hi;
       bxd[qb][1] = lo;
     }
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(NW * 64)
     const char *ldsV = ldsK + TILEB;
     const char *ldsX = ldsXb + cur * BK * XROWB;
 
-    // x^T = K.Q'^T + (mask - LSE) ; g^T = V.dO^T - delta/drop_scale   (accumulators visited round-robin)
+    // x^T = K.Q'^T + (mask - LSE) ; g^T = drop_scale*V.dO^T - delta   (accumulators visited round-robin)
     f32x16 x[QB][NSB], g[QB][NSB];
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(NW * 64)
             if (diag) xv = (kk + t <= q) ? xv : BIGNEG;
             const float p = fast_exp2(xv);
             float gv = g[qb][sb][4 * gq + t];
-            if (DROP == 1) gv = drop_keep_byte(wd[gq], t, a.drop.thr) ? gv * a.drop_scale : -delta[qb];
+            if (DROP == 1) gv = drop_keep_byte(wd[gq], t, a.drop.thr) ? gv : -delta[qb];
             ds[4 * gq + t] = p * gv;
           }
         }
@@ -427,9 +429,12 @@ __global__ __launch_bounds__(NW * 64)
         tv = *(const u32x4 *)(Vb + off);
       }
       const v8 kraw = as_v8<T>(tk);
-      vreg[kb][ks] = as_v8<T>(tv);
+      const v8 vraw = as_v8<T>(tv);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) kreg[kb][ks][j] = (T)((float)kraw[j] * a.scale_l2);
+      for (int j = 0; j < 8; ++j) {
+        kreg[kb][ks][j] = (T)((float)kraw[j] * a.scale_l2);
+        vreg[kb][ks][j] = DROP == 1 ? (T)((float)vraw[j] * a.drop_scale) : vraw[j];
+      }
     }
     float mk = 0.f;
     if (MASK == kMaskPerKey && key < a.sk)
@@ -506,7 +511,7 @@ __global__ __launch_bounds__(NW * 64)
       xs[3] = (T)1.f;
       xs[4] = (T)1.f;
       xs[5] = (T)1.f;
-      split_hi_lo<T>(-dl * a.inv_drop_scale, hi, lo);
+      split_hi_lo<T>(-dl, hi, lo);
       xd[0] = hi;
       xd[1] = lo;
       v8 *ds_ = (v8 *)(ldsXb + (stage * 2 + 0) * BQ * XROWB + tid * XROWB);
@@ -553,7 +558,7 @@ __global__ __launch_bounds__(NW * 64)
     const char *ldsXd = ldsXb + (cur * 2 + 1) * BQ * XROWB;
     const float *ldsD = ldsDl + cur * BQ;
 
-    // x = Q.K'^T + (mask - LSE) ; g = dO.V^T - delta/drop_scale
+    // x = Q.K'^T + (mask - LSE) ; g = drop_scale*dO.V^T - delta
     f32x16 x[KB][NSB], g[KB][NSB];
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
@@ -618,7 +623,7 @@ __global__ __launch_bounds__(NW * 64)
             float pzv = p;
             if (DROP == 1) {
               const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
-              gv = keep ? gv * a.drop_scale : -Dl[t];
+              gv = keep ? gv : -Dl[t];
               pzv = keep ? p * a.drop_scale : 0.f;
             }
             pz[4 * gq + t] = pzv;

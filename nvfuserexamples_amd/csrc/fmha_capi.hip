@@ -218,7 +218,6 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   a.scale_l2 = p->scale * FMHA_LOG2E;
   a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
   if (!(a.drop_scale > 0.f)) return FMHA_E_ARG;
-  a.inv_drop_scale = 1.f / a.drop_scale;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
 
