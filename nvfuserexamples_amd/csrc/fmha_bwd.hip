@@ -24,7 +24,7 @@ template <typename K> int set_lds(K kern, int bytes) {
                              bytes) == hipSuccess ? 0 : 2;
 }
 
-template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s) {
+template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipStream_t s) {
   constexpr int kLdsQ = BwdCfg<FMHA_TU_D, bwd_dq_tile_rows<FMHA_TU_D>()>::LDS_BYTES;
   constexpr int kLdsK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>::LDS_BYTES;
   auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP>;
@@ -33,21 +33,35 @@ template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, hipStream_t s)
   if (attr) return 2;
   constexpr int QT = kNW * kQB * 32, KT = kNW * kKB * 32;
   // dQ first: it also writes delta, which the dK/dV kernel reads (same stream => ordered)
+  // causal: workgroups take pairs of tiles (see the kernels) when that leaves at least two
+  // rounds of workgroups for the device
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      n = 0;
+    return n;
+  }();
   a.ntile = (a.sq + QT - 1) / QT;
-  long long nblk = (long long)a.bh * a.ntile;
+  auto want_pair = [&](int ntile) {
+    if (!CAUSAL) return false;
+    return pair >= 0 ? pair != 0 : (long long)a.bh * ((ntile + 1) / 2) >= 4LL * cus;
+  };
+  a.pair = want_pair(a.ntile);
+  long long nblk = (long long)a.bh * (a.pair ? (a.ntile + 1) / 2 : a.ntile);
   if (nblk > 0x7fffffffLL) return 2;
   hipLaunchKernelGGL(kq, dim3((unsigned)nblk), dim3(kNW * 64), kLdsQ, s, a);
   if (hipGetLastError() != hipSuccess) return 2;
   a.ntile = (a.sk + KT - 1) / KT;
-  nblk = (long long)a.bh * a.ntile;
+  a.pair = want_pair(a.ntile);
+  nblk = (long long)a.bh * (a.pair ? (a.ntile + 1) / 2 : a.ntile);
   if (nblk > 0x7fffffffLL) return 2;
   hipLaunchKernelGGL(kk, dim3((unsigned)nblk), dim3(kNW * 64), kLdsK, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
-template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, int drop, hipStream_t s) {
-  if (drop == 0) return launch<MASK, CAUSAL, 0>(a, s);
-  if (drop == 1) return launch<MASK, CAUSAL, 1>(a, s);
+template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
+  if (v.drop == 0) return launch<MASK, CAUSAL, 0>(a, v.pair, s);
+  if (v.drop == 1) return launch<MASK, CAUSAL, 1>(a, v.pair, s);
   return 1;
 }
 
@@ -55,10 +69,10 @@ template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, int drop, hipStream_t s
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
   if (v.mask == kMaskPerKey)
-    return v.causal ? by_drop<kMaskPerKey, true>(a, v.drop, s) : by_drop<kMaskPerKey, false>(a, v.drop, s);
+    return v.causal ? by_drop<kMaskPerKey, true>(a, v, s) : by_drop<kMaskPerKey, false>(a, v, s);
   if (v.mask == kMaskFull)
-    return v.causal ? by_drop<kMaskFull, true>(a, v.drop, s) : by_drop<kMaskFull, false>(a, v.drop, s);
-  return v.causal ? by_drop<kMaskNone, true>(a, v.drop, s) : by_drop<kMaskNone, false>(a, v.drop, s);
+    return v.causal ? by_drop<kMaskFull, true>(a, v, s) : by_drop<kMaskFull, false>(a, v, s);
+  return v.causal ? by_drop<kMaskNone, true>(a, v, s) : by_drop<kMaskNone, false>(a, v, s);
 }
 
 } // namespace fmha

@@ -46,6 +46,7 @@ struct BwdArgs {
   float mask_a, mask_b;
   int32_t bh, sq, sk;
   int32_t ntile; // tiles per head of the kernel being launched
+  int32_t pair;  // causal only: a workgroup takes the tile pair (i, ntile-1-i) instead of one tile
   float scale_l2, scale, drop_scale;
   DropCtx drop;
   int32_t flags;
@@ -109,9 +110,17 @@ __global__ __launch_bounds__(NW * 64)
   int bid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
-  const int bh = bid / a.ntile;
-  int qt = bid - bh * a.ntile;
-  if (CAUSAL) qt = a.ntile - 1 - qt;
+  // With a causal mask the work of a query tile grows with its index, so a workgroup takes a
+  // pair of tiles (i, n-1-i), one after the other: every workgroup then has the same amount of
+  // work (the host launches ceil(n/2) workgroups per head; it does so when that still fills the
+  // device, otherwise one tile per workgroup, longest first).
+  const bool paired = CAUSAL && a.pair;
+  const int npair = paired ? (a.ntile + 1) / 2 : a.ntile;
+  const int bh = bid / npair;
+  const int pi = bid - bh * npair;
+  const int npass = (paired && a.ntile - 1 - pi != pi) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+  const int qt = CAUSAL ? (pass == 0 ? a.ntile - 1 - pi : pi) : pi;
   const int q0w = qt * QT + w * (QB * 32);
 
   const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
@@ -374,6 +383,8 @@ __global__ __launch_bounds__(NW * 64)
       for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQb + (size_t)q * D + db * 32, dq[qb][db], a.scale, h);
     }
   }
+  __syncthreads(); // the next pass refills the tiles
+  } // pass
 }
 
 // --------------------------------------------------------------------------- dK, dV
@@ -403,8 +414,14 @@ __global__ __launch_bounds__(NW * 64)
   int bid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
-  const int bh = bid / a.ntile;
-  const int ktile = bid - bh * a.ntile;
+  // causal: a pair of key tiles (i, n-1-i) per workgroup, as in the dQ kernel
+  const bool paired = CAUSAL && a.pair;
+  const int npair = paired ? (a.ntile + 1) / 2 : a.ntile;
+  const int bh = bid / npair;
+  const int pi = bid - bh * npair;
+  const int npass = (paired && a.ntile - 1 - pi != pi) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+  const int ktile = pass == 0 ? pi : a.ntile - 1 - pi;
   const int k0w = ktile * KT + w * (KB * 32);
 
   const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
@@ -673,6 +690,8 @@ __global__ __launch_bounds__(NW * 64)
       }
     }
   }
+  __syncthreads(); // the next pass refills the tiles
+  } // pass
 }
 
 } // namespace fmha

@@ -40,7 +40,8 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
   return c;
 }
 
-// Tuning override for experiments: FMHA_FWD_QB=1|2 forces the query blocks per wave.
+// Tuning overrides for experiments and tests: FMHA_FWD_QB=1|2 forces the query blocks per wave of
+// the forward, FMHA_BWD_PAIR=0|1 the pairing of causal tiles in the backward.
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
   return e ? std::atoi(e) : dflt;
@@ -225,6 +226,7 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0;
+  v.pair = env_int("FMHA_BWD_PAIR", -1); // tuning / test override: 0 or 1
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;
   if (p->dtype == FMHA_DTYPE_F16)

@@ -26,6 +26,7 @@ struct BwdVariant {
   int mask;  // kMaskNone / kMaskPerKey / kMaskFull
   bool causal;
   int drop; // 0 none, 1 Philox
+  int pair; // causal tile pairing: -1 decide from the amount of work, 0 off, 1 on
 };
 
 int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);

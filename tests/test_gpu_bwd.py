@@ -31,6 +31,12 @@ CASES = [
     (2, 256, 256, 128, "fp16", None, False, 0.1),
     (2, 1024, 1024, 128, "bf16", None, True, 0.0),     # wide-head bf16 causal
     (4, 192, 192, 64, "bf16", "pad", False, 0.1),
+    # causal: a workgroup takes a pair of tiles (i, n-1-i); odd tile counts leave the middle one alone,
+    # and with sk > sq the last key tiles see no query at all
+    (3, 300, 300, 64, "fp16", None, True, 0.0),
+    (2, 200, 333, 64, "fp16", None, True, 0.1),
+    (2, 333, 200, 64, "fp16", "pad", True, 0.0),
+    (2, 640, 640, 128, "bf16", None, True, 0.0),
 ]
 
 
@@ -105,3 +111,25 @@ def test_backward_properties_at_headline_shape():
                   o0, lse0, mask=mc[[h // H for h in heads]].reshape(len(heads), 1, S).contiguous())
     for name, t in zip(("dq", "dk", "dv"), g0):
         assert rel_to_max(f32(t.cpu()), ref[name]) <= 1e-2, name
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,p", [(6, 300, 300, 64, "fp16", 0.1), (4, 200, 333, 64, "fp16", 0.0),
+                                                 (4, 640, 512, 128, "bf16", 0.0)])
+def test_causal_tile_pairing_is_bit_identical(bh, sq, sk, d, dtype, p, monkeypatch):
+    """With a causal mask and enough heads a workgroup of the backward kernels takes a pair of tiles
+    (i, n-1-i) so that all workgroups carry equal work.  Which tiles share a workgroup must not change
+    a single bit: the paired schedule (forced here, it is otherwise chosen only for large batches) is
+    compared with the one-tile-per-workgroup schedule that the oracle tests above exercise."""
+    q, k, v, do = make_qkv(bh, sq, sk, d, seed=5, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
+    qc, kc, vc, doc = (t.cuda() for t in (q, k, v, do))
+    kw = dict(causal=True)
+    if p:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=7, offset=3)
+    o, lse, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    outs = []
+    for pair in ("0", "1"):
+        monkeypatch.setenv("FMHA_BWD_PAIR", pair)
+        outs.append([t.clone() for t in capi.bwd(doc, qc, kc, vc, o, lse, **kw)])
+        torch.cuda.synchronize()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
