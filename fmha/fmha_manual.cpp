@@ -178,11 +178,24 @@ std::vector<at::Tensor> fmha_train_saveim_nvfuser(const at::Tensor &input, const
 
 // ---- general forward / backward (not in the reference) -------------------------------
 
+// Optional valid key counts: an int32 vector of B entries on q's device, B dividing BH.
+template <typename P> void set_kv_len(P &p, const c10::optional<at::Tensor> &kv_len, const at::Tensor &q,
+                                      at::Tensor &keep) {
+  if (!kv_len.has_value() || !kv_len->defined()) return;
+  TORCH_CHECK(kv_len->is_cuda() && kv_len->scalar_type() == at::kInt && kv_len->dim() == 1 && kv_len->numel() > 0 &&
+                  q.size(0) % kv_len->numel() == 0,
+              "mha_manual: kv_len must be an int32 GPU vector whose length divides BH");
+  keep = kv_len->contiguous();
+  p.kv_len = keep.data_ptr<int32_t>();
+  p.kv_len_bh_div = static_cast<int32_t>(q.size(0) / keep.numel());
+}
+
 // scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
 // (seed, offset); p_drop == 0 disables dropout.  Returns (O, LSE[bh,sq] fp32).
 std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
                                             const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
-                                            double p_drop, int64_t seed, int64_t offset) {
+                                            double p_drop, int64_t seed, int64_t offset,
+                                            const c10::optional<at::Tensor> &kv_len) {
   check_qkv(q, k, v);
   at::DeviceGuard guard(q.device());
   at::Tensor o = at::empty_like(q);
@@ -208,6 +221,8 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q, const at::Tenso
     p.seed = static_cast<uint64_t>(seed);
     p.offset = static_cast<uint64_t>(offset);
   }
+  at::Tensor kv_keep;
+  set_kv_len(p, kv_len, q, kv_keep);
   launch_fwd(p, q);
   return std::make_tuple(o, lse);
 }
@@ -215,7 +230,7 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q, const at::Tenso
 std::tuple<at::Tensor, at::Tensor, at::Tensor>
 fmha_bwd(const at::Tensor &dout, const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
          const at::Tensor &o, const at::Tensor &lse, const c10::optional<at::Tensor> &mask, double scale,
-         bool is_causal, double p_drop, int64_t seed, int64_t offset) {
+         bool is_causal, double p_drop, int64_t seed, int64_t offset, const c10::optional<at::Tensor> &kv_len) {
   check_qkv(q, k, v);
   at::DeviceGuard guard(q.device());
   TORCH_CHECK(dout.is_cuda() && o.is_cuda() && lse.is_cuda(), "mha_manual: dout/o/lse must live on the GPU");
@@ -263,6 +278,8 @@ fmha_bwd(const at::Tensor &dout, const at::Tensor &q, const at::Tensor &k, const
     p.seed = static_cast<uint64_t>(seed);
     p.offset = static_cast<uint64_t>(offset);
   }
+  at::Tensor kv_keep;
+  set_kv_len(p, kv_len, q, kv_keep);
   const int rc = fmha_bwd_launch(&p, current_stream(q));
   TORCH_CHECK(rc == FMHA_OK, "mha_manual backward: ", fmha_strerror(rc));
   return std::make_tuple(dq, dk, dv);
@@ -288,9 +305,9 @@ TORCH_LIBRARY(mha_manual, m) {
   m.def("fmha_train_saveim_nvfuser(Tensor input, Tensor qk, Tensor v, Tensor pad_mask, Tensor dropout_mask) -> "
         "Tensor[]");
   m.def("fmha_fwd(Tensor q, Tensor k, Tensor v, Tensor? mask, float scale, bool is_causal, float p_drop, int seed, "
-        "int offset) -> (Tensor, Tensor)");
+        "int offset, Tensor? kv_len=None) -> (Tensor, Tensor)");
   m.def("fmha_bwd(Tensor dout, Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor? mask, float scale, bool "
-        "is_causal, float p_drop, int seed, int offset) -> (Tensor, Tensor, Tensor)");
+        "is_causal, float p_drop, int seed, int offset, Tensor? kv_len=None) -> (Tensor, Tensor, Tensor)");
   m.def("fmha_philox_keep_mask(Tensor like, int bh, int sq, int sk, float p_drop, int seed, int offset) -> Tensor");
 }
 

@@ -95,6 +95,13 @@ typedef struct fmha_fwd_params {
   int32_t dtype;
   float scale; /* > 0; 1/8 in the reference (fmha_manual.cpp:68) */
   int32_t flags; /* reserved, pass 0 */
+
+  /* Optional valid key counts (the "padded version" the reference leaves as a TODO,
+   * fmha_manual.cpp:110,178): head b attends keys [0, kv_len[b / kv_len_bh_div]) only, exactly
+   * as if the others carried a -inf mask, and whole key tiles past the count are never touched.
+   * Device pointer to int32, or NULL for all sk keys.  Not with FMHA_DROP_TENSOR / the save outputs. */
+  const int32_t *kv_len;
+  int32_t kv_len_bh_div;
 } fmha_fwd_params;
 
 /* Enqueue the forward kernel on `hip_stream` (a hipStream_t; NULL = default stream). */
@@ -131,6 +138,9 @@ typedef struct fmha_bwd_params {
   int32_t dtype;
   float scale;
   int32_t flags; /* reserved, pass 0 */
+
+  const int32_t *kv_len; /* as in fmha_fwd_params; dk and dv rows at or past the count are zero */
+  int32_t kv_len_bh_div;
 } fmha_bwd_params;
 
 int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);

@@ -13,28 +13,32 @@ from . import load_ops
 
 class _Attention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, mask, scale, is_causal, p_drop, seed, offset):
+    def forward(ctx, q, k, v, mask, scale, is_causal, p_drop, seed, offset, kv_len):
         ops = load_ops()
-        o, lse = ops.fmha_fwd(q, k, v, mask, scale, is_causal, p_drop, seed, offset)
-        ctx.save_for_backward(q, k, v, o, lse, mask if mask is not None else q.new_empty(0))
+        o, lse = ops.fmha_fwd(q, k, v, mask, scale, is_causal, p_drop, seed, offset, kv_len)
+        ctx.save_for_backward(q, k, v, o, lse, mask if mask is not None else q.new_empty(0),
+                              kv_len if kv_len is not None else q.new_empty(0, dtype=torch.int32))
         ctx.has_mask = mask is not None
+        ctx.has_len = kv_len is not None
         ctx.args = (scale, is_causal, p_drop, seed, offset)
         return o
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, o, lse, mask = ctx.saved_tensors
+        q, k, v, o, lse, mask, kv_len = ctx.saved_tensors
         scale, is_causal, p_drop, seed, offset = ctx.args
         ops = load_ops()
         dq, dk, dv = ops.fmha_bwd(dout.contiguous(), q, k, v, o, lse, mask if ctx.has_mask else None,
-                                  scale, is_causal, p_drop, seed, offset)
-        return dq, dk, dv, None, None, None, None, None, None
+                                  scale, is_causal, p_drop, seed, offset, kv_len if ctx.has_len else None)
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
-def attention(q, k, v, mask=None, scale=0.0, is_causal=False, p_drop=0.0, seed=0, offset=0):
+def attention(q, k, v, mask=None, scale=0.0, is_causal=False, p_drop=0.0, seed=0, offset=0, kv_len=None):
     """softmax(scale * q k^T + mask [causal]) with Philox dropout, times v.
 
     q ``[B*H,Sq,D]``, k/v ``[B*H,Sk,D]`` (fp16 or bf16, contiguous, on the GPU); ``mask`` additive,
     shaped ``[B*H,Sq,Sk]``, ``[B*H,1,Sk]`` or ``[B,1,1,Sk]``; ``scale <= 0`` means ``1/sqrt(D)``.
-    The mask receives no gradient."""
-    return _Attention.apply(q, k, v, mask, float(scale), bool(is_causal), float(p_drop), int(seed), int(offset))
+    ``kv_len``: optional int32 GPU vector of B valid key counts (B divides B*H): keys at or past a
+    head's count are excluded and their key tiles skipped.  Masks and counts receive no gradient."""
+    return _Attention.apply(q, k, v, mask, float(scale), bool(is_causal), float(p_drop), int(seed), int(offset),
+                            kv_len)

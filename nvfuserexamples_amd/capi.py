@@ -29,6 +29,7 @@ class FwdParams(C.Structure):
         ("save_softmax", C.c_void_p), ("save_dropout", C.c_void_p),
         ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
         ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
+        ("kv_len", C.c_void_p), ("kv_len_bh_div", C.c_int32),
     ]
 
 
@@ -44,6 +45,7 @@ class BwdParams(C.Structure):
         ("seed", C.c_uint64), ("offset", C.c_uint64),
         ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
         ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
+        ("kv_len", C.c_void_p), ("kv_len_bh_div", C.c_int32),
     ]
 
 
@@ -114,10 +116,23 @@ def mask_layout(mask, bh, sq, sk):
     return mask, div, mask.shape[1] * sk, (0 if mask.shape[1] == 1 else sk)
 
 
+def _set_kv_len(P, kv_len, bh):
+    import torch
+    if kv_len is None:
+        return
+    if not (kv_len.is_cuda and kv_len.is_contiguous() and kv_len.dtype == torch.int32 and kv_len.dim() == 1
+            and kv_len.numel() > 0 and bh % kv_len.numel() == 0):
+        raise FmhaError(-5, "kv_len must be a contiguous int32 device vector whose length divides bh")
+    P.kv_len, P.kv_len_bh_div = kv_len.data_ptr(), bh // kv_len.numel()
+
+
 def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False, scale=None,
         drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
-        want_lse=False, save=False, flags=0, out=None):
-    """Launch the forward on the current stream.  Returns (o, lse|None, softmax|None, dropout|None)."""
+        want_lse=False, save=False, flags=0, out=None, kv_len=None):
+    """Launch the forward on the current stream.  Returns (o, lse|None, softmax|None, dropout|None).
+
+    kv_len: optional int32 device tensor of B valid key counts (bh must be a multiple of B); head i
+    attends keys [0, kv_len[i // (bh // B)]) only."""
     import torch
     bh, sq, d = q.shape
     sk = k.shape[1]
@@ -156,14 +171,15 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
         dr = torch.empty((bh, sq, sk), dtype=q.dtype, device=q.device)
         P.save_softmax, P.save_dropout = sm.data_ptr(), dr.data_ptr()
     P.flags = flags
+    _set_kv_len(P, kv_len, bh)
     check(lib().fmha_fwd_launch(C.byref(P), _stream_ptr()))
     return o, lse, sm, dr
 
 
 def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False,
         scale=None, drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
-        flags=0, delta=None, grads=None):
-    """Launch the backward on the current stream.  Returns (dq, dk, dv)."""
+        flags=0, delta=None, grads=None, kv_len=None):
+    """Launch the backward on the current stream.  Returns (dq, dk, dv).  kv_len as in fwd()."""
     import torch
     bh, sq, d = q.shape
     sk = k.shape[1]
@@ -195,6 +211,7 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     P.drop_scale = drop_scale
     P.seed, P.offset = seed, offset
     P.flags = flags
+    _set_kv_len(P, kv_len, bh)
     check(lib().fmha_bwd_launch(C.byref(P), _stream_ptr()))
     return dq, dk, dv
 

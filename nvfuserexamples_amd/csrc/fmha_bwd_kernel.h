@@ -50,6 +50,8 @@ struct BwdArgs {
   float scale_l2, scale, drop_scale;
   DropCtx drop;
   int32_t flags;
+  const int32_t *kv_len; // optional valid key count per group of kv_div heads
+  int32_t kv_div;
 };
 
 // BT: rows per LDS tile (keys in the dQ kernel, queries in the dK/dV kernel).  The dK/dV kernel
@@ -74,6 +76,13 @@ template <int D, int BT_> struct BwdCfg {
   // two tiles x 2 stages + two sets of extra rows x 2 stages + {delta} x 2 stages
   static constexpr int LDS_BYTES = 4 * TILEB + 2 * 2 * BT * XROWB + 2 * BT * 4;
 };
+
+// Keys a head may see at all: [0, sk) or its valid count (possibly 0).
+FMHA_DEV int bwd_valid_keys(const BwdArgs &a, int bh) {
+  if (!a.kv_len) return a.sk;
+  const int n = a.kv_len[bh / a.kv_div];
+  return n < 0 ? 0 : (n < a.sk ? n : a.sk);
+}
 
 // A value as hi + lo in the element type (|error| ~ 2^-2p relative), clamped to a large finite
 // negative number so that it may be multiplied by zero.
@@ -188,14 +197,17 @@ __global__ __launch_bounds__(NW * 64)
     }
   }
 
-  int nkt = (a.sk + BK - 1) / BK;
+  const int skv = bwd_valid_keys(a, bh);
+  int nkt = (skv + BK - 1) / BK;
+  if (nkt < 1) nkt = 1; // no valid key at all: one tile of keys that are all "past the end"
   if (CAUSAL) {
     int qmax = qt * QT + QT - 1;
     if (qmax > a.sq - 1) qmax = a.sq - 1;
     const int need = qmax / BK + 1;
     if (need < nkt) nkt = need;
   }
-  const int kend = nkt * BK < a.sk ? nkt * BK : a.sk;
+  const int kend = nkt * BK < skv ? nkt * BK : skv;
+  const int kclamp = kend > 0 ? kend : 1; // row bound for addresses
 
   // ---- staging.  K and V tiles are copied from global memory straight into LDS (rows past the
   // end re-read the last valid row; their scores are pushed to -60000 by the extra step, so
@@ -209,15 +221,15 @@ __global__ __launch_bounds__(NW * 64)
   tcopy.init(tid);
   auto dma_kv = [&](int kt) {
     const uint32_t dst = lds_base + (uint32_t)(kt & 1) * 2 * TILEB;
-    tcopy.issue(Kb, kt * BK, kend, dst, tid);
-    tcopy.issue(Vb, kt * BK, kend, dst + TILEB, tid);
+    tcopy.issue(Kb, kt * BK, kclamp, dst, tid);
+    tcopy.issue(Vb, kt * BK, kclamp, dst + TILEB, tid);
   };
   T mraw = (T)0.f;
   bool mvalid = false;
   auto gloadX = [&](int kt) {
     const int kr = kt * BK + (tid & (BK - 1));
     mvalid = kr < kend;
-    if (MASK == kMaskPerKey) mraw = mkey[mvalid ? kr : kend - 1];
+    if (MASK == kMaskPerKey) mraw = mkey[mvalid ? kr : kclamp - 1];
   };
   auto lstoreX = [&](int stage) {
     if (tid < BK) {
@@ -433,6 +445,7 @@ __global__ __launch_bounds__(NW * 64)
 
   // ---- per-key operands: K' and V rows as B operands, the extra-step columns
   v8 kreg[KB][KS], vreg[KB][KS];
+  const int skv = bwd_valid_keys(a, bh); // keys at or past it are invalid: their dK, dV rows are zero
   v8 bxs[KB], bxd[KB]; // (1, 1, mask_hi, mask_lo, c_hi, c_lo, 0, 0) and (1, 1, 0 ...) on the lower half-wave
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
@@ -440,7 +453,7 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 tk = {0u, 0u, 0u, 0u}, tv = {0u, 0u, 0u, 0u};
-      if (key < a.sk) {
+      if (key < skv) {
         const size_t off = (size_t)key * D + ks * 16 + h * 8;
         tk = *(const u32x4 *)(Kb + off);
         tv = *(const u32x4 *)(Vb + off);
@@ -454,9 +467,9 @@ __global__ __launch_bounds__(NW * 64)
       }
     }
     float mk = 0.f;
-    if (MASK == kMaskPerKey && key < a.sk)
+    if (MASK == kMaskPerKey && key < skv)
       mk = fmaf((float)((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + key], a.mask_a, a.mask_b);
-    if (key >= a.sk) mk = BIGNEG;
+    if (key >= skv) mk = BIGNEG;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       bxs[kb][j] = (T)0.f;
@@ -481,7 +494,8 @@ __global__ __launch_bounds__(NW * 64)
   const T *mbase = (MASK == kMaskFull) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
   const int nqt = (a.sq + BQ - 1) / BQ;
-  const int qt0 = CAUSAL ? (ktile * KT) / BQ : 0; // first query tile that sees any of these keys
+  // first query tile that sees any of these keys; none at all if the whole key tile is invalid
+  const int qt0 = ktile * KT >= skv ? nqt : (CAUSAL ? (ktile * KT) / BQ : 0);
 
   // ---- staging: Q and dO tiles copied straight into LDS (rows past the end repeat the last
   // valid row); the per-query extra rows take the register path one tile further ahead, as in

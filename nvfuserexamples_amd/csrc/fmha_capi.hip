@@ -108,6 +108,10 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   const bool saving = p->save_softmax || p->save_dropout;
   if (saving && (p->drop_kind == FMHA_DROP_PHILOX || p->causal)) return FMHA_E_UNSUPPORTED;
   if (p->drop_kind == FMHA_DROP_TENSOR && p->causal) return FMHA_E_UNSUPPORTED;
+  if (p->kv_len) {
+    if (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u)) return FMHA_E_ARG;
+    if (saving || p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED;
+  }
 
   FwdArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.lse = p->lse;
@@ -139,6 +143,8 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
+  a.kv_len = p->kv_len;
+  a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
@@ -194,6 +200,7 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_PHILOX && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED; // backward regenerates Philox decisions only
+  if (p->kv_len && (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u))) return FMHA_E_ARG;
 
   BwdArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.dout = p->dout;
@@ -221,6 +228,8 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   if (!(a.drop_scale > 0.f)) return FMHA_E_ARG;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
+  a.kv_len = p->kv_len;
+  a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
 
   BwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);

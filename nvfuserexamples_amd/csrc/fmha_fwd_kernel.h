@@ -62,6 +62,8 @@ struct FwdArgs {
   float drop_scale;
   DropCtx drop;
   int32_t flags;
+  const int32_t *kv_len; // optional valid key count per group of kv_div heads (pipelined kernel only)
+  int32_t kv_div;
 };
 
 // how the mask tensor is read

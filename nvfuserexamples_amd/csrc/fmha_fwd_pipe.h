@@ -136,14 +136,22 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     // round: long and short items then alternate within each workgroup.  (Within a round the
     // map stays one-to-one, so every item is still visited exactly once.)
     if (CAUSAL && ((idx / G) & 1) == 0) it.qt = a.nqt - 1 - it.qt;
-    int nkt = (a.sk + BK - 1) / BK;
+    // keys this head may see at all: [0, sk) or its valid count (possibly 0: then every key is
+    // treated as past the end, which yields O = 0 and LSE = -inf)
+    int sk = a.sk;
+    if (a.kv_len) {
+      const int n = a.kv_len[it.bh / a.kv_div];
+      sk = n < 0 ? 0 : (n < sk ? n : sk);
+    }
+    int nkt = (sk + BK - 1) / BK;
+    if (nkt < 1) nkt = 1;
     if (CAUSAL) {
       int qmax = it.qt * QT + QT - 1;
       if (qmax > a.sq - 1) qmax = a.sq - 1;
       const int need = qmax / BK + 1;
       if (need < nkt) nkt = need;
     }
-    it.kend = nkt * BK < a.sk ? nkt * BK : a.sk;
+    it.kend = nkt * BK < sk ? nkt * BK : sk;
     it.nkt2 = (nkt + 1) & ~1;
     it.Kb = (const T *)a.k + (size_t)it.bh * a.sk * D;
     it.Vb = (const T *)a.v + (size_t)it.bh * a.sk * D;
@@ -163,7 +171,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   TileCopy<T, D, BK, NT> tcopy;
   tcopy.init(tid);
   auto dma_tile = [&](const T *base, int kend, int tile, uint32_t area_off) {
-    tcopy.issue(base, tile * BK, kend, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
+    tcopy.issue(base, tile * BK, kend > 0 ? kend : 1, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
   };
   // K tile u of the stream that runs from the current item on into the next one (u may reach
   // past the current item's last tile; nkt2 is even, so the stage parity carries over)
@@ -223,7 +231,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     const int kr = tile * BK + (tid & (BK - 1));
     st.mvalid = kr < kend;
     st.mraw = (T)0.f;
-    if (MASK == kMaskPerKey) st.mraw = mk[st.mvalid ? kr : kend - 1];
+    if (MASK == kMaskPerKey) st.mraw = mk[st.mvalid ? kr : (kend > 0 ? kend - 1 : 0)];
   };
   auto lstoreX = [&](int tile, const XStage &st) {
     if (tid < BK) {
