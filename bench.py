@@ -111,6 +111,67 @@ def time_launches(torch, step, steps, warmup):
     return sum(a.elapsed_time(b) for a, b in ev) / steps
 
 
+def power_probe(torch, step, seconds=2.0):
+    """Socket power and graphics clocks as the board's management firmware reports them (amd-smi),
+    sampled while `step` runs back to back on a second thread.  The attention kernels are
+    power-limited on this part, so the figures belong beside the roofline fraction: the MFMA peak
+    is quoted at the maximum clock, which the board does not hold under this load.
+    Returns None where the tool is missing or its output has no such fields."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    exe = shutil.which("amd-smi") or "/opt/rocm/bin/amd-smi"
+    if not os.path.exists(exe):
+        return None
+
+    def sample():
+        try:
+            r = subprocess.run([exe, "metric", "-g", "0", "-c", "-p"], stdout=subprocess.PIPE,
+                               stderr=subprocess.DEVNULL, text=True, timeout=20)
+        except Exception:
+            return None
+        pw = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", r.stdout)
+        clk = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", r.stdout)]
+        mx = re.search(r"MAX_CLK:\s*(\d+)\s*MHz", r.stdout)
+        if not pw or not clk:
+            return None
+        return {"socket_power_w": int(pw.group(1)), "gfx_clk_mhz_mean": round(sum(clk) / len(clk)),
+                "gfx_clk_mhz_min": min(clk), "gfx_max_clk_mhz": int(mx.group(1)) if mx else None}
+
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+    idle = sample()
+    stop = [False]
+
+    def load():
+        i = 0
+        while not stop[0]:
+            for _ in range(100):
+                step(i)
+                i += 1
+            torch.cuda.synchronize()
+
+    th = threading.Thread(target=load)
+    th.start()
+    busy = []
+    t_end = time.perf_counter() + seconds
+    time.sleep(0.5)
+    while time.perf_counter() < t_end:
+        b = sample()
+        if b:
+            busy.append(b)
+    stop[0] = True
+    th.join()
+    if not idle or not busy:
+        return None
+    top = max(busy, key=lambda b: b["socket_power_w"])
+    return {"tool": "amd-smi metric -c -p, sampled while the headline kernel runs back to back",
+            "idle_socket_power_w": idle["socket_power_w"], "busy_socket_power_w": top["socket_power_w"],
+            "busy_gfx_clk_mhz_mean": top["gfx_clk_mhz_mean"], "busy_gfx_clk_mhz_min": top["gfx_clk_mhz_min"],
+            "gfx_max_clk_mhz": top["gfx_max_clk_mhz"], "samples": len(busy)}
+
+
 def cpu_baseline(torch, budget_s=12.0):
     """The reference's eager composition (its ground truth) on the host cores, fp32,
     on the reference-sized CPU case B8 H12 S128 D64 with a [B,1,1,S] padding mask."""
@@ -148,6 +209,7 @@ def main():
     ap.add_argument("--sets", type=int, default=4, help="input sets rotated to defeat the last-level cache")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-bwd", action="store_true", help="skip the train-step (fwd+bwd) leg")
+    ap.add_argument("--no-power", action="store_true", help="skip the socket power / clock telemetry leg")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: under `rocprofv3 --pmc FETCH_SIZE` "
                          "(or WRITE_SIZE) its known traffic calibrates the counter for the attention kernels")
@@ -207,6 +269,17 @@ def main():
         L.fmha_fwd_launch(C.byref(lps[i % len(lps)]), stream)
     capi.check(L.fmha_fwd_launch(C.byref(lps[0]), stream))
     ms_len, _ = time_steps(torch, fwd_len, args.steps, args.warmup)
+    # effective core clock while the headline kernel runs: counters of its first workgroup, read in the
+    # middle of a back-to-back run (clock_probe of the C ABI)
+    probe = torch.zeros(4, dtype=torch.int64, device="cuda")
+    fps[0].clock_probe = probe.data_ptr()
+    for i in range(args.warmup + 60):
+        fwd_step(i + 1)  # ends on input set 0
+    torch.cuda.synchronize()
+    fps[0].clock_probe = None
+    c0, t0, c1, t1 = probe.tolist()
+    eff_clock = round((c1 - c0) / ((t1 - t0) / 100.0), 1) if t1 > t0 else None
+    power = None if args.no_power else power_probe(torch, fwd_step)
     del sets, fps, lps, lens
 
     out = {
@@ -235,6 +308,9 @@ def main():
         "fwd_kv_len": {"workload": "same batches, valid lengths passed as counts instead of the mask tensor",
                        "ms_per_step": round(ms_len, 5), "speedup_vs_mask": round(ms / ms_len, 3)},
     }
+
+    out["power"] = power
+    out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
     # ---- train step (forward with LSE + Philox dropout, then backward)
     if not args.no_bwd:

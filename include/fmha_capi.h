@@ -102,6 +102,14 @@ typedef struct fmha_fwd_params {
    * Device pointer to int32, or NULL for all sk keys.  Not with FMHA_DROP_TENSOR / the save outputs. */
   const int32_t *kv_len;
   int32_t kv_len_bh_div;
+
+  /* Optional diagnostic (no counterpart in the reference): device pointer to four uint64, or NULL.
+   * The first workgroup of the pipelined forward kernel writes {core clock counter at its start,
+   * constant 100 MHz counter at its start, core clock counter at its end, 100 MHz counter at its
+   * end}; (c_end - c_start) / (t_end - t_start) * 100 is the effective core clock in MHz while
+   * the kernel ran, which on a power-limited board is well below the maximum clock that the
+   * published MFMA peak assumes.  Left untouched by the non-pipelined kernel. */
+  uint64_t *clock_probe;
 } fmha_fwd_params;
 
 /* Enqueue the forward kernel on `hip_stream` (a hipStream_t; NULL = default stream). */

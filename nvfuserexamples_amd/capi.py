@@ -30,6 +30,7 @@ class FwdParams(C.Structure):
         ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
         ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
         ("kv_len", C.c_void_p), ("kv_len_bh_div", C.c_int32),
+        ("clock_probe", C.c_void_p),
     ]
 
 

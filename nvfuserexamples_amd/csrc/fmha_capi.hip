@@ -112,6 +112,7 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
     if (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u)) return FMHA_E_ARG;
     if (saving || p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED;
   }
+  if ((uintptr_t)p->clock_probe & 7u) return FMHA_E_ARG;
 
   FwdArgs a;
   a.q = p->q; a.k = p->k; a.v = p->v; a.o = p->o; a.lse = p->lse;
@@ -145,6 +146,7 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   a.flags = p->flags;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
+  a.clock_probe = (unsigned long long *)p->clock_probe;
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);

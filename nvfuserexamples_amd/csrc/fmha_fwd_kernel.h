@@ -64,6 +64,7 @@ struct FwdArgs {
   int32_t flags;
   const int32_t *kv_len; // optional valid key count per group of kv_div heads (pipelined kernel only)
   int32_t kv_div;
+  unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
 };
 
 // how the mask tensor is read

@@ -112,6 +112,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   const int ql = l & 31;
   const int h = l >> 5;
 
+  // diagnostic: core clock counter and constant 100 MHz counter when the first workgroup starts
+  // (and, at the end of the kernel, when it finishes)
+  const bool probe = a.clock_probe != nullptr && blockIdx.x == 0 && tid == 0;
+  if (probe) {
+    a.clock_probe[0] = __builtin_readcyclecounter();
+    a.clock_probe[1] = __builtin_amdgcn_s_memrealtime();
+  }
+
   // ---- persistent schedule: this workgroup handles items lb, lb + G, lb + 2G, ...
   // Workgroups are dealt round-robin to the 8 XCDs; lb is chosen so that one XCD (one L2)
   // works on a contiguous run of items at any time, i.e. on the query tiles of few heads.
@@ -684,6 +692,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     if (!more) break;
     idx = nidx;
     cur = nxt;
+  }
+  if (probe) {
+    a.clock_probe[2] = __builtin_readcyclecounter();
+    a.clock_probe[3] = __builtin_amdgcn_s_memrealtime();
   }
 }
 
