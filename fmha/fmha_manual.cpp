@@ -18,6 +18,7 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/extension.h>
 
+#include <algorithm>
 #include <cmath>
 #include <tuple>
 #include <vector>
@@ -56,8 +57,8 @@ void check_qkv(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v) {
 }
 
 // Accepts [BH,Sq,Sk], [BH,1,Sk], [B,1,1,Sk] or [B,1,Sq,Sk] (B dividing BH).
-MaskLayout mask_layout(const at::Tensor &mask_in, const at::Tensor &q, int64_t sk, const char *what) {
-  const int64_t bh = q.size(0), sq = q.size(1);
+MaskLayout mask_layout(const at::Tensor &mask_in, const at::Tensor &q, int64_t bh, int64_t sq, int64_t sk,
+                       const char *what) {
   TORCH_CHECK(mask_in.is_cuda() && mask_in.device() == q.device(), "mha_manual: ", what, " must be on q's device");
   TORCH_CHECK(mask_in.scalar_type() == q.scalar_type(), "mha_manual: ", what, " must have q's dtype");
   at::Tensor m = mask_in;
@@ -108,7 +109,7 @@ at::Tensor fmha_nvfuser(const at::Tensor &input, const at::Tensor &qk, const at:
                         const at::Tensor &amask) {
   check_qkv(input, qk, v);
   at::DeviceGuard guard(input.device());
-  MaskLayout m = mask_layout(amask, input, qk.size(1), "amask");
+  MaskLayout m = mask_layout(amask, input, input.size(0), input.size(1), qk.size(1), "amask");
   at::Tensor o = at::empty_like(input);
   fmha_fwd_params p = {};
   fill_common(p, input, qk, v, o, default_scale(input));
@@ -132,7 +133,7 @@ std::vector<at::Tensor> train_forward(const at::Tensor &input, const at::Tensor 
   check_qkv(input, qk, v);
   at::DeviceGuard guard(input.device());
   const int64_t bh = input.size(0), sq = input.size(1), sk = qk.size(1);
-  MaskLayout m = mask_layout(pad_mask, input, sk, "pad_mask");
+  MaskLayout m = mask_layout(pad_mask, input, input.size(0), input.size(1), sk, "pad_mask");
   TORCH_CHECK(dropout_mask.is_cuda() && dropout_mask.device() == input.device() &&
                   dropout_mask.scalar_type() == input.scalar_type() && dropout_mask.dim() == 3 &&
                   dropout_mask.size(0) == bh && dropout_mask.size(1) == sq && dropout_mask.size(2) == sk,
@@ -178,35 +179,81 @@ std::vector<at::Tensor> fmha_train_saveim_nvfuser(const at::Tensor &input, const
 
 // ---- general forward / backward (not in the reference) -------------------------------
 
+// One of q, k, v, o, dout as the C ABI sees it: folded contiguous [BH,S,D] (heads = 0), or a 4-d
+// [B,H,S,D] tensor of any batch / head / row strides whose rows are contiguous (heads = H).
+struct RowsOf {
+  at::Tensor t; // the tensor itself, or a dense copy where its strides cannot be passed on
+  int64_t bh = 0, s = 0, d = 0;
+  int32_t heads = 0;
+  int64_t st[3] = {0, 0, 0};
+};
+
+RowsOf rows_of(const at::Tensor &x, const char *what) {
+  TORCH_CHECK(x.is_cuda(), "mha_manual: ", what, " must live on the GPU");
+  TORCH_CHECK(x.dim() == 3 || x.dim() == 4, "mha_manual: ", what, " must be [B*H,S,D] or [B,H,S,D]");
+  RowsOf r;
+  if (x.dim() == 3) {
+    r.t = x.contiguous();
+    r.bh = x.size(0);
+    r.s = x.size(1);
+    r.d = x.size(2);
+    return r;
+  }
+  bool ok = x.stride(3) == 1 && (reinterpret_cast<uintptr_t>(x.data_ptr()) & 15u) == 0;
+  for (int i = 0; i < 3; ++i) ok = ok && x.stride(i) >= 0 && x.stride(i) % 8 == 0;
+  ok = ok && x.stride(2) >= x.size(3) && x.stride(2) < (int64_t(1) << 24);
+  r.t = ok ? x : x.contiguous();
+  r.bh = x.size(0) * x.size(1);
+  r.s = x.size(2);
+  r.d = x.size(3);
+  r.heads = static_cast<int32_t>(x.size(1));
+  for (int i = 0; i < 3; ++i) r.st[i] = r.t.stride(i);
+  return r;
+}
+
+// A new tensor of x's shape with x's order of dimensions in memory, but dense: a [B,H,S,D] view of
+// [B,S,H,D] memory (or of a slice of a packed projection) gets fresh [B,S,H,D] memory.
+at::Tensor empty_like_rows(const at::Tensor &x) {
+  if (x.dim() != 4) return at::empty(x.sizes(), x.options());
+  std::vector<int64_t> order{0, 1, 2, 3};
+  std::stable_sort(order.begin(), order.end(), [&](int64_t a, int64_t b) { return x.stride(a) > x.stride(b); });
+  std::vector<int64_t> sizes(4), inv(4);
+  for (int i = 0; i < 4; ++i) {
+    sizes[i] = x.size(order[i]);
+    inv[order[i]] = i;
+  }
+  return at::empty(sizes, x.options()).permute(inv);
+}
+
+void set_stride(int64_t (&dst)[3], const RowsOf &r) {
+  for (int i = 0; i < 3; ++i) dst[i] = r.st[i];
+}
+
+void check_rows(const RowsOf &q, const RowsOf &k, const RowsOf &v) {
+  TORCH_CHECK(q.t.scalar_type() == k.t.scalar_type() && q.t.scalar_type() == v.t.scalar_type(),
+              "mha_manual: q/k/v must share one dtype");
+  TORCH_CHECK(q.heads == k.heads && q.heads == v.heads, "mha_manual: q/k/v must be all 3-d or all 4-d with one H");
+  TORCH_CHECK(k.bh == q.bh && v.bh == q.bh && k.d == q.d && v.d == q.d && v.s == k.s,
+              "mha_manual: shapes must be q [..,Sq,D], k [..,Sk,D], v [..,Sk,D] over the same heads");
+  TORCH_CHECK(k.t.device() == q.t.device() && v.t.device() == q.t.device(), "mha_manual: q/k/v on different devices");
+}
+
 // Optional valid key counts: an int32 vector of B entries on q's device, B dividing BH.
-template <typename P> void set_kv_len(P &p, const c10::optional<at::Tensor> &kv_len, const at::Tensor &q,
-                                      at::Tensor &keep) {
+template <typename P> void set_kv_len(P &p, const c10::optional<at::Tensor> &kv_len, int64_t bh, at::Tensor &keep) {
   if (!kv_len.has_value() || !kv_len->defined()) return;
   TORCH_CHECK(kv_len->is_cuda() && kv_len->scalar_type() == at::kInt && kv_len->dim() == 1 && kv_len->numel() > 0 &&
-                  q.size(0) % kv_len->numel() == 0,
+                  bh % kv_len->numel() == 0,
               "mha_manual: kv_len must be an int32 GPU vector whose length divides BH");
   keep = kv_len->contiguous();
   p.kv_len = keep.data_ptr<int32_t>();
-  p.kv_len_bh_div = static_cast<int32_t>(q.size(0) / keep.numel());
+  p.kv_len_bh_div = static_cast<int32_t>(bh / keep.numel());
 }
 
-// scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
-// (seed, offset); p_drop == 0 disables dropout.  Returns (O, LSE[bh,sq] fp32).
-std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
-                                            const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
-                                            double p_drop, int64_t seed, int64_t offset,
-                                            const c10::optional<at::Tensor> &kv_len) {
-  check_qkv(q, k, v);
-  at::DeviceGuard guard(q.device());
-  at::Tensor o = at::empty_like(q);
-  at::Tensor lse = at::empty({q.size(0), q.size(1)}, q.options().dtype(at::kFloat));
-  fmha_fwd_params p = {};
-  fill_common(p, q, k, v, o, scale > 0 ? scale : default_scale(q));
-  p.lse = lse.data_ptr<float>();
-  p.causal = is_causal ? 1 : 0;
-  MaskLayout m;
+template <typename P>
+void set_mask_and_dropout(P &p, MaskLayout &m, const c10::optional<at::Tensor> &mask, const RowsOf &q, int64_t sk,
+                          double p_drop, int64_t seed, int64_t offset) {
   if (mask.has_value() && mask->defined()) {
-    m = mask_layout(*mask, q, k.size(1), "mask");
+    m = mask_layout(*mask, q.t, q.bh, q.s, sk, "mask");
     p.mask = m.t.data_ptr();
     p.mask_kind = FMHA_MASK_ADDITIVE;
     p.mask_bh_div = m.bh_div;
@@ -221,66 +268,102 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q, const at::Tenso
     p.seed = static_cast<uint64_t>(seed);
     p.offset = static_cast<uint64_t>(offset);
   }
+}
+
+// q, k, v: [B*H,S,D] contiguous (the reference's layout) or [B,H,S,D] views of any batch / head /
+// row strides (e.g. x.view(B,S,H,D).transpose(1,2), or a slice of a packed QKV projection), read
+// in place.  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
+// (seed, offset); p_drop == 0 disables dropout.  Returns (O, LSE fp32): O in q's shape and
+// dimension order, LSE [B*H,Sq] or [B,H,Sq].
+std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,
+                                            const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
+                                            double p_drop, int64_t seed, int64_t offset,
+                                            const c10::optional<at::Tensor> &kv_len) {
+  const RowsOf q = rows_of(q_, "q"), k = rows_of(k_, "k"), v = rows_of(v_, "v");
+  check_rows(q, k, v);
+  at::DeviceGuard guard(q.t.device());
+  at::Tensor o = empty_like_rows(q.t);
+  const RowsOf orow = rows_of(o, "o");
+  at::Tensor lse = q.heads ? at::empty({q_.size(0), q_.size(1), q.s}, q.t.options().dtype(at::kFloat))
+                           : at::empty({q.bh, q.s}, q.t.options().dtype(at::kFloat));
+  fmha_fwd_params p = {};
+  p.q = q.t.data_ptr();
+  p.k = k.t.data_ptr();
+  p.v = v.t.data_ptr();
+  p.o = o.data_ptr();
+  p.bh = static_cast<int32_t>(q.bh);
+  p.sq = static_cast<int32_t>(q.s);
+  p.sk = static_cast<int32_t>(k.s);
+  p.d = static_cast<int32_t>(q.d);
+  p.dtype = dtype_code(q.t);
+  p.scale = static_cast<float>(scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(q.d)));
+  p.heads = q.heads;
+  set_stride(p.q_stride, q);
+  set_stride(p.k_stride, k);
+  set_stride(p.v_stride, v);
+  set_stride(p.o_stride, orow);
+  p.lse = lse.data_ptr<float>();
+  p.causal = is_causal ? 1 : 0;
+  MaskLayout m;
+  set_mask_and_dropout(p, m, mask, q, k.s, p_drop, seed, offset);
   at::Tensor kv_keep;
-  set_kv_len(p, kv_len, q, kv_keep);
-  launch_fwd(p, q);
+  set_kv_len(p, kv_len, q.bh, kv_keep);
+  launch_fwd(p, q.t);
   return std::make_tuple(o, lse);
 }
 
+// Gradients of fmha_fwd's inputs; tensors as there (dout and o in q's shape, any strides), lse as
+// fmha_fwd returned it.  dq, dk, dv come back in the dimension order of q, k, v.
 std::tuple<at::Tensor, at::Tensor, at::Tensor>
-fmha_bwd(const at::Tensor &dout, const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
-         const at::Tensor &o, const at::Tensor &lse, const c10::optional<at::Tensor> &mask, double scale,
+fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,
+         const at::Tensor &o_, const at::Tensor &lse, const c10::optional<at::Tensor> &mask, double scale,
          bool is_causal, double p_drop, int64_t seed, int64_t offset, const c10::optional<at::Tensor> &kv_len) {
-  check_qkv(q, k, v);
-  at::DeviceGuard guard(q.device());
-  TORCH_CHECK(dout.is_cuda() && o.is_cuda() && lse.is_cuda(), "mha_manual: dout/o/lse must live on the GPU");
-  TORCH_CHECK(dout.sizes() == q.sizes() && o.sizes() == q.sizes() && dout.scalar_type() == q.scalar_type() &&
-                  o.scalar_type() == q.scalar_type(),
+  const RowsOf q = rows_of(q_, "q"), k = rows_of(k_, "k"), v = rows_of(v_, "v");
+  check_rows(q, k, v);
+  at::DeviceGuard guard(q.t.device());
+  TORCH_CHECK(dout_.sizes() == q_.sizes() && o_.sizes() == q_.sizes() && dout_.scalar_type() == q.t.scalar_type() &&
+                  o_.scalar_type() == q.t.scalar_type(),
               "mha_manual: dout and o must match q in shape and dtype");
-  TORCH_CHECK(lse.scalar_type() == at::kFloat && lse.dim() == 2 && lse.size(0) == q.size(0) &&
-                  lse.size(1) == q.size(1),
-              "mha_manual: lse must be float32 [BH,Sq]");
-  at::Tensor doutc = dout.contiguous(), oc = o.contiguous(), lsec = lse.contiguous();
-  at::Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v);
+  const RowsOf dout = rows_of(dout_, "dout"), o = rows_of(o_, "o");
+  TORCH_CHECK(lse.is_cuda() && lse.scalar_type() == at::kFloat && lse.numel() == q.bh * q.s &&
+                  lse.size(-1) == q.s,
+              "mha_manual: lse must be float32 [BH,Sq] or [B,H,Sq]");
+  at::Tensor lsec = lse.contiguous();
+  at::Tensor dq = empty_like_rows(q.t), dk = empty_like_rows(k.t), dv = empty_like_rows(v.t);
+  const RowsOf dqr = rows_of(dq, "dq"), dkr = rows_of(dk, "dk"), dvr = rows_of(dv, "dv");
   at::Tensor delta = at::empty_like(lsec);
   fmha_bwd_params p = {};
-  p.q = q.data_ptr();
-  p.k = k.data_ptr();
-  p.v = v.data_ptr();
-  p.o = oc.data_ptr();
-  p.dout = doutc.data_ptr();
+  p.q = q.t.data_ptr();
+  p.k = k.t.data_ptr();
+  p.v = v.t.data_ptr();
+  p.o = o.t.data_ptr();
+  p.dout = dout.t.data_ptr();
   p.lse = lsec.data_ptr<float>();
   p.delta = delta.data_ptr<float>();
   p.dq = dq.data_ptr();
   p.dk = dk.data_ptr();
   p.dv = dv.data_ptr();
-  p.bh = static_cast<int32_t>(q.size(0));
-  p.sq = static_cast<int32_t>(q.size(1));
-  p.sk = static_cast<int32_t>(k.size(1));
-  p.d = static_cast<int32_t>(q.size(2));
-  p.dtype = dtype_code(q);
-  p.scale = static_cast<float>(scale > 0 ? scale : default_scale(q));
+  p.bh = static_cast<int32_t>(q.bh);
+  p.sq = static_cast<int32_t>(q.s);
+  p.sk = static_cast<int32_t>(k.s);
+  p.d = static_cast<int32_t>(q.d);
+  p.dtype = dtype_code(q.t);
+  p.scale = static_cast<float>(scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(q.d)));
   p.causal = is_causal ? 1 : 0;
+  p.heads = q.heads;
+  set_stride(p.q_stride, q);
+  set_stride(p.k_stride, k);
+  set_stride(p.v_stride, v);
+  set_stride(p.o_stride, o);
+  set_stride(p.do_stride, dout);
+  set_stride(p.dq_stride, dqr);
+  set_stride(p.dk_stride, dkr);
+  set_stride(p.dv_stride, dvr);
   MaskLayout m;
-  if (mask.has_value() && mask->defined()) {
-    m = mask_layout(*mask, q, k.size(1), "mask");
-    p.mask = m.t.data_ptr();
-    p.mask_kind = FMHA_MASK_ADDITIVE;
-    p.mask_bh_div = m.bh_div;
-    p.mask_stride_b = m.stride_b;
-    p.mask_stride_q = m.stride_q;
-  }
-  TORCH_CHECK(p_drop >= 0.0 && p_drop < 1.0, "mha_manual: p_drop must be in [0,1)");
-  if (p_drop > 0.0) {
-    p.drop_kind = FMHA_DROP_PHILOX;
-    p.p_drop = static_cast<float>(p_drop);
-    p.drop_scale = static_cast<float>(1.0 / (1.0 - p_drop));
-    p.seed = static_cast<uint64_t>(seed);
-    p.offset = static_cast<uint64_t>(offset);
-  }
+  set_mask_and_dropout(p, m, mask, q, k.s, p_drop, seed, offset);
   at::Tensor kv_keep;
-  set_kv_len(p, kv_len, q, kv_keep);
-  const int rc = fmha_bwd_launch(&p, current_stream(q));
+  set_kv_len(p, kv_len, q.bh, kv_keep);
+  const int rc = fmha_bwd_launch(&p, current_stream(q.t));
   TORCH_CHECK(rc == FMHA_OK, "mha_manual backward: ", fmha_strerror(rc));
   return std::make_tuple(dq, dk, dv);
 }

@@ -110,6 +110,18 @@ typedef struct fmha_fwd_params {
    * the kernel ran, which on a power-limited board is well below the maximum clock that the
    * published MFMA peak assumes.  Left untouched by the non-pipelined kernel. */
   uint64_t *clock_probe;
+
+  /* Optional row layout of q, k, v and o (no counterpart in the reference: its operators take
+   * folded, contiguous [bh, s, d] tensors and its perf scripts exclude the permute that produces
+   * them, perf_measurement.py:52).  heads == 0: that layout, strides ignored.  heads = H > 0:
+   * bh = B*H, head index i means (batch i / H, head i % H), and row r of that head of tensor x
+   * starts at element (i / H) * x_stride[0] + (i % H) * x_stride[1] + r * x_stride[2]; rows are d
+   * contiguous elements.  Every stride must be a non-negative multiple of 8 elements, stride[2]
+   * at least d and below 2^24, and k and v must share stride[2].  E.g. a [B, s, H, d] tensor:
+   * {s*H*d, d, H*d}; the q part of a packed [B, s, 3, H, d] tensor: {s*3*H*d, d, 3*H*d}.
+   * lse (and delta) stay [bh, sq] contiguous.  Outputs must not overlap inputs. */
+  int32_t heads;
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];
 } fmha_fwd_params;
 
 /* Enqueue the forward kernel on `hip_stream` (a hipStream_t; NULL = default stream). */
@@ -149,6 +161,11 @@ typedef struct fmha_bwd_params {
 
   const int32_t *kv_len; /* as in fmha_fwd_params; dk and dv rows at or past the count are zero */
   int32_t kv_len_bh_div;
+
+  /* Optional row layouts, as in fmha_fwd_params, of q, k, v, o, dout and of the outputs dq, dk, dv. */
+  int32_t heads;
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3], do_stride[3];
+  int64_t dq_stride[3], dk_stride[3], dv_stride[3];
 } fmha_bwd_params;
 
 int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);

@@ -40,10 +40,10 @@ def _tus():
     tus = [("fmha_capi.hip", "fmha_capi.o", [])]
     for bf in (0, 1):
         for d in (64, 128):
-            tag = f"{'bf16' if bf else 'f16'}_d{d}"
-            defs = [f"-DFMHA_TU_BF16={bf}", f"-DFMHA_TU_D={d}"]
-            tus.append(("fmha_fwd.hip", f"fmha_fwd_{tag}.o", defs))
-            if os.path.exists(os.path.join(CSRC, "fmha_bwd.hip")):
+            for strided in (0, 1):  # folded contiguous tensors / row layouts given at run time
+                tag = f"{'bf16' if bf else 'f16'}_d{d}" + ("_strided" if strided else "")
+                defs = [f"-DFMHA_TU_BF16={bf}", f"-DFMHA_TU_D={d}", f"-DFMHA_TU_STRIDED={strided}"]
+                tus.append(("fmha_fwd.hip", f"fmha_fwd_{tag}.o", defs))
                 tus.append(("fmha_bwd.hip", f"fmha_bwd_{tag}.o", defs))
     return tus
 

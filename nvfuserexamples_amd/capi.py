@@ -31,6 +31,9 @@ class FwdParams(C.Structure):
         ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
         ("kv_len", C.c_void_p), ("kv_len_bh_div", C.c_int32),
         ("clock_probe", C.c_void_p),
+        ("heads", C.c_int32),
+        ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
+        ("o_stride", C.c_int64 * 3),
     ]
 
 
@@ -47,6 +50,10 @@ class BwdParams(C.Structure):
         ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
         ("dtype", C.c_int32), ("scale", C.c_float), ("flags", C.c_int32),
         ("kv_len", C.c_void_p), ("kv_len_bh_div", C.c_int32),
+        ("heads", C.c_int32),
+        ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
+        ("o_stride", C.c_int64 * 3), ("do_stride", C.c_int64 * 3),
+        ("dq_stride", C.c_int64 * 3), ("dk_stride", C.c_int64 * 3), ("dv_stride", C.c_int64 * 3),
     ]
 
 
@@ -127,23 +134,69 @@ def _set_kv_len(P, kv_len, bh):
     P.kv_len, P.kv_len_bh_div = kv_len.data_ptr(), bh // kv_len.numel()
 
 
+def _rows(t, name):
+    """(bh, rows, d, heads, strides) of a [bh, rows, d] contiguous or a [B, H, rows, d] strided tensor."""
+    if t.dim() == 3:
+        if not t.is_contiguous():
+            raise FmhaError(-5, f"{name}: 3-d tensors must be contiguous [bh, s, d]; pass a 4-d [B, H, s, d] view for other layouts")
+        return t.shape[0], t.shape[1], t.shape[2], 0, (0, 0, 0)
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise FmhaError(-5, f"{name} must be [bh, s, d] or [B, H, s, d] with contiguous rows")
+    return t.shape[0] * t.shape[1], t.shape[2], t.shape[3], t.shape[1], (t.stride(0), t.stride(1), t.stride(2))
+
+
+def empty_like_rows(t):
+    """New tensor of t's shape whose dimensions are laid out in t's order but densely (a slice
+    of a packed [B, s, 3, H, d] tensor gives a [B, H, s, d] view of fresh [B, s, H, d] memory)."""
+    import torch
+    if t.dim() == 3:
+        return torch.empty_like(t)
+    order = sorted(range(4), key=lambda i: (-t.stride(i), i))
+    base = torch.empty([t.shape[i] for i in order], dtype=t.dtype, device=t.device)
+    inv = [order.index(i) for i in range(4)]
+    return base.permute(inv)
+
+
+def _set_rows(P, heads, **tensors):
+    """Fill P.heads and P.<name>_stride; all tensors must agree on 3-d (folded) or 4-d with one H."""
+    hs = {h for _, h, _ in tensors.values()}
+    if len(hs) != 1:
+        raise FmhaError(-5, "tensors must be all [bh, s, d] or all [B, H, s, d] with the same H")
+    P.heads = heads
+    for name, (_, _, st) in tensors.items():
+        arr = getattr(P, name + "_stride")
+        for i in range(3):
+            arr[i] = st[i]
+
+
 def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False, scale=None,
         drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
         want_lse=False, save=False, flags=0, out=None, kv_len=None):
     """Launch the forward on the current stream.  Returns (o, lse|None, softmax|None, dropout|None).
 
     kv_len: optional int32 device tensor of B valid key counts (bh must be a multiple of B); head i
-    attends keys [0, kv_len[i // (bh // B)]) only."""
+    attends keys [0, kv_len[i // (bh // B)]) only.
+
+    q, k, v: contiguous [bh, s, d] (the reference's layout), or 4-d [B, H, s, d] tensors with
+    arbitrary batch / head / row strides (multiples of 8 elements; rows contiguous), e.g.
+    ``x.view(B, s, H, d).transpose(1, 2)`` or a slice of a packed QKV projection: no copy is made.
+    o then comes back as [B, H, sq, d] in q's dimension order and lse as [B, H, sq]."""
     import torch
-    bh, sq, d = q.shape
-    sk = k.shape[1]
+    bh, sq, d, heads, qs = _rows(q, "q")
+    bhk, sk, dk_, hk, ks = _rows(k, "k")
+    bhv, skv, dv_, hv, vs = _rows(v, "v")
+    if (bhk, dk_, bhv, skv, dv_) != (bh, d, bh, sk, d):
+        raise FmhaError(-3, "q/k/v shapes do not agree")
     P = FwdParams()
     P.dtype = _dtype_code(q)
     for t in (q, k, v):
-        if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype):
-            raise FmhaError(-5, "q/k/v must be contiguous device tensors of one dtype")
-    o = out if out is not None else torch.empty_like(q)
-    lse = torch.empty((bh, sq), dtype=torch.float32, device=q.device) if want_lse else None
+        if not (t.is_cuda and t.dtype == q.dtype):
+            raise FmhaError(-5, "q/k/v must be device tensors of one dtype")
+    o = out if out is not None else empty_like_rows(q)
+    _, _, _, ho, os_ = _rows(o, "out")
+    _set_rows(P, heads, q=(0, heads, qs), k=(0, hk, ks), v=(0, hv, vs), o=(0, ho, os_))
+    lse = torch.empty((bh, sq) if heads == 0 else (q.shape[0], heads, sq), dtype=torch.float32,
+                      device=q.device) if want_lse else None
     P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
     P.lse = lse.data_ptr() if lse is not None else None
     P.bh, P.sq, P.sk, P.d = bh, sq, sk, d
@@ -180,18 +233,28 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
 def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False,
         scale=None, drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
         flags=0, delta=None, grads=None, kv_len=None):
-    """Launch the backward on the current stream.  Returns (dq, dk, dv).  kv_len as in fwd()."""
+    """Launch the backward on the current stream.  Returns (dq, dk, dv).  kv_len and the tensor
+    layouts as in fwd(); each gradient comes back in its input's dimension order."""
     import torch
-    bh, sq, d = q.shape
-    sk = k.shape[1]
+    bh, sq, d, heads, qs = _rows(q, "q")
+    _, sk, _, hk, ks = _rows(k, "k")
+    _, _, _, hv, vs = _rows(v, "v")
+    _, _, _, ho, os_ = _rows(o, "o")
+    _, _, _, hd, ds_ = _rows(dout, "dout")
+    if not (k.shape == v.shape and o.shape == q.shape and dout.shape == q.shape and k.shape[-1] == d):
+        raise FmhaError(-3, "q/k/v/o/dout shapes do not agree")
     P = BwdParams()
     P.dtype = _dtype_code(q)
     for t in (q, k, v, o, dout):
-        if not (t.is_cuda and t.is_contiguous() and t.dtype == q.dtype):
-            raise FmhaError(-5, "q/k/v/o/dout must be contiguous device tensors of one dtype")
+        if not (t.is_cuda and t.dtype == q.dtype):
+            raise FmhaError(-5, "q/k/v/o/dout must be device tensors of one dtype")
     if delta is None:
         delta = torch.empty((bh, sq), dtype=torch.float32, device=q.device)
-    dq, dk, dv = grads if grads is not None else (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    if not lse.is_contiguous():
+        raise FmhaError(-5, "lse must be contiguous")
+    dq, dk, dv = grads if grads is not None else (empty_like_rows(q), empty_like_rows(k), empty_like_rows(v))
+    _set_rows(P, heads, q=(0, heads, qs), k=(0, hk, ks), v=(0, hv, vs), o=(0, ho, os_), do=(0, hd, ds_),
+              dq=(0,) + _rows(dq, "dq")[3:], dk=(0,) + _rows(dk, "dk")[3:], dv=(0,) + _rows(dv, "dv")[3:])
     P.q, P.k, P.v, P.o, P.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), dout.data_ptr()
     P.lse, P.delta = lse.data_ptr(), delta.data_ptr()
     P.dq, P.dk, P.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()

@@ -1,5 +1,5 @@
-// Instantiates the backward kernels for one (element type, head dim) pair, chosen with
-// -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128}, and exports their dispatcher.
+// Instantiates the backward kernels for one (element type, head dim, row layout kind) triple, chosen
+// with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1}, and exports their dispatcher.
 #include "fmha_launch.h"
 
 #if FMHA_TU_BF16
@@ -9,7 +9,14 @@
 #define FMHA_TU_T _Float16
 #define FMHA_TU_TNAME f16
 #endif
+#ifndef FMHA_TU_STRIDED
+#define FMHA_TU_STRIDED 0
+#endif
+#if FMHA_TU_STRIDED
+#define FMHA_CAT3(a, b, c) a##b##_d##c##_strided
+#else
 #define FMHA_CAT3(a, b, c) a##b##_d##c
+#endif
 #define FMHA_NAME(t, d) FMHA_CAT3(bwd_dispatch_, t, d)
 
 namespace fmha {
@@ -18,6 +25,7 @@ namespace {
 constexpr int kNW = 4;
 constexpr int kQB = 1; // 32-query blocks per wave in the dQ kernel
 constexpr int kKB = 1; // 32-key blocks per wave in the dK/dV kernel
+constexpr bool kStrided = FMHA_TU_STRIDED != 0;
 
 template <typename K> int set_lds(K kern, int bytes) {
   return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -27,8 +35,8 @@ template <typename K> int set_lds(K kern, int bytes) {
 template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipStream_t s) {
   constexpr int kLdsQ = BwdCfg<FMHA_TU_D, bwd_dq_tile_rows<FMHA_TU_D>()>::LDS_BYTES;
   constexpr int kLdsK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>::LDS_BYTES;
-  auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP>;
-  auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP>;
+  auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP, kStrided>;
+  auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP, kStrided>;
   static const int attr = set_lds(kq, kLdsQ) | set_lds(kk, kLdsK);
   if (attr) return 2;
   constexpr int QT = kNW * kQB * 32, KT = kNW * kKB * 32;

@@ -52,6 +52,7 @@ struct BwdArgs {
   int32_t flags;
   const int32_t *kv_len; // optional valid key count per group of kv_div heads
   int32_t kv_div;
+  RowMap mq, mk, mv, mo, mdo, mdq, mdk, mdv; // row layouts (mk.ss == mv.ss)
 };
 
 // BT: rows per LDS tile (keys in the dQ kernel, queries in the dK/dV kernel).  The dK/dV kernel
@@ -96,9 +97,10 @@ template <typename T> FMHA_DEV void split_hi_lo(float v, T &hi, T &lo) {
 // ------------------------------------------------------------------------------ dQ
 // (At head dim 128 some variants need a few registers more than a two-waves-per-SIMD budget:
 // spill those few rather than drop to one wave per SIMD, +10 % measured.)
-template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
+template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED>
 __global__ __launch_bounds__(NW * 64)
     __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 1, 2))) void fmha_bwd_dq_kernel(const BwdArgs a) {
+  using RW = Rows<STRIDED, D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -132,11 +134,11 @@ __global__ __launch_bounds__(NW * 64)
   const int qt = CAUSAL ? (pass == 0 ? a.ntile - 1 - pi : pi) : pi;
   const int q0w = qt * QT + w * (QB * 32);
 
-  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
-  const T *Ob = (const T *)a.o + (size_t)bh * a.sq * D;
-  const T *dOb = (const T *)a.dout + (size_t)bh * a.sq * D;
-  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
-  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+  const T *Qb = (const T *)a.q + RW::head(a.mq, bh, a.sq);
+  const T *Ob = (const T *)a.o + RW::head(a.mo, bh, a.sq);
+  const T *dOb = (const T *)a.dout + RW::head(a.mdo, bh, a.sq);
+  const T *Kb = (const T *)a.k + RW::head(a.mk, bh, a.sk);
+  const T *Vb = (const T *)a.v + RW::head(a.mv, bh, a.sk);
   const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
   // ---- per-row operands: Q' and dO as B operands, the extra-step columns, delta
@@ -151,10 +153,10 @@ __global__ __launch_bounds__(NW * 64)
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 tq = {0u, 0u, 0u, 0u}, td = {0u, 0u, 0u, 0u}, to = {0u, 0u, 0u, 0u};
       if (q < a.sq) {
-        const size_t off = (size_t)q * D + ks * 16 + h * 8;
-        tq = *(const u32x4 *)(Qb + off);
-        td = *(const u32x4 *)(dOb + off);
-        to = *(const u32x4 *)(Ob + off);
+        const size_t col = ks * 16 + h * 8;
+        tq = *(const u32x4 *)(Qb + (size_t)q * RW::ss(a.mq) + col);
+        td = *(const u32x4 *)(dOb + (size_t)q * RW::ss(a.mdo) + col);
+        to = *(const u32x4 *)(Ob + (size_t)q * RW::ss(a.mo) + col);
       }
       const v8 qraw = as_v8<T>(tq);
       const v8 doraw = as_v8<T>(td);
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(NW * 64)
   PanelLane pl;
   pl.init(l);
   TileCopy<T, D, BK, NT> tcopy;
-  tcopy.init(tid);
+  tcopy.init(tid, RW::ss(a.mk)); // K and V rows are equally far apart
   auto dma_kv = [&](int kt) {
     const uint32_t dst = lds_base + (uint32_t)(kt & 1) * 2 * TILEB;
     tcopy.issue(Kb, kt * BK, kclamp, dst, tid);
@@ -386,13 +388,13 @@ __global__ __launch_bounds__(NW * 64)
     __syncthreads();
   }
 
-  T *dQb = (T *)a.dq + (size_t)bh * a.sq * D;
+  T *dQb = (T *)a.dq + RW::head(a.mdq, bh, a.sq);
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int q = q0w + qb * 32 + ql;
     if (q < a.sq) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQb + (size_t)q * D + db * 32, dq[qb][db], a.scale, h);
+      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQb + (size_t)q * RW::ss(a.mdq) + db * 32, dq[qb][db], a.scale, h);
     }
   }
   __syncthreads(); // the next pass refills the tiles
@@ -400,9 +402,10 @@ __global__ __launch_bounds__(NW * 64)
 }
 
 // --------------------------------------------------------------------------- dK, dV
-template <typename T, int D, int KB, int NW, int MASK, bool CAUSAL, int DROP>
+template <typename T, int D, int KB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED>
 __global__ __launch_bounds__(NW * 64)
     __attribute__((amdgpu_waves_per_eu(bwd_dkdv_small_tiles<D, CAUSAL, DROP>() ? 2 : 1, 2))) void fmha_bwd_dkdv_kernel(const BwdArgs a) {
+  using RW = Rows<STRIDED, D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -436,10 +439,10 @@ __global__ __launch_bounds__(NW * 64)
   const int ktile = pass == 0 ? pi : a.ntile - 1 - pi;
   const int k0w = ktile * KT + w * (KB * 32);
 
-  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
-  const T *dOb = (const T *)a.dout + (size_t)bh * a.sq * D;
-  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
-  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+  const T *Qb = (const T *)a.q + RW::head(a.mq, bh, a.sq);
+  const T *dOb = (const T *)a.dout + RW::head(a.mdo, bh, a.sq);
+  const T *Kb = (const T *)a.k + RW::head(a.mk, bh, a.sk);
+  const T *Vb = (const T *)a.v + RW::head(a.mv, bh, a.sk);
   const float *lseb = a.lse + (size_t)bh * a.sq;
   const float *delb = a.delta + (size_t)bh * a.sq;
 
@@ -454,9 +457,9 @@ __global__ __launch_bounds__(NW * 64)
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 tk = {0u, 0u, 0u, 0u}, tv = {0u, 0u, 0u, 0u};
       if (key < skv) {
-        const size_t off = (size_t)key * D + ks * 16 + h * 8;
-        tk = *(const u32x4 *)(Kb + off);
-        tv = *(const u32x4 *)(Vb + off);
+        const size_t col = ks * 16 + h * 8;
+        tk = *(const u32x4 *)(Kb + (size_t)key * RW::ss(a.mk) + col);
+        tv = *(const u32x4 *)(Vb + (size_t)key * RW::ss(a.mv) + col);
       }
       const v8 kraw = as_v8<T>(tk);
       const v8 vraw = as_v8<T>(tv);
@@ -503,12 +506,13 @@ __global__ __launch_bounds__(NW * 64)
   const uint32_t lds_base = lds_address(lds);
   PanelLane pl;
   pl.init(l);
-  TileCopy<T, D, BQ, NT> tcopy;
-  tcopy.init(tid);
+  TileCopy<T, D, BQ, NT> tcopy, tcopy_do; // Q and dO rows need not be equally far apart
+  tcopy.init(tid, RW::ss(a.mq));
+  tcopy_do.init(tid, RW::ss(a.mdo));
   auto dma_qdo = [&](int qt) {
     const uint32_t dst = lds_base + (uint32_t)(qt & 1) * 2 * TILEB;
     tcopy.issue(Qb, qt * BQ, a.sq, dst, tid);
-    tcopy.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid);
+    tcopy_do.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid);
   };
   float lraw = 0.f, draw = 0.f;
   bool qvalid = false;
@@ -691,16 +695,16 @@ __global__ __launch_bounds__(NW * 64)
     __syncthreads();
   }
 
-  T *dKb = (T *)a.dk + (size_t)bh * a.sk * D;
-  T *dVb = (T *)a.dv + (size_t)bh * a.sk * D;
+  T *dKb = (T *)a.dk + RW::head(a.mdk, bh, a.sk);
+  T *dVb = (T *)a.dv + RW::head(a.mdv, bh, a.sk);
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     const int key = k0w + kb * 32 + kl;
     if (key < a.sk) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        store_acc_block_row<T>(dKb + (size_t)key * D + db * 32, dk[kb][db], a.scale, h);
-        store_acc_block_row<T>(dVb + (size_t)key * D + db * 32, dv[kb][db], 1.f, h);
+        store_acc_block_row<T>(dKb + (size_t)key * RW::ss(a.mdk) + db * 32, dk[kb][db], a.scale, h);
+        store_acc_block_row<T>(dVb + (size_t)key * RW::ss(a.mdv) + db * 32, dv[kb][db], 1.f, h);
       }
     }
   }

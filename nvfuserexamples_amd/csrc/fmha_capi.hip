@@ -63,10 +63,10 @@ const char *fmha_strerror(int code) {
   case FMHA_OK: return "ok";
   case FMHA_E_NULL: return "a required pointer is NULL";
   case FMHA_E_DTYPE: return "unknown dtype (0 = fp16, 1 = bf16)";
-  case FMHA_E_SHAPE: return "bad shape: sizes must be positive and head dim must be 64 or 128";
-  case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned";
+  case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64 or 128, and one head's rows must span less than 2^31 elements";
+  case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned and their strides multiples of 8 elements";
   case FMHA_E_ARG: return "argument out of range (scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
-  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox; the backward takes Philox dropout only)";
+  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox; the backward takes Philox dropout only; k and v rows must be equally far apart)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
   default: return "unknown error code";
   }
@@ -88,6 +88,36 @@ int fmha_philox_keep_mask(uint64_t seed, uint64_t offset, float p_drop, int32_t 
                      sq, sk, total, out);
   return hipGetLastError() == hipSuccess ? FMHA_OK : FMHA_E_LAUNCH;
 }
+
+} // extern "C"
+
+// Row layout of one tensor from the caller's (heads, strides); see fmha_capi.h.  `strided` is
+// set when the layout is not the folded contiguous one (it is never cleared).
+static int make_row_map(RowMap &m, int32_t heads, const int64_t st[3], int32_t bh, int32_t rows, int32_t d,
+                        bool &strided) {
+  m.heads_rcp = 0;
+  if (heads == 0) {
+    m.sb = (int64_t)rows * d;
+    m.sh = 0;
+    m.ss = d;
+    m.heads = 1;
+    return (int64_t)rows * d < (1ll << 31) ? FMHA_OK : FMHA_E_SHAPE; // offsets inside a head are 31-bit
+  }
+  if (heads < 0 || bh % heads != 0) return FMHA_E_ARG;
+  for (int i = 0; i < 3; ++i)
+    if (st[i] < 0 || (st[i] & 7) != 0) return FMHA_E_ALIGN;
+  if (st[2] < d || st[2] >= (1ll << 24)) return FMHA_E_ARG;
+  if ((int64_t)(rows - 1) * st[2] + d >= (1ll << 31) || (int64_t)bh * heads >= (1ll << 32)) return FMHA_E_SHAPE;
+  m.heads_rcp = (uint32_t)((1ull << 32) / (uint64_t)heads) + 1u; // unused when heads == 1
+  m.sb = st[0];
+  m.sh = st[1];
+  m.ss = st[2];
+  m.heads = heads;
+  if (!(st[2] == d && st[1] == (int64_t)rows * d && st[0] == (int64_t)heads * rows * d)) strided = true;
+  return FMHA_OK;
+}
+
+extern "C" {
 
 int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   if (!p || !p->q || !p->k || !p->v || !p->o) return FMHA_E_NULL;
@@ -147,18 +177,27 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
   a.clock_probe = (unsigned long long *)p->clock_probe;
+  int mrc;
+  bool strided = false;
+  if ((mrc = make_row_map(a.mq, p->heads, p->q_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mk, p->heads, p->k_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mv, p->heads, p->v_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mo, p->heads, p->o_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
+  if (strided && (saving || p->drop_kind == FMHA_DROP_TENSOR)) return FMHA_E_UNSUPPORTED;
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
-  // flop.  That pays (about 5 % measured) for the plain variants at head dim 64 on long key
+  // flop.  That pays (4-6 % measured) for the unmasked variant at head dim 64 on long key
   // ranges when there is enough work for every resident workgroup to get several 256-query
-  // items; with dropout, a causal or a full mask the per-element work dominates, and on short
-  // key ranges the longer per-item prologue does, so one block per wave is faster there.
+  // items; with dropout or any mask the per-element work dominates (a per-key mask measures
+  // 4-7 % slower with two blocks), and on short key ranges the longer per-item prologue does,
+  // so one block per wave is faster there.
   v.qb = 1;
-  if (p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull) {
+  if (p->d == 64 && !v.causal && v.drop == 0 && v.mask == kMaskNone) {
     static const int cus = [] {
       int dev = 0, n = 0;
       if (hipGetDevice(&dev) != hipSuccess ||
@@ -173,10 +212,16 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   }
   const int force = env_int("FMHA_FWD_QB", 0); // tuning override: 1 or 2
   if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;
+  if (strided) v.qb = 1; // the two-block variant is built for the folded layout only
 
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;
-  if (p->dtype == FMHA_DTYPE_F16)
+  if (strided) {
+    if (p->dtype == FMHA_DTYPE_F16)
+      rc = p->d == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : fwd_dispatch_f16_d128_strided(a, v, s);
+    else
+      rc = p->d == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : fwd_dispatch_bf16_d128_strided(a, v, s);
+  } else if (p->dtype == FMHA_DTYPE_F16)
     rc = p->d == 64 ? fwd_dispatch_f16_d64(a, v, s) : fwd_dispatch_f16_d128(a, v, s);
   else
     rc = p->d == 64 ? fwd_dispatch_bf16_d64(a, v, s) : fwd_dispatch_bf16_d128(a, v, s);
@@ -232,6 +277,17 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   a.flags = p->flags;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
+  int mrc;
+  bool strided = false;
+  if ((mrc = make_row_map(a.mq, p->heads, p->q_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mk, p->heads, p->k_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mv, p->heads, p->v_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mo, p->heads, p->o_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mdo, p->heads, p->do_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mdq, p->heads, p->dq_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mdk, p->heads, p->dk_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if ((mrc = make_row_map(a.mdv, p->heads, p->dv_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
 
   BwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
@@ -240,7 +296,12 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
   v.pair = env_int("FMHA_BWD_PAIR", -1); // tuning / test override: 0 or 1
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;
-  if (p->dtype == FMHA_DTYPE_F16)
+  if (strided) {
+    if (p->dtype == FMHA_DTYPE_F16)
+      rc = p->d == 64 ? bwd_dispatch_f16_d64_strided(a, v, s) : bwd_dispatch_f16_d128_strided(a, v, s);
+    else
+      rc = p->d == 64 ? bwd_dispatch_bf16_d64_strided(a, v, s) : bwd_dispatch_bf16_d128_strided(a, v, s);
+  } else if (p->dtype == FMHA_DTYPE_F16)
     rc = p->d == 64 ? bwd_dispatch_f16_d64(a, v, s) : bwd_dispatch_f16_d128(a, v, s);
   else
     rc = p->d == 64 ? bwd_dispatch_bf16_d64(a, v, s) : bwd_dispatch_bf16_d128(a, v, s);

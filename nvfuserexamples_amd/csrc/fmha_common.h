@@ -144,11 +144,41 @@ FMHA_DEV void dma_global_to_lds_b128(const void *uniform_base, uint32_t lane_off
 // Copies rows [row0, row0 + BT) of a row-major [rows][D] matrix into a swizzled tile; NT
 // threads take part.  Rows >= rend re-read row rend - 1 (callers neutralise them through
 // their extra-step rows).  The lane's byte offsets inside a tile are computed once (init).
+// Where the rows of head bh of a [heads..., rows, D] tensor live: head bh = (bh / heads, bh % heads)
+// starts at element (bh / heads) * sb + (bh % heads) * sh and its rows are ss elements apart
+// (D contiguous elements each).  The folded [B*H, rows, D] layout is heads = 1, sb = rows * D,
+// ss = D; a [B, rows, H, D] tensor is heads = H, sb = rows * H * D, sh = D, ss = H * D.
+// heads_rcp = floor(2^32 / heads) + 1 turns the division into a multiplication (exact while
+// bh * heads < 2^32, which the host checks); offsets inside one head fit 31 bits (also checked).
+struct RowMap {
+  int64_t sb, sh, ss;
+  int32_t heads;
+  uint32_t heads_rcp;
+  FMHA_DEV size_t head(int bh) const {
+    const uint32_t b = heads == 1 ? (uint32_t)bh : __umulhi((uint32_t)bh, heads_rcp);
+    return (size_t)b * (size_t)sb + (size_t)((uint32_t)bh - b * (uint32_t)heads) * (size_t)sh;
+  }
+};
+// Kernels are built twice: for the folded contiguous layout, whose strides are compile-time
+// constants (the row map is not read at all), and for row maps given at run time, which cost a
+// few per cent in scalar address arithmetic and registers.
+template <bool STRIDED, int D> struct Rows {
+  static FMHA_DEV size_t head(const RowMap &m, int bh, int rows) {
+    if constexpr (STRIDED) return m.head(bh);
+    else return (size_t)bh * (size_t)rows * D;
+  }
+  static FMHA_DEV uint32_t ss(const RowMap &m) {
+    if constexpr (STRIDED) return (uint32_t)m.ss;
+    else return (uint32_t)D;
+  }
+};
+
 template <typename T, int D, int BT, int NT> struct TileCopy {
   static constexpr int CHUNKS = BT * D / 8;
   static constexpr int CPT = CHUNKS / NT;
   static_assert(D % 64 == 0 && CHUNKS % NT == 0, "tile must divide evenly over the workgroup");
   uint32_t voff[CPT];
+  uint32_t ss; // elements between rows of the source tensor
 
   // chunk slot c of a tile: panel c / (8*BT), row (c / 8) % BT, position c % 8, which holds the
   // row's chunk panel*8 + (position ^ ((row >> 1) & 7))
@@ -157,19 +187,21 @@ template <typename T, int D, int BT, int NT> struct TileCopy {
     row = (c / 8) % BT;
     col = panel * 8 + (pos ^ ((row >> 1) & 7));
   }
-  FMHA_DEV void init(int tid) {
+  FMHA_DEV void init(int tid, int64_t row_stride) {
+    ss = (uint32_t)row_stride;
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       int row, col;
       slot(tid + i * NT, row, col);
-      voff[i] = (uint32_t)(row * D * 2 + col * 16);
+      voff[i] = (uint32_t)row * ss * 2u + (uint32_t)(col * 16);
     }
   }
-  // lds_tile: LDS byte address of the destination tile; tid: the caller's index among the NT threads
+  // base: row 0 of the head; lds_tile: LDS byte address of the destination tile; tid: the caller's
+  // index among the NT threads
   FMHA_DEV void issue(const T *base, int row0, int rend, uint32_t lds_tile, int tid) const {
     const uint32_t wave_dst = lds_tile + (uint32_t)(tid >> 6) * 1024u;
     if (row0 + BT <= rend) { // wave-uniform: a full tile needs no per-lane address arithmetic
-      const T *tb = base + (size_t)row0 * D;
+      const T *tb = base + (uint32_t)row0 * ss;
 #pragma unroll
       for (int i = 0; i < CPT; ++i) dma_global_to_lds_b128(tb, voff[i], wave_dst + (uint32_t)(i * NT * 16));
     } else {
@@ -179,7 +211,7 @@ template <typename T, int D, int BT, int NT> struct TileCopy {
         slot(tid + i * NT, row, col);
         int r = row0 + row;
         r = r < rend ? r : rend - 1;
-        dma_global_to_lds_b128(base + (size_t)r * D + col * 8, wave_dst + (uint32_t)(i * NT * 16));
+        dma_global_to_lds_b128(base + ((uint32_t)r * ss + (uint32_t)(col * 8)), wave_dst + (uint32_t)(i * NT * 16));
       }
     }
   }

@@ -1,5 +1,5 @@
-// Instantiates the forward kernel for one (element type, head dim) pair, chosen with
-// -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128}, and exports its dispatcher.
+// Instantiates the forward kernel for one (element type, head dim, row layout kind) triple, chosen
+// with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1}, and exports its dispatcher.
 #include "fmha_launch.h"
 #include "fmha_fwd_pipe.h"
 
@@ -10,7 +10,14 @@
 #define FMHA_TU_T _Float16
 #define FMHA_TU_TNAME f16
 #endif
+#ifndef FMHA_TU_STRIDED
+#define FMHA_TU_STRIDED 0
+#endif
+#if FMHA_TU_STRIDED
+#define FMHA_CAT3(a, b, c) a##b##_d##c##_strided
+#else
 #define FMHA_CAT3(a, b, c) a##b##_d##c
+#endif
 #define FMHA_NAME(t, d) FMHA_CAT3(fwd_dispatch_, t, d)
 
 namespace fmha {
@@ -20,6 +27,7 @@ namespace {
 #define FMHA_FWD_NW 4
 #endif
 constexpr int kNW = FMHA_FWD_NW;
+constexpr bool kStrided = FMHA_TU_STRIDED != 0;
 
 template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
   constexpr bool kPipe = DROP != 2;
@@ -27,7 +35,7 @@ template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStr
   // tensor dropout and the save pass run on the plain loop; everything else is software-pipelined
   auto kern = [] {
     if constexpr (DROP == 2) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
-    else return fmha_fwd_pipe_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+    else return fmha_fwd_pipe_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP, kStrided>;
   }();
   // once per kernel: allow the dynamic LDS size, and for the persistent kernel find how many
   // workgroups the device keeps resident (that is its grid size)
@@ -84,8 +92,8 @@ template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
-#ifdef FMHA_DEV_MINIMAL
-  if (v.drop == 2) return 1;
+#if defined(FMHA_DEV_MINIMAL) || FMHA_TU_STRIDED
+  if (v.drop == 2 || v.qb == 2) return 1; // folded layout only
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;

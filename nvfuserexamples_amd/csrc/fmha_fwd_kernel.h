@@ -65,6 +65,7 @@ struct FwdArgs {
   const int32_t *kv_len; // optional valid key count per group of kv_div heads (pipelined kernel only)
   int32_t kv_div;
   unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
+  RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
 };
 
 // how the mask tensor is read
@@ -97,6 +98,7 @@ template <> FMHA_DEV float dot2_ones<__bf16>(bf16x8 v, int pair, float acc) {
 
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
 __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
+  using RW = Rows<false, D>; // this kernel serves the reference's operators: folded contiguous tensors only
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -132,9 +134,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   if (CAUSAL) qt = a.nqt - 1 - qt; // longest rows first
   const int q0w = qt * QT + w * (QB * 32);
 
-  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
-  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
-  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+  const T *Qb = (const T *)a.q + RW::head(a.mq, bh, a.sq);
+  const T *Kb = (const T *)a.k + RW::head(a.mk, bh, a.sk);
+  const T *Vb = (const T *)a.v + RW::head(a.mv, bh, a.sk);
   const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
   // ---- Q' = Q * scale * log2(e) as B-operand registers
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       u32x4 t = {0u, 0u, 0u, 0u};
-      if (q < a.sq) t = *(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8);
+      if (q < a.sq) t = *(const u32x4 *)(Qb + (size_t)q * RW::ss(a.mq) + ks * 16 + h * 8);
       const v8 raw = as_v8<T>(t);
 #pragma unroll
       for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
@@ -173,8 +175,8 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       const int kr = k0 + row;
       u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
       if (kr < a.sk) {
-        kk = *(const u32x4 *)(Kb + (size_t)kr * D + col * 8);
-        vv = *(const u32x4 *)(Vb + (size_t)kr * D + col * 8);
+        kk = *(const u32x4 *)(Kb + (size_t)kr * RW::ss(a.mk) + col * 8);
+        vv = *(const u32x4 *)(Vb + (size_t)kr * RW::ss(a.mv) + col * 8);
       }
       kst[i] = kk;
       vst[i] = vv;
@@ -498,7 +500,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   }
 
   // ---- epilogue: normalise, round, store O and the row log-sum-exp
-  T *Ob = (T *)a.o + (size_t)bh * a.sq * D;
+  T *Ob = (T *)a.o + RW::head(a.mo, bh, a.sq);
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int q = q0w + qb * 32 + ql;
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
           v4 t;
 #pragma unroll
           for (int i = 0; i < 4; ++i) t[i] = (T)(o[qb][db][4 * g + i] * inv);
-          *(v4 *)(Ob + (size_t)q * D + db * 32 + 8 * g + 4 * h) = t;
+          *(v4 *)(Ob + (size_t)q * RW::ss(a.mo) + db * 32 + 8 * g + 4 * h) = t;
         }
       // the constant part of a full mask's term entered the product rounded to T; the
       // difference cancels in O but belongs in the log-sum-exp

@@ -84,8 +84,9 @@ template <int NSB, int KS, int DB, bool WITH_FIRST_PRODUCT> constexpr FwdOperand
 // (Two query blocks per wave, and head dim 128, need more than the 256 registers of a
 // two-waves-per-SIMD budget by a few; the occupancy attribute makes the compiler spill those
 // few instead of settling for one wave per SIMD, which measures 8-30 % faster.)
-template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
+template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 2 || D == 128) ? 2 : 1, 2))) void fmha_fwd_pipe_kernel(const FwdArgs a) {
+  using RW = Rows<STRIDED, D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -161,8 +162,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     }
     it.kend = nkt * BK < sk ? nkt * BK : sk;
     it.nkt2 = (nkt + 1) & ~1;
-    it.Kb = (const T *)a.k + (size_t)it.bh * a.sk * D;
-    it.Vb = (const T *)a.v + (size_t)it.bh * a.sk * D;
+    it.Kb = (const T *)a.k + RW::head(a.mk, it.bh, a.sk);
+    it.Vb = (const T *)a.v + RW::head(a.mv, it.bh, a.sk);
     it.mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(it.bh / a.mask_div) * a.mask_sb : nullptr;
     return it;
   };
@@ -177,7 +178,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // offset area_off.  Rows past kend re-read the last valid row: their scores get -inf through
   // the extra step, and finite garbage in V is multiplied by P = 0.
   TileCopy<T, D, BK, NT> tcopy;
-  tcopy.init(tid);
+  tcopy.init(tid, RW::ss(a.mk)); // K and V rows are equally far apart
   auto dma_tile = [&](const T *base, int kend, int tile, uint32_t area_off) {
     tcopy.issue(base, tile * BK, kend > 0 ? kend : 1, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
   };
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   auto q_row = [&](const Item &it, int qb) {
     int q = it.qt * QT + w * (QB * 32) + qb * 32 + ql;
     q = q < a.sq ? q : a.sq - 1; // rows past the end repeat the last valid row and are never stored
-    return (const T *)a.q + ((size_t)it.bh * a.sq + q) * D + h * 8;
+    return (const T *)a.q + RW::head(a.mq, it.bh, a.sq) + (size_t)q * RW::ss(a.mq) + h * 8;
   };
   auto dmaQ = [&](const Item &it) {
 #pragma unroll
@@ -675,7 +676,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     }
 
     // ---- item epilogue
-    T *Ob = (T *)a.o + (size_t)bh * a.sq * D;
+    T *Ob = (T *)a.o + RW::head(a.mo, bh, a.sq);
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const int q = q0w + qb * 32 + ql;
@@ -683,7 +684,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
       if (q < a.sq) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * D + db * 32, o[qb][db], inv, h);
+        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * RW::ss(a.mo) + db * 32, o[qb][db], inv, h);
         const float cfix = (MASK == kMaskFull) ? a.mask_b - (float)(T)a.mask_b : 0.f;
         if (a.lse && h == 0)
           a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + cfix + fast_log2(lt)) * FMHA_LN2 : NEG_INF;

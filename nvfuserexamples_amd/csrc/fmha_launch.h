@@ -1,7 +1,8 @@
 // Internal interface between the C-ABI translation unit and the per-(element type,
 // head dim) kernel translation units.  Each kernel TU is compiled once per
-// combination with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} and exports one
-// dispatcher per pass.
+// combination with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1} and exports
+// one dispatcher per pass (the _strided ones read the row maps of the argument block; the
+// others assume folded contiguous tensors).
 #pragma once
 #include <hip/hip_runtime.h>
 #include "fmha_fwd_kernel.h"
@@ -21,6 +22,10 @@ int fwd_dispatch_f16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_f16_d64_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_f16_d128_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_bf16_d64_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_bf16_d128_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 
 struct BwdVariant {
   int mask;  // kMaskNone / kMaskPerKey / kMaskFull
@@ -33,5 +38,9 @@ int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_f16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_f16_d128_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_bf16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_bf16_d128_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 
 } // namespace fmha
