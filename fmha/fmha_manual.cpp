@@ -225,6 +225,14 @@ at::Tensor empty_like_rows(const at::Tensor &x) {
   return at::empty(sizes, x.options()).permute(inv);
 }
 
+// The kernels copy K and V tiles with one set of offsets: where their rows are not equally far
+// apart, both are replaced by dense copies.
+void same_row_pitch(RowsOf &k, RowsOf &v) {
+  if (k.heads == 0 || v.heads == 0 || k.st[2] == v.st[2]) return;
+  k = rows_of(k.t.contiguous(), "k");
+  v = rows_of(v.t.contiguous(), "v");
+}
+
 void set_stride(int64_t (&dst)[3], const RowsOf &r) {
   for (int i = 0; i < 3; ++i) dst[i] = r.st[i];
 }
@@ -279,7 +287,9 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tens
                                             const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
                                             double p_drop, int64_t seed, int64_t offset,
                                             const c10::optional<at::Tensor> &kv_len) {
-  const RowsOf q = rows_of(q_, "q"), k = rows_of(k_, "k"), v = rows_of(v_, "v");
+  const RowsOf q = rows_of(q_, "q");
+  RowsOf k = rows_of(k_, "k"), v = rows_of(v_, "v");
+  same_row_pitch(k, v);
   check_rows(q, k, v);
   at::DeviceGuard guard(q.t.device());
   at::Tensor o = empty_like_rows(q.t);
@@ -318,7 +328,9 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor>
 fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,
          const at::Tensor &o_, const at::Tensor &lse, const c10::optional<at::Tensor> &mask, double scale,
          bool is_causal, double p_drop, int64_t seed, int64_t offset, const c10::optional<at::Tensor> &kv_len) {
-  const RowsOf q = rows_of(q_, "q"), k = rows_of(k_, "k"), v = rows_of(v_, "v");
+  const RowsOf q = rows_of(q_, "q");
+  RowsOf k = rows_of(k_, "k"), v = rows_of(v_, "v");
+  same_row_pitch(k, v);
   check_rows(q, k, v);
   at::DeviceGuard guard(q.t.device());
   TORCH_CHECK(dout_.sizes() == q_.sizes() && o_.sizes() == q_.sizes() && dout_.scalar_type() == q.t.scalar_type() &&

@@ -145,6 +145,9 @@ def test_operators_and_autograd_take_strided_tensors():
     buf[..., :d] = q.view(b, h, s, d).permute(0, 2, 1, 3)
     o5, _ = ops.fmha_fwd(buf[..., :d].permute(0, 2, 1, 3), k4, v4, m, 0.0, False, 0.1, 7, 3)
     assert torch.equal(o5.reshape(b * h, s, d), o3)
+    # so are K and V whose rows are not equally far apart
+    o6, _ = ops.fmha_fwd(q4, k.view(b, h, s, d), v4, m, 0.0, False, 0.1, 7, 3)
+    assert torch.equal(o6.reshape(b * h, s, d), o3)
     # autograd through a packed projection: gradients land in the packed buffer's layout
     packed = torch.empty(b, s, 3, h, d, dtype=torch.float16, device="cuda")
     for i, x in enumerate((q, k, v)):
