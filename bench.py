@@ -27,7 +27,7 @@ sys.path.insert(0, ROOT)
 PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
 # rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) of the headline forward kernel, bytes per launch
-MEASURED_TRAFFIC_BYTES = int((98557 + 32768) * 1024)
+MEASURED_TRAFFIC_BYTES = int((98585 + 32768) * 1024)
 
 B, H, S, D = 32, 16, 512, 64
 
