@@ -81,11 +81,11 @@ template <int NSB, int KS, int DB, bool WITH_FIRST_PRODUCT> constexpr FwdOperand
   return L;
 }
 
-// (Two query blocks per wave, and head dim 128, need more than the 256 registers of a
-// two-waves-per-SIMD budget by a few; the occupancy attribute makes the compiler spill those
+// (Two query blocks per wave, head dim 128, and the staged values of a full mask tensor under a
+// causal mask need more than the 256 registers of a two-waves-per-SIMD budget by a few; the occupancy attribute makes the compiler spill those
 // few instead of settling for one wave per SIMD, which measures 8-30 % faster.)
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 2 || D == 128) ? 2 : 1, 2))) void fmha_fwd_pipe_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 2 || D == 128 || MASK == kMaskFull) ? 2 : 1, 2))) void fmha_fwd_pipe_kernel(const FwdArgs a) {
   using RW = Rows<STRIDED, D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
@@ -273,16 +273,41 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     return panel_read_transposed<T, BK>(ldsV, pl, sb, db, c);
   };
 
-  const T *mrow[QB]; // this lane's rows of a full mask tensor, set when an item starts
-  auto load4 = [&](const T *row, int kk, bool safe, float out[4]) {
-    if (safe) {
-      v4 t = as_v4<T>(*(const u32x2 *)(row + kk));
+  // A full mask tensor takes the register path, one tile ahead: this lane's 32 mask values of the
+  // next tile are requested right after the current tile's have been consumed, so the load has a
+  // whole iteration to land (requested and consumed in the same iteration, it left the wave
+  // waiting on memory in every tile: 135 instead of 85 us at the headline shape).
+  // (At head dim 128 the registers for that are not there: the values are requested where they
+  // are consumed, as they come.)
+  constexpr bool MASK_AHEAD = MASK == kMaskFull && D == 64;
+  const T *mrow[QB];     // this lane's rows of the mask tensor for the current item
+  const T *mrow_nxt[QB]; // ... and for the next item, whose first tile is requested by the last iteration
+  v4 mreg[QB][NSB][4];
+  auto mask_rows = [&](const Item &it, const T *(&rows)[QB]) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = (float)t[i];
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = (kk + i < a.sk) ? (float)row[kk + i] : 0.f;
+    for (int qb = 0; qb < QB; ++qb) {
+      int q = it.qt * QT + w * (QB * 32) + qb * 32 + ql;
+      if (q > a.sq - 1) q = a.sq - 1;
+      rows[qb] = (const T *)a.mask + (size_t)(it.bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
     }
+  };
+  auto mload = [&](const T *const (&mrow)[QB], int tile) {
+    const int k0 = tile * BK;
+    const bool vec_ok = a.mask_vec && (k0 + BK <= a.sk);
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int kk = k0 + sb * 32 + 8 * g + 4 * h;
+          if (vec_ok) {
+            mreg[qb][sb][g] = as_v4<T>(*(const u32x2 *)(mrow[qb] + kk));
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mreg[qb][sb][g][i] = (kk + i < a.sk) ? mrow[qb][kk + i] : (T)0.f;
+          }
+        }
   };
 
   // ---- running state
@@ -418,7 +443,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     constexpr bool GUARDED = decltype(guarded_tag)::value;
     if (MASK == kMaskFull || GUARDED) {
       const int k0 = tile * BK;
-      const bool vec_ok = a.mask_vec && (k0 + BK <= a.sk);
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
         const int q = q0w + qb * 32 + ql;
@@ -427,12 +451,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int kk = k0 + sb * 32 + 8 * g + 4 * h;
-            float mv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (MASK == kMaskFull) load4(mrow[qb], kk, vec_ok, mv);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
               float xv = x[qb][sb][4 * g + t];
-              if (MASK == kMaskFull) xv = fmaf(mv[t], a.mask_a, xv);
+              if (MASK == kMaskFull) xv = fmaf((float)mreg[qb][sb][g][t], a.mask_a, xv);
               if (GUARDED) xv = (kk + t <= q) ? xv : NEG_INF;
               x[qb][sb][4 * g + t] = xv;
             }
@@ -530,9 +552,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     constexpr bool LAST = decltype(last_tag)::value;
     lstoreX(t + 2, xs);
     gloadX(t + 3, xs);
+    if (MASK_AHEAD) {
+      // consume this tile's mask values and request the next tile's before the copies go out: the
+      // compiler's wait for these loads, in the next iteration, then finds nothing younger in flight
+      adjust(t, xc, guarded_tag);
+      if (t + 1 < cur.nkt2) mload(mrow, t + 1);
+      else mload(mrow_nxt, 0); // without a successor: this item's rows again, harmlessly
+    }
     dmaK(t + 2);
     dmaV(t);
-    adjust(t, xc, guarded_tag);
+    if (!MASK_AHEAD) {
+      if (MASK == kMaskFull) mload(mrow, t);
+      adjust(t, xc, guarded_tag);
+    }
     if (FIRST) {
       float shift[QB];
 #pragma unroll
@@ -595,6 +627,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     set_after_next(idx);
     bh = cur.bh;
     q0w = cur.qt * QT + w * (QB * 32);
+    if (MASK == kMaskFull) {
+      mask_rows(cur, mrow);
+      if (MASK_AHEAD) {
+        mask_rows(nxt, mrow_nxt);
+        if (idx == lb) mload(mrow, 0); // later items: requested by the previous item's last iteration
+      }
+    }
 
     // ---- item prologue: Q' registers, state, first product of tile 0
     // Only the first item has copies in flight here (Q, K(0), K(1)) and extra rows that other
@@ -639,11 +678,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
         bx[qb][2] = (T)1.f;
         if (MASK == kMaskFull) bx[qb][3] = (T)a.mask_b;
       }
-      int q = q0w + qb * 32 + ql;
-      if (q > a.sq - 1) q = a.sq - 1;
-      mrow[qb] = nullptr;
-      if (MASK == kMaskFull)
-        mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
     }
     g1(0, xA, bkA, limA);
     __syncthreads(); // tile 0's K stage is refilled during the first iteration
