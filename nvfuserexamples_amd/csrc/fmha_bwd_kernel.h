@@ -95,11 +95,12 @@ template <typename T> FMHA_DEV void split_hi_lo(float v, T &hi, T &lo) {
 }
 
 // ------------------------------------------------------------------------------ dQ
-// (At head dim 128 some variants need a few registers more than a two-waves-per-SIMD budget:
-// spill those few rather than drop to one wave per SIMD, +10 % measured.)
+// (At head dim 128, and with a full mask tensor under a causal mask and dropout, some variants need
+// a few registers more than a two-waves-per-SIMD budget: spill those few rather than drop to one
+// wave per SIMD, +10 % measured.)
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED>
 __global__ __launch_bounds__(NW * 64)
-    __attribute__((amdgpu_waves_per_eu(D == 128 ? 2 : 1, 2))) void fmha_bwd_dq_kernel(const BwdArgs a) {
+    __attribute__((amdgpu_waves_per_eu((D == 128 || MASK == kMaskFull) ? 2 : 1, 2))) void fmha_bwd_dq_kernel(const BwdArgs a) {
   using RW = Rows<STRIDED, D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
