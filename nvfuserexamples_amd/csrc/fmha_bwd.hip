@@ -34,7 +34,8 @@ template <typename K> int set_lds(K kern, int bytes) {
 
 template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipStream_t s) {
   constexpr int kLdsQ = BwdCfg<FMHA_TU_D, bwd_dq_tile_rows<FMHA_TU_D>()>::LDS_BYTES;
-  constexpr int kLdsK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>::LDS_BYTES;
+  using CfgK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>;
+  constexpr int kLdsK = CfgK::LDS_BYTES + (MASK == kMaskFull ? CfgK::MASK_BYTES : 0);
   auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP, kStrided>;
   auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP, kStrided>;
   static const int attr = set_lds(kq, kLdsQ) | set_lds(kk, kLdsK);

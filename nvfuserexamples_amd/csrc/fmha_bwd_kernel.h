@@ -76,6 +76,9 @@ template <int D, int BT_> struct BwdCfg {
   static constexpr int XROWB = 32;        // extra-step rows: 16 elements
   // two tiles x 2 stages + two sets of extra rows x 2 stages + {delta} x 2 stages
   static constexpr int LDS_BYTES = 4 * TILEB + 2 * 2 * BT * XROWB + 2 * BT * 4;
+  // dK/dV kernel with a full mask tensor: [stage][BT queries][128 keys of the workgroup + 8] mask values
+  static constexpr int MASK_PITCH = 128 + 8;
+  static constexpr int MASK_BYTES = 2 * BT * MASK_PITCH * 2;
 };
 
 // Keys a head may see at all: [0, sk) or its valid count (possibly 0).
@@ -268,15 +271,29 @@ __global__ __launch_bounds__(NW * 64)
     if (MASK == kMaskFull)
       mrow[qb] = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + (size_t)q * a.mask_sq;
   }
-  auto load4 = [&](const T *row, int kk, bool safe, float out[4]) {
-    if (safe) {
-      v4 t = as_v4<T>(*(const u32x2 *)(row + kk));
+  // A full mask tensor takes the register path, one tile ahead (at head dim 64, where the
+  // registers are there): this lane's 32 mask values of the next tile are requested as soon as
+  // the current tile's have been consumed -- they seed the score accumulators, so that happens at
+  // the top of the iteration, before the copies go out.
+  constexpr bool MASK_AHEAD = MASK == kMaskFull && D == 64;
+  v4 mreg[QB][NSB][4];
+  auto mload = [&](int tile) {
+    const int mk0 = tile * BK;
+    const bool vec_ok = a.mask_vec && (mk0 + BK <= a.sk);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = (float)t[i];
-    } else {
+    for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = (kk + i < a.sk) ? (float)row[kk + i] : 0.f;
-    }
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int kk = mk0 + sb * 32 + 8 * g + 4 * h;
+          if (vec_ok) {
+            mreg[qb][sb][g] = as_v4<T>(*(const u32x2 *)(mrow[qb] + kk));
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mreg[qb][sb][g][i] = (kk + i < a.sk) ? mrow[qb][kk + i] : (T)0.f;
+          }
+        }
   };
 
   f32x16 dq[QB][DB];
@@ -287,6 +304,7 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
       for (int r = 0; r < 16; ++r) dq[qb][db][r] = 0.f;
 
+  if (MASK_AHEAD) mload(0);
   dma_kv(0);
   gloadX(0);
   lstoreX(0);
@@ -297,6 +315,20 @@ __global__ __launch_bounds__(NW * 64)
   for (int kt = 0; kt < nkt; ++kt) {
     const int cur = kt & 1;
     const int k0 = kt * BK;
+    // x^T = K.Q'^T + (mask - LSE) ; g^T = drop_scale*V.dO^T - delta   (accumulators visited round-robin)
+    // A full mask tensor's term seeds the score accumulators.
+    f32x16 x[QB][NSB], g[QB][NSB];
+    if (MASK == kMaskFull && !MASK_AHEAD) mload(kt);
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          x[qb][sb][r] = MASK == kMaskFull ? (float)mreg[qb][sb][r / 4][r % 4] * a.mask_a : 0.f;
+          g[qb][sb][r] = 0.f;
+        }
+    if (MASK_AHEAD && kt + 1 < nkt) mload(kt + 1);
     if (kt + 1 < nkt) {
       lstoreX(cur ^ 1); // rows of tile kt+1, loaded one iteration ago
       gloadX(kt + 2);
@@ -306,17 +338,6 @@ __global__ __launch_bounds__(NW * 64)
     const char *ldsV = ldsK + TILEB;
     const char *ldsX = ldsXb + cur * BK * XROWB;
 
-    // x^T = K.Q'^T + (mask - LSE) ; g^T = drop_scale*V.dO^T - delta   (accumulators visited round-robin)
-    f32x16 x[QB][NSB], g[QB][NSB];
-#pragma unroll
-    for (int sb = 0; sb < NSB; ++sb)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          x[qb][sb][r] = 0.f;
-          g[qb][sb][r] = 0.f;
-        }
 #pragma unroll
     for (int ks = 0; ks <= KS; ++ks)
 #pragma unroll
@@ -340,7 +361,6 @@ __global__ __launch_bounds__(NW * 64)
       }
 
     const bool diag = CAUSAL && (k0 + BK - 1 > q0w);
-    const bool vec_ok = a.mask_vec && (k0 + BK <= a.sk);
     v8 dsfrag[QB][NSB][2];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -353,12 +373,9 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
           const int kk = k0 + sb * 32 + 8 * gq + 4 * h;
-          float mv[4] = {0.f, 0.f, 0.f, 0.f};
-          if (MASK == kMaskFull) load4(mrow[qb], kk, vec_ok, mv);
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             float xv = x[qb][sb][4 * gq + t];
-            if (MASK == kMaskFull) xv = fmaf(mv[t], a.mask_a, xv);
             if (diag) xv = (kk + t <= q) ? xv : BIGNEG;
             const float p = fast_exp2(xv);
             float gv = g[qb][sb][4 * gq + t];
@@ -495,7 +512,16 @@ __global__ __launch_bounds__(NW * 64)
       bxd[kb][1] = (T)1.f;
     }
   }
+  // A full mask tensor reaches the lanes (one key each) through LDS: the [BQ queries x 128 keys]
+  // tile is loaded row-wise, 8 bytes per thread and load, one tile ahead like the extra rows, and
+  // each lane then reads its key's column.  (Read straight from global memory, two bytes per lane
+  // and element, the mask made this kernel five times slower.)
   const T *mbase = (MASK == kMaskFull) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
+  constexpr int MP = C::MASK_PITCH;
+  constexpr int MLOADS = BQ * 32 / NT; // 8-byte pieces per thread: the tile has BQ rows of 32
+  static_assert(MASK != kMaskFull || (KT == 128 && (BQ * 32) % NT == 0), "mask tile staging assumes 128 keys per workgroup");
+  T *ldsM = (T *)(lds + C::LDS_BYTES);
+  u32x2 mraw[MASK == kMaskFull ? MLOADS : 1];
 
   const int nqt = (a.sq + BQ - 1) / BQ;
   // first query tile that sees any of these keys; none at all if the whole key tile is invalid
@@ -523,8 +549,39 @@ __global__ __launch_bounds__(NW * 64)
     qr = qvalid ? qr : a.sq - 1;
     lraw = lseb[qr];
     draw = delb[qr];
+    if (MASK == kMaskFull) {
+      const int kbase = ktile * KT;
+      const bool vec_ok = a.mask_vec && (kbase + KT <= a.sk);
+#pragma unroll
+      for (int i = 0; i < MLOADS; ++i) {
+        const int c = i * NT + tid, row = c >> 5, col = (c & 31) * 4;
+        int q = qt * BQ + row;
+        q = q < a.sq ? q : a.sq - 1;
+        const T *src = mbase + (size_t)q * a.mask_sq + kbase + col;
+        if (vec_ok) {
+          mraw[i] = *(const u32x2 *)src;
+        } else { // ragged or unaligned: element by element, inside the row
+          v4 t;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int kc = kbase + col + j < a.sk ? kbase + col + j : a.sk - 1;
+            t[j] = mbase[(size_t)q * a.mask_sq + kc];
+          }
+          union { v4 v; u32x2 u; } cv;
+          cv.v = t;
+          mraw[i] = cv.u;
+        }
+      }
+    }
   };
   auto lstoreX = [&](int stage) {
+    if (MASK == kMaskFull) {
+#pragma unroll
+      for (int i = 0; i < MLOADS; ++i) {
+        const int c = i * NT + tid, row = c >> 5, col = (c & 31) * 4;
+        *(u32x2 *)(ldsM + (stage * BQ + row) * MP + col) = mraw[i];
+      }
+    }
     if (tid < BQ) {
       // rows past the end (whose Q/dO rows repeat the last valid row) and fully masked rows: P = 0
       float nl = BIGNEG, dl = 0.f;
@@ -602,7 +659,11 @@ __global__ __launch_bounds__(NW * 64)
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          x[kb][sb][r] = 0.f;
+          // a full mask tensor's term seeds the score accumulators: row = query 8*(r/4) + 4h + r%4 of
+          // the 32-query block, column = this lane's key
+          x[kb][sb][r] = MASK == kMaskFull
+                             ? (float)ldsM[(cur * BQ + sb * 32 + 8 * (r / 4) + 4 * h + r % 4) * MP + w * (KB * 32) + kb * 32 + kl] * a.mask_a
+                             : 0.f;
           g[kb][sb][r] = 0.f;
         }
 #pragma unroll
@@ -648,11 +709,6 @@ __global__ __launch_bounds__(NW * 64)
           for (int t = 0; t < 4; ++t) {
             const int q = q0 + qq + t;
             float xv = x[kb][sb][4 * gq + t];
-            if (MASK == kMaskFull) {
-              const int qc = q < a.sq ? q : a.sq - 1;
-              const int kc = key < a.sk ? key : a.sk - 1;
-              xv = fmaf((float)mbase[(size_t)qc * a.mask_sq + kc], a.mask_a, xv);
-            }
             if (diag) xv = (key <= q) ? xv : BIGNEG;
             const float p = fast_exp2(xv);
             float gv = g[kb][sb][4 * gq + t];
