@@ -190,6 +190,7 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
+  v.saving = saving;
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
   // flop.  That pays (4-6 % measured) for the unmasked variant at head dim 64 on long key
   // ranges when there is enough work for every resident workgroup to get several 256-query

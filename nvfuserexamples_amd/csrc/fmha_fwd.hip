@@ -29,12 +29,12 @@ namespace {
 constexpr int kNW = FMHA_FWD_NW;
 constexpr bool kStrided = FMHA_TU_STRIDED != 0;
 
-template <int QB, int MASK, bool CAUSAL, int DROP> int launch(FwdArgs &a, hipStream_t s) {
-  constexpr bool kPipe = DROP != 2;
+template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int launch(FwdArgs &a, hipStream_t s) {
   constexpr int kLds = kPipe ? PipeCfg<FMHA_TU_D, QB>::lds_bytes(kNW) : FwdCfg<FMHA_TU_D>::LDS_BYTES;
-  // tensor dropout and the save pass run on the plain loop; everything else is software-pipelined
+  // the save pass (and tensor dropout at head dim 128) runs on the plain loop; everything else is
+  // software-pipelined
   auto kern = [] {
-    if constexpr (DROP == 2) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+    if constexpr (!kPipe) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
     else return fmha_fwd_pipe_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP, kStrided>;
   }();
   // once per kernel: allow the dynamic LDS size, and for the persistent kernel find how many
@@ -97,6 +97,13 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;
+#if FMHA_TU_D == 64
+    if (!v.saving) { // dropout tensor alone: pipelined kernel
+      if (v.mask == kMaskPerKey) return launch<1, kMaskPerKey, false, 2, true>(a, s);
+      if (v.mask == kMaskFull) return launch<1, kMaskFull, false, 2, true>(a, s);
+      return launch<1, kMaskNone, false, 2, true>(a, s);
+    }
+#endif
     if (v.mask == kMaskPerKey) return launch<1, kMaskPerKey, false, 2>(a, s);
     if (v.mask == kMaskFull) return launch<1, kMaskFull, false, 2>(a, s);
     return launch<1, kMaskNone, false, 2>(a, s);

@@ -85,7 +85,7 @@ template <int NSB, int KS, int DB, bool WITH_FIRST_PRODUCT> constexpr FwdOperand
 // causal mask need more than the 256 registers of a two-waves-per-SIMD budget by a few; the occupancy attribute makes the compiler spill those
 // few instead of settling for one wave per SIMD, which measures 8-30 % faster.)
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 2 || D == 128 || MASK == kMaskFull) ? 2 : 1, 2))) void fmha_fwd_pipe_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 2 || D == 128 || MASK == kMaskFull || DROP == 2) ? 2 : 1, 2))) void fmha_fwd_pipe_kernel(const FwdArgs a) {
   using RW = Rows<STRIDED, D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
@@ -96,7 +96,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
   static_assert(NT >= BK, "the extra rows are staged by the first BK threads");
-  static_assert(DROP == 0 || DROP == 1, "tensor dropout and the save pass use fmha_fwd_kernel");
+  static_assert(DROP == 0 || DROP == 1 || (DROP == 2 && D == 64 && !CAUSAL),
+                "the save pass, and tensor dropout at head dim 128, use fmha_fwd_kernel");
   static_assert(D % 64 == 0, "tiles are stored as panels of 64 columns");
   constexpr float NEG_INF = -__builtin_inff();
   constexpr float WINDOW = 16384.f;
@@ -308,6 +309,43 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
             for (int i = 0; i < 4; ++i) mreg[qb][sb][g][i] = (kk + i < a.sk) ? mrow[qb][kk + i] : (T)0.f;
           }
         }
+  };
+
+  // A dropout tensor (the reference's train operators: 0/1 values in the element type, shaped like
+  // the scores) takes the same register path, one tile BEHIND: tile t's values are requested in
+  // iteration t and multiply P(t) at the top of iteration t+1, just before the second product
+  // consumes it, so they too have a whole iteration to land and need one set of registers.
+  const T *drow[QB];
+  v4 dreg[QB][NSB][4];
+  auto dload = [&](int tile) {
+    const int k0 = tile * BK;
+    const bool vec_ok = a.mask_vec && (k0 + BK <= a.sk);
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int kk = k0 + sb * 32 + 8 * g + 4 * h;
+          if (vec_ok) {
+            dreg[qb][sb][g] = as_v4<T>(*(const u32x2 *)(drow[qb] + kk));
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dreg[qb][sb][g][i] = (kk + i < a.sk) ? drow[qb][kk + i] : (T)0.f;
+          }
+        }
+  };
+  auto apply_drop = [&](v8 (&p)[QB][NSB][2]) {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            p[qb][sb][g >> 1][4 * (g & 1) + t] =
+                (T)((float)p[qb][sb][g >> 1][4 * (g & 1) + t] * (float)dreg[qb][sb][g][t]);
   };
 
   // ---- running state
@@ -547,7 +585,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // wait for a load it knows about also waits for every copy issued ahead of it.
   auto body = [&](int t, auto first_tag, auto last_tag, auto guarded_tag, f32x16 (&xc)[QB][NSB], float (&bkc)[QB],
                   float (&limc)[QB], f32x16 (&xn)[QB][NSB], float (&bkn)[QB], float (&limn)[QB],
-                  const v8 (&pprev)[QB][NSB][2], v8 (&pcur)[QB][NSB][2]) {
+                  v8 (&pprev)[QB][NSB][2], v8 (&pcur)[QB][NSB][2]) {
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr bool LAST = decltype(last_tag)::value;
     lstoreX(t + 2, xs);
@@ -558,6 +596,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       adjust(t, xc, guarded_tag);
       if (t + 1 < cur.nkt2) mload(mrow, t + 1);
       else mload(mrow_nxt, 0); // without a successor: this item's rows again, harmlessly
+    }
+    if (DROP == 2) {
+      if (!FIRST) apply_drop(pprev); // with tile t-1's values, requested one iteration ago
+      dload(t);
     }
     dmaK(t + 2);
     dmaV(t);
@@ -627,6 +669,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     set_after_next(idx);
     bh = cur.bh;
     q0w = cur.qt * QT + w * (QB * 32);
+    if (DROP == 2) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        int q = q0w + qb * 32 + ql;
+        if (q > a.sq - 1) q = a.sq - 1;
+        drow[qb] = (const T *)a.drop_mask + ((size_t)bh * a.sq + q) * a.sk;
+      }
+    }
     if (MASK == kMaskFull) {
       mask_rows(cur, mrow);
       if (MASK_AHEAD) {
@@ -706,6 +756,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       if (diag(t)) body(t, No{}, Yes{}, Yes{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
       else body(t, No{}, Yes{}, No{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
       tile_sync();
+      if (DROP == 2) apply_drop(pB);
       g2(t, pB);
     }
 

@@ -15,6 +15,7 @@ struct FwdVariant {
   int mask;     // kMaskNone / kMaskPerKey (constant along queries) / kMaskFull
   bool causal;
   int drop;     // 0 none, 1 Philox, 2 tensor / save-intermediates
+  bool saving;  // drop == 2: the save-intermediates pass is wanted (plain kernel only)
 };
 
 // Return 0 on success, 1 if the variant is not built, 2 if the launch failed.

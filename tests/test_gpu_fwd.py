@@ -149,6 +149,30 @@ def test_train_ops_and_saved_intermediates():
     assert torch.equal(o2, o)  # the save pass does not disturb O
 
 
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,mask", [
+    (6, 200, 333, 64, "fp16", "pad"),        # ragged tiles, per-key mask
+    (4, 192, 192, 64, "bf16", "add_full"),   # full mask tensor and dropout tensor together
+    (600, 128, 192, 64, "fp16", None),       # more items than resident workgroups
+    (4, 160, 224, 128, "fp16", "pad"),       # head dim 128: the plain kernel
+])
+def test_tensor_dropout_matches_oracle(bh, sq, sk, d, dtype, mask):
+    """An explicit 0/1 dropout tensor scaled by 2 (reference fmha/fmha_manual.cpp:478-480) beyond the
+    reference's fixed shape: ragged tiles, broadcast and full masks, many items per workgroup."""
+    q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sq, std=0.5 if d == 128 else 1.0, dtype=dtype)
+    g = torch.Generator().manual_seed(sk)
+    dm = torch.empty(bh, sq, sk).random_(2, generator=g).to(TDT[dtype])
+    m = None
+    if mask == "pad":
+        m = pad_mask(2, sk, sk // 2, sk).to(TDT[dtype])
+    elif mask == "add_full":
+        m = (torch.empty(bh, sq, sk).random_(2, generator=g) * -1000).to(TDT[dtype])
+    o, _, _, _ = _run(q, k, v, mask=None if m is None else m.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(),
+                      drop_scale=2.0)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=None if m is None else f32(m), drop_mask=f32(dm),
+                           drop_scale=2.0, want=("o",))
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= (4e-3 if dtype == "fp16" else 4e-2)   # O is up to 2x larger here
+
+
 def test_size_independent_properties_at_headline_shape():
     """B32 H16 S512 D64 (full size): properties that need no CPU answer, plus oracle parity on a
     sample of heads."""
