@@ -111,6 +111,71 @@ def time_launches(torch, step, steps, warmup):
     return sum(a.elapsed_time(b) for a, b in ev) / steps
 
 
+def short_sequence_legs(torch, capi, L, stream, steps, warmup):
+    """The bandwidth-bound shapes: the reference's own operators at the reference's fixed shape
+    (BH 512, S 128, D 64 with full [BH,S,S] mask tensors: fmha/fmha_manual.cpp:24-29, test.py:20-23)
+    and the BERT-base configuration that the CPU baseline is timed on.  Reported as time and as
+    algorithmic bytes per second against the HBM peak, beside the headline, never as `value`.
+    The reference-shape legs rotate six input sets (302 / 403 MB, more than the 256 MB last-level
+    cache); the BERT-base leg is 6 MB and stays cache-resident whatever is rotated."""
+    legs = {}
+
+    def run(name, Ps, nbytes, note):
+        def step(i):
+            L.fmha_fwd_launch(C.byref(Ps[i % len(Ps)]), stream)
+        capi.check(L.fmha_fwd_launch(C.byref(Ps[0]), stream))
+        ms, _ = time_steps(torch, step, steps, warmup)
+        legs[name] = {"us": round(ms * 1e3, 2), "algorithmic_MB": round(nbytes / 1e6, 2),
+                      "hbm_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                      "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "inputs": note}
+
+    g = torch.Generator().manual_seed(7)
+    bh, s, d = 512, 128, 64
+    keep, infer, train = [], [], []
+    for _ in range(6):
+        q, k, v = (torch.randn(bh, s, d, generator=g).to(torch.float16).cuda() for _ in range(3))
+        o = torch.empty_like(q)
+        amask = (torch.rand(bh, s, s, generator=g) > 0.1).to(torch.float16).cuda()
+        pad = (torch.rand(bh, s, s, generator=g) > 0.9).to(torch.float16).mul_(-1000.0).cuda()
+        dm = (torch.rand(bh, s, s, generator=g) > 0.5).to(torch.float16).cuda()
+        keep.append((q, k, v, o, amask, pad, dm))
+        for kind in ("infer", "train"):
+            P = capi.FwdParams()
+            P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+            P.bh, P.sq, P.sk, P.d = bh, s, s, d
+            P.dtype, P.scale = capi.F16, 0.125
+            P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = 1, s * s, s
+            if kind == "infer":
+                P.mask, P.mask_kind, P.mask_neg = amask.data_ptr(), capi.MASK_KEEP01, -10000.0
+                infer.append(P)
+            else:
+                P.mask, P.mask_kind = pad.data_ptr(), capi.MASK_ADDITIVE
+                P.drop_kind, P.drop_mask, P.drop_scale = capi.DROP_TENSOR, dm.data_ptr(), 2.0
+                train.append(P)
+    run("fmha_nvfuser_BH512_S128_D64_full_mask", infer, 4 * bh * s * d * 2 + bh * s * s * 2, "6 sets rotated")
+    run("fmha_train_nvfuser_BH512_S128_D64_full_masks", train, 4 * bh * s * d * 2 + 2 * bh * s * s * 2,
+        "6 sets rotated")
+    del keep, infer, train
+
+    b1, h1 = 8, 12   # BERT-base forward: the configuration of the CPU baseline
+    q1, k1, v1 = (torch.randn(b1 * h1, s, d, generator=g).to(torch.float16).cuda() for _ in range(3))
+    o1 = torch.empty_like(q1)
+    m1 = torch.zeros(b1, 1, 1, s)
+    for i in range(b1):
+        m1[i, 0, 0, 64 + 8 * i:] = -10000.0
+    m1 = m1.to(torch.float16).cuda()
+    P = capi.FwdParams()
+    P.q, P.k, P.v, P.o = q1.data_ptr(), k1.data_ptr(), v1.data_ptr(), o1.data_ptr()
+    P.bh, P.sq, P.sk, P.d = b1 * h1, s, s, d
+    P.dtype, P.scale = capi.F16, 0.125
+    P.mask, P.mask_kind = m1.data_ptr(), capi.MASK_ADDITIVE
+    P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = h1, s, 0
+    name = "B8_H12_S128_D64_pad_mask"
+    run(name, [P], 4 * b1 * h1 * s * d * 2 + b1 * s * 2, "one set, cache-resident")
+    legs[name]["tflops"] = round(4.0 * b1 * h1 * s * s * d / (legs[name]["us"] * 1e-6) / 1e12, 2)
+    return legs
+
+
 def power_probe(torch, step, seconds=2.0):
     """Socket power and graphics clocks as the board's management firmware reports them (amd-smi),
     sampled while `step` runs back to back on a second thread.  The attention kernels are
@@ -342,6 +407,7 @@ def main():
                            "permute_copies_spared_ms": round(ms_perm, 5)},
     }
 
+    out["short_sequences"] = short_sequence_legs(torch, capi, L, stream, args.steps, args.warmup)
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
