@@ -31,6 +31,13 @@ CASES = [
     (2, 256, 256, 128, "fp16", None, False, 0.1),
     (2, 1024, 1024, 128, "bf16", None, True, 0.0),     # wide-head bf16 causal
     (4, 192, 192, 64, "bf16", "pad", False, 0.1),
+    (4, 1, 1000, 64, "fp16", None, False, 0.0),        # one query against a long key range (decode step)
+    (4, 300, 1, 64, "fp16", None, False, 0.0),         # one key: P = 1, dQ = dK = 0 exactly (with dropout the
+                                                       # rounding of O in delta leaves ~3e-3 absolute in a zero gradient)
+    (2, 130, 257, 64, "fp16", "add_full", False, 0.0), # full mask rows that are not 8-byte aligned
+    (2, 192, 320, 128, "bf16", "add_full", False, 0.1),  # full mask tensor at head dim 128
+    (2, 260, 260, 64, "bf16", "add_full", True, 0.1),  # full mask + causal + dropout
+    (300, 128, 192, 64, "fp16", "add_full", False, 0.0),  # full mask, many workgroups
     # causal: a workgroup takes a pair of tiles (i, n-1-i); odd tile counts leave the middle one alone,
     # and with sk > sq the last key tiles see no query at all
     (3, 300, 300, 64, "fp16", None, True, 0.0),
