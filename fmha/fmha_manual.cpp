@@ -112,6 +112,7 @@ at::Tensor fmha_nvfuser(const at::Tensor &input, const at::Tensor &qk, const at:
   MaskLayout m = mask_layout(amask, input, input.size(0), input.size(1), qk.size(1), "amask");
   at::Tensor o = at::empty_like(input);
   fmha_fwd_params p = {};
+  p.struct_bytes = sizeof p;
   fill_common(p, input, qk, v, o, default_scale(input));
   p.mask = m.t.data_ptr();
   p.mask_kind = FMHA_MASK_KEEP01;
@@ -141,6 +142,7 @@ std::vector<at::Tensor> train_forward(const at::Tensor &input, const at::Tensor 
   at::Tensor dm = dropout_mask.contiguous();
   at::Tensor o = at::empty_like(input);
   fmha_fwd_params p = {};
+  p.struct_bytes = sizeof p;
   fill_common(p, input, qk, v, o, default_scale(input));
   p.mask = m.t.data_ptr();
   p.mask_kind = FMHA_MASK_ADDITIVE;
@@ -297,6 +299,7 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tens
   at::Tensor lse = q.heads ? at::empty({q_.size(0), q_.size(1), q.s}, q.t.options().dtype(at::kFloat))
                            : at::empty({q.bh, q.s}, q.t.options().dtype(at::kFloat));
   fmha_fwd_params p = {};
+  p.struct_bytes = sizeof p;
   p.q = q.t.data_ptr();
   p.k = k.t.data_ptr();
   p.v = v.t.data_ptr();
@@ -345,6 +348,7 @@ fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, co
   const RowsOf dqr = rows_of(dq, "dq"), dkr = rows_of(dk, "dk"), dvr = rows_of(dv, "dv");
   at::Tensor delta = at::empty_like(lsec);
   fmha_bwd_params p = {};
+  p.struct_bytes = sizeof p;
   p.q = q.t.data_ptr();
   p.k = k.t.data_ptr();
   p.v = v.t.data_ptr();

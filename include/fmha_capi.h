@@ -70,6 +70,10 @@ enum {
  * store (fmha_manual.cpp:95).
  */
 typedef struct fmha_fwd_params {
+  /* sizeof(fmha_fwd_params) as the caller was compiled.  Fields are only ever appended: the library
+   * reads that many bytes and takes every field beyond them as zero, so a caller built against an
+   * older header keeps working.  Zero-initialise the struct (`= {}`) and set this first. */
+  uint64_t struct_bytes;
   const void *q, *k, *v;
   void *o;
   float *lse; /* optional [bh,sq]: log(sum_j exp(score_ij)), saved for the backward */
@@ -137,6 +141,7 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream);
  * `delta` is caller-provided scratch of bh*sq floats (written, then read).
  */
 typedef struct fmha_bwd_params {
+  uint64_t struct_bytes; /* sizeof(fmha_bwd_params) as the caller was compiled; see fmha_fwd_params */
   const void *q, *k, *v, *o, *dout;
   const float *lse;
   float *delta;

@@ -18,8 +18,17 @@ EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_philox_keep_mask", "fmha_
            "fmha_strerror", "fmha_version")
 
 
-class FwdParams(C.Structure):
+class _Params(C.Structure):
+    """Parameter structs carry their own size first (the library reads that many bytes)."""
+
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        self.struct_bytes = C.sizeof(self)
+
+
+class FwdParams(_Params):
     _fields_ = [
+        ("struct_bytes", C.c_uint64),
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("lse", C.c_void_p),
         ("mask", C.c_void_p), ("mask_kind", C.c_int32), ("causal", C.c_int32),
         ("mask_bh_div", C.c_int64), ("mask_stride_b", C.c_int64), ("mask_stride_q", C.c_int64),
@@ -37,8 +46,9 @@ class FwdParams(C.Structure):
     ]
 
 
-class BwdParams(C.Structure):
+class BwdParams(_Params):
     _fields_ = [
+        ("struct_bytes", C.c_uint64),
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("dout", C.c_void_p),
         ("lse", C.c_void_p), ("delta", C.c_void_p),
         ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),

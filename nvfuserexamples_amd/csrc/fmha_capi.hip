@@ -4,6 +4,8 @@
 #include "fmha_launch.h"
 
 #include <cmath>
+#include <cstddef>
+#include <cstring>
 #include <cstdlib>
 
 using namespace fmha;
@@ -65,7 +67,7 @@ const char *fmha_strerror(int code) {
   case FMHA_E_DTYPE: return "unknown dtype (0 = fp16, 1 = bf16)";
   case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64 or 128, and one head's rows must span less than 2^31 elements";
   case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned and their strides multiples of 8 elements";
-  case FMHA_E_ARG: return "argument out of range (scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
+  case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
   case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox; the backward takes Philox dropout only; k and v rows must be equally far apart)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
   default: return "unknown error code";
@@ -119,8 +121,15 @@ static int make_row_map(RowMap &m, int32_t heads, const int64_t st[3], int32_t b
 
 extern "C" {
 
-int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
-  if (!p || !p->q || !p->k || !p->v || !p->o) return FMHA_E_NULL;
+int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
+  // the caller's struct may be shorter (older header) or longer (newer) than this library's
+  if (!caller) return FMHA_E_NULL;
+  if (caller->struct_bytes < offsetof(fmha_fwd_params, kv_len)) return FMHA_E_ARG;
+  fmha_fwd_params local;
+  std::memset(&local, 0, sizeof local);
+  std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
+  const fmha_fwd_params *p = &local;
+  if (!p->q || !p->k || !p->v || !p->o) return FMHA_E_NULL;
   if (p->dtype != FMHA_DTYPE_F16 && p->dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
   if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;
   if (p->d != 64 && p->d != 128) return FMHA_E_SHAPE;
@@ -229,8 +238,14 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream) {
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 
-int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream) {
-  if (!p || !p->q || !p->k || !p->v || !p->o || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk || !p->dv)
+int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
+  if (!caller) return FMHA_E_NULL;
+  if (caller->struct_bytes < offsetof(fmha_bwd_params, kv_len)) return FMHA_E_ARG;
+  fmha_bwd_params local;
+  std::memset(&local, 0, sizeof local);
+  std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
+  const fmha_bwd_params *p = &local;
+  if (!p->q || !p->k || !p->v || !p->o || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk || !p->dv)
     return FMHA_E_NULL;
   if (p->dtype != FMHA_DTYPE_F16 && p->dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
   if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;

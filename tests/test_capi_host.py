@@ -48,6 +48,8 @@ def _valid_params():
 
 @pytest.mark.parametrize("mutate,code", [
     (lambda P: setattr(P, "q", None), -1),
+    (lambda P: setattr(P, "struct_bytes", 0), -5),                    # the struct must carry its size
+    (lambda P: setattr(P, "struct_bytes", 64), -5),                   # ... at least up to the first release's fields
     (lambda P: setattr(P, "dtype", 7), -2),
     (lambda P: setattr(P, "d", 80), -3),
     (lambda P: setattr(P, "sq", 0), -3),

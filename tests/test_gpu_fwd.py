@@ -173,6 +173,27 @@ def test_tensor_dropout_matches_oracle(bh, sq, sk, d, dtype, mask):
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= (4e-3 if dtype == "fp16" else 4e-2)   # O is up to 2x larger here
 
 
+def test_a_caller_built_against_an_older_header_keeps_working():
+    """The parameter struct carries its own size: the library reads that many bytes and takes the fields
+    beyond them as zero, whatever the memory after a shorter struct holds."""
+    import ctypes as C
+    q, k, v = (t.cuda() for t in make_qkv(4, 96, 160, 64, seed=6))
+    want = capi.fwd(q, k, v)[0]
+    P = capi.FwdParams()
+    o = torch.empty_like(q)
+    P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+    P.bh, P.sq, P.sk, P.d = 4, 96, 160, 64
+    P.dtype, P.scale = capi.F16, 64 ** -0.5
+    # everything from kv_len on is "after the end" of an old caller's struct: poison it
+    P.struct_bytes = capi.FwdParams.kv_len.offset
+    P.kv_len, P.kv_len_bh_div, P.heads = 0xdead0, 3, 5
+    P.q_stride[:] = [7, 7, 7]
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert capi.lib().fmha_fwd_launch(C.byref(P), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(o, want)
+
+
 def test_size_independent_properties_at_headline_shape():
     """B32 H16 S512 D64 (full size): properties that need no CPU answer, plus oracle parity on a
     sample of heads."""
