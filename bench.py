@@ -116,7 +116,7 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
     (BH 512, S 128, D 64 with full [BH,S,S] mask tensors: fmha/fmha_manual.cpp:24-29, test.py:20-23)
     and the BERT-base configuration that the CPU baseline is timed on.  Reported as time and as
     algorithmic bytes per second against the HBM peak, beside the headline, never as `value`.
-    The reference-shape legs rotate six input sets (302 / 403 MB, more than the 256 MB last-level
+    The reference-shape legs rotate six input sets (302 to 604 MB, more than the 256 MB last-level
     cache); the BERT-base leg is 6 MB and stays cache-resident whatever is rotated."""
     legs = {}
 
@@ -131,15 +131,16 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
 
     g = torch.Generator().manual_seed(7)
     bh, s, d = 512, 128, 64
-    keep, infer, train = [], [], []
+    keep, infer, train, save = [], [], [], []
     for _ in range(6):
         q, k, v = (torch.randn(bh, s, d, generator=g).to(torch.float16).cuda() for _ in range(3))
         o = torch.empty_like(q)
         amask = (torch.rand(bh, s, s, generator=g) > 0.1).to(torch.float16).cuda()
         pad = (torch.rand(bh, s, s, generator=g) > 0.9).to(torch.float16).mul_(-1000.0).cuda()
         dm = (torch.rand(bh, s, s, generator=g) > 0.5).to(torch.float16).cuda()
-        keep.append((q, k, v, o, amask, pad, dm))
-        for kind in ("infer", "train"):
+        sm, dr = (torch.empty(bh, s, s, dtype=torch.float16, device="cuda") for _ in range(2))
+        keep.append((q, k, v, o, amask, pad, dm, sm, dr))
+        for kind in ("infer", "train", "save"):
             P = capi.FwdParams()
             P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
             P.bh, P.sq, P.sk, P.d = bh, s, s, d
@@ -151,11 +152,15 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
             else:
                 P.mask, P.mask_kind = pad.data_ptr(), capi.MASK_ADDITIVE
                 P.drop_kind, P.drop_mask, P.drop_scale = capi.DROP_TENSOR, dm.data_ptr(), 2.0
-                train.append(P)
+                if kind == "save":
+                    P.save_softmax, P.save_dropout = sm.data_ptr(), dr.data_ptr()
+                (save if kind == "save" else train).append(P)
     run("fmha_nvfuser_BH512_S128_D64_full_mask", infer, 4 * bh * s * d * 2 + bh * s * s * 2, "6 sets rotated")
     run("fmha_train_nvfuser_BH512_S128_D64_full_masks", train, 4 * bh * s * d * 2 + 2 * bh * s * s * 2,
         "6 sets rotated")
-    del keep, infer, train
+    run("fmha_train_saveim_nvfuser_BH512_S128_D64_full_masks", save, 4 * bh * s * d * 2 + 4 * bh * s * s * 2,
+        "6 sets rotated")
+    del keep, infer, train, save
 
     b1, h1 = 8, 12   # BERT-base forward: the configuration of the CPU baseline
     q1, k1, v1 = (torch.randn(b1 * h1, s, d, generator=g).to(torch.float16).cuda() for _ in range(3))

@@ -43,7 +43,8 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 }
 
 // Tuning overrides for experiments and tests: FMHA_FWD_QB=1|2 forces the query blocks per wave of
-// the forward, FMHA_BWD_PAIR=0|1 the pairing of causal tiles in the backward.
+// the forward, FMHA_FWD_SHORT=0 keeps short key ranges off the one-pass kernel, FMHA_BWD_PAIR=0|1
+// the pairing of causal tiles in the backward.
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
   return e ? std::atoi(e) : dflt;
@@ -200,6 +201,13 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   v.causal = p->causal != 0;
   v.drop = (p->drop_kind == FMHA_DROP_TENSOR || saving) ? 2 : (p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0);
   v.saving = saving;
+  // Short key ranges under a full mask tensor run in one pass with whole-row accesses to the
+  // [.., sq, sk] tensors, which must then start on 16-byte boundaries row by row.
+  v.short_keys = !strided && p->d == 64 && p->sk <= 128 && (p->sk % 8) == 0 && v.mask == kMaskFull && !v.causal &&
+                 v.drop != 1 && !p->kv_len && aligned16(a.mask) && (a.mask_sb % 8) == 0 && (a.mask_sq % 8) == 0 &&
+                 (!a.drop_mask || aligned16(a.drop_mask)) && (!a.save_softmax || aligned16(a.save_softmax)) &&
+                 (!a.save_dropout || aligned16(a.save_dropout)) && (!saving || a.drop_mask) &&
+                 env_int("FMHA_FWD_SHORT", 1) != 0;
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
   // flop.  That pays (4-6 % measured) for the unmasked variant at head dim 64 on long key
   // ranges when there is enough work for every resident workgroup to get several 256-query

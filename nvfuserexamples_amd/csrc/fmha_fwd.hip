@@ -2,6 +2,15 @@
 // with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1}, and exports its dispatcher.
 #include "fmha_launch.h"
 #include "fmha_fwd_pipe.h"
+#ifndef FMHA_TU_STRIDED
+#define FMHA_TU_STRIDED 0
+#endif
+#if FMHA_TU_D == 64 && !FMHA_TU_STRIDED
+#define FMHA_TU_SHORT 1
+#include "fmha_fwd_short.h"
+#else
+#define FMHA_TU_SHORT 0
+#endif
 
 #if FMHA_TU_BF16
 #define FMHA_TU_T __bf16
@@ -9,9 +18,6 @@
 #else
 #define FMHA_TU_T _Float16
 #define FMHA_TU_TNAME f16
-#endif
-#ifndef FMHA_TU_STRIDED
-#define FMHA_TU_STRIDED 0
 #endif
 #if FMHA_TU_STRIDED
 #define FMHA_CAT3(a, b, c) a##b##_d##c##_strided
@@ -63,6 +69,22 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
+#if FMHA_TU_SHORT
+// short key ranges under a full mask tensor (the reference's operators at their own shape)
+template <bool DROPT, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
+  auto kern = fmha_fwd_short_kernel<FMHA_TU_T, DROPT, SAVE>;
+  static const bool ready = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                ShortCfg::LDS_BYTES) == hipSuccess;
+  if (!ready) return 2;
+  a.nqt = (a.sq + ShortCfg::QT - 1) / ShortCfg::QT;
+  const long long nblk = (long long)a.bh * a.nqt;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(ShortCfg::NW * 64), ShortCfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+#endif
+
 template <int QB, int MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<QB, MASK, CAUSAL, 0>(a, s);
   if (drop == 1) return launch<QB, MASK, CAUSAL, 1>(a, s);
@@ -94,6 +116,14 @@ template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 #if defined(FMHA_DEV_MINIMAL) || FMHA_TU_STRIDED
   if (v.drop == 2 || v.qb == 2) return 1; // folded layout only
+#endif
+#if FMHA_TU_SHORT
+  if (v.short_keys) {
+    if (v.saving) return launch_short<true, true>(a, s);
+    return v.drop == 2 ? launch_short<true, false>(a, s) : launch_short<false, false>(a, s);
+  }
+#else
+  if (v.short_keys) return 1;
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;

@@ -1,0 +1,276 @@
+// Forward kernel for short key ranges (sk <= 128) under a full [.., sq, sk] mask tensor: the shape
+// class of the reference's three operators, which take [512,128,64] tensors with [512,128,128]
+// masks (reference fmha/fmha_manual.cpp:39-47, test.py:20-23) and optionally return the
+// normalised softmax and its dropped copy (fmha/fmha_manual.cpp:891-897).
+//
+// At these shapes the operators move 50-100 MB for 2 GFLOP: the time is memory time, and most of
+// the bytes are the [.., sq, sk] tensors (mask, dropout mask, the two saved outputs).  So this
+// kernel is organised around them rather than around the matrix pipe:
+//   * one pass: the scores of a wave's 32 queries against ALL keys stay in registers (4 accumulator
+//     blocks), so the softmax is exact (true row maximum, fp32 sum) and nothing is read twice;
+//   * every load of the workgroup is requested up front (K and V as global->LDS copies, then Q, mask
+//     and dropout rows into registers) and consumed in that order: the first product runs while the
+//     mask rows arrive, the softmax while the dropout rows arrive, and stores start only after the
+//     last load has been used;
+//   * mask and dropout rows are read, and the saved outputs written, as whole 256-byte rows
+//     (16 bytes per lane, 16 lanes per row).  The MFMA accumulator layout wants the opposite
+//     (lane = query row, 8-byte pieces), which as a global access pattern touches 32 different
+//     cache lines per instruction; a wave-private LDS scratch turns one layout into the other.
+// The second product takes the dropped, normalised probabilities -- the very values of the
+// saved "dropout" output -- as its operand, as the reference does (fmha/fmha_manual.cpp:478-490).
+#pragma once
+#include "fmha_fwd_kernel.h"
+
+namespace fmha {
+
+struct ShortCfg {
+  static constexpr int D = 64;
+  static constexpr int NW = 4;                      // waves per workgroup, 32 queries each (two-wave workgroups measured 15-20 % slower)
+  static constexpr int QT = NW * 32;
+  static constexpr int SKMAX = 128;
+  static constexpr int NSB = SKMAX / 32;            // 32-key accumulator blocks
+  static constexpr int BT = 64;                     // rows per swizzled LDS tile
+  static constexpr int TILEB = BT * D * 2;
+  static constexpr int SCR_PITCH = SKMAX * 2 + 16;  // scratch row pitch: 16 bytes of padding per row
+  static constexpr int SCR_BYTES = 32 * SCR_PITCH;
+  static constexpr int LDS_BYTES = 4 * TILEB + NW * SCR_BYTES; // K, V (two tiles each) + one scratch per wave
+};
+
+template <typename T, bool DROPT, bool SAVE>
+__global__ __launch_bounds__(ShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void fmha_fwd_short_kernel(const FwdArgs a) {
+  using E = Elem<T>;
+  using v8 = typename E::v8;
+  using v4 = typename E::v4;
+  using C = ShortCfg;
+  constexpr int D = C::D, KS = D / 16, DB = D / 32, NSB = C::NSB, NT = C::NW * 64;
+  constexpr int TILEB = C::TILEB, PITCH = C::SCR_PITCH;
+  constexpr float NEG_INF = -__builtin_inff();
+
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int w = tid >> 6;
+  const int l = tid & 63;
+  const int ql = l & 31;
+  const int h = l >> 5;
+
+  // one XCD (one L2) owns a contiguous range of (head, query tile) pairs
+  int bid = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
+  const int bh = bid / a.nqt;
+  const int qt = bid - bh * a.nqt;
+  const int q0w = qt * C::QT + w * 32;
+
+  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
+  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
+  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+
+  // ---- every request of this workgroup, up front
+  TileCopy<T, D, C::BT, NT> tcopy;
+  tcopy.init(tid, D);
+  const uint32_t lds0 = lds_address(lds);
+  const bool two_tiles = a.sk > C::BT;
+  tcopy.issue(Kb, 0, a.sk, lds0, tid);
+  if (two_tiles) tcopy.issue(Kb, C::BT, a.sk, lds0 + TILEB, tid);
+  tcopy.issue(Vb, 0, a.sk, lds0 + 2 * TILEB, tid);
+  if (two_tiles) tcopy.issue(Vb, C::BT, a.sk, lds0 + 3 * TILEB, tid);
+
+  v8 qreg[KS];
+  {
+    int q = q0w + ql;
+    q = q < a.sq ? q : a.sq - 1;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qreg[ks] = as_v8<T>(*(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8));
+  }
+
+  // [.., sq, sk] rows as the wave reads and writes them: instruction i covers rows 4i .. 4i+3 of the
+  // wave's 32, sixteen lanes per row, 8 keys (16 bytes) per lane
+  const int rsub = l >> 4;
+  const int chunk = l & 15;
+  const bool cvalid = chunk * 8 < a.sk;
+  u32x4 mreg[8], dreg[8];
+  {
+    const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + chunk * 8;
+    const T *db_ = DROPT ? (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk + chunk * 8 : nullptr;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    int qrow[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = q0w + 4 * i + rsub;
+      qrow[i] = q < a.sq ? q : a.sq - 1;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mreg[i] = cvalid ? *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq) : z;
+    if (DROPT) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dreg[i] = cvalid ? *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk) : z;
+    }
+  }
+  // Loads complete in the order they were requested.  The K and V copies went out first: once at most
+  // the 4 Q, 8 mask and 8 dropout-row loads requested after them are outstanding, they have landed;
+  // the first product then runs while the [.., sq, sk] rows are still on their way.  (Lanes whose
+  // chunk lies past sk skip their row loads together, as a branch around all of them or as a masked
+  // load that is still counted; either way no more than these loads follow the copies.)
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + 8 + (DROPT ? 8 : 0)) : "memory");
+  __syncthreads();
+
+  PanelLane pl;
+  pl.init(l);
+  char *scr = lds + 4 * TILEB + w * C::SCR_BYTES;
+  char *scr_row = scr + (rsub * PITCH + chunk * 16); // + 4i rows: this lane's 16 bytes of instruction i
+  char *scr_frag = scr + (ql * PITCH + h * 8);       // + 64 sb + 16 g: this lane's 8-byte piece (sb, g)
+  // The scratch belongs to one wave, whose LDS accesses execute in order: between the two layouts
+  // it is enough to keep the compiler from moving accesses across.
+  auto scratch_turn = [] {
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  // ---- x^T = K . Q^T for all keys (lane = query, registers = keys 32 sb + 8g + 4h + t)
+  f32x16 x[NSB];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x[sb][r] = 0.f;
+    if (sb * 32 < a.sk) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        x[sb] = E::mfma(panel_read_rows<T, C::BT>(lds + (sb >> 1) * TILEB, pl, sb & 1, ks), qreg[ks], x[sb]);
+    }
+  }
+
+  // ---- scale and mask (log2 units); keys past the end drop out
+#pragma unroll
+  for (int i = 0; i < 8; ++i) *(u32x4 *)(scr_row + 4 * i * PITCH) = mreg[i];
+  scratch_turn();
+  float mx = NEG_INF;
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const v4 mv = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int kk = sb * 32 + 8 * g + 4 * h + t;
+        float xv = fmaf(x[sb][4 * g + t], a.scale_l2, fmaf((float)mv[t], a.mask_a, a.mask_b));
+        xv = kk < a.sk ? xv : NEG_INF;
+        x[sb][4 * g + t] = xv;
+        mx = fmaxf(mx, xv);
+      }
+    }
+  scratch_turn();
+  mx = xhalf_max(mx);
+  const float mref = mx == NEG_INF ? 0.f : mx;
+
+  // ---- exact softmax of the row
+  float sum = 0.f;
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = fast_exp2(x[sb][r] - mref);
+      x[sb][r] = p;
+      sum += p;
+    }
+  const float lt = xhalf_sum(sum);
+  const float inv = lt > 0.f ? 1.f / lt : 0.f;
+
+  // rows of the scratch leave as whole rows of a [.., sq, sk] output
+  auto store_rows = [&](void *out) {
+    T *ob = (T *)out + (size_t)bh * a.sq * a.sk + chunk * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = q0w + 4 * i + rsub;
+      const u32x4 t = *(const u32x4 *)(scr_row + 4 * i * PITCH);
+      if (cvalid && q < a.sq) *(u32x4 *)(ob + (size_t)q * a.sk) = t;
+    }
+  };
+  auto put_piece = [&](int sb, int g, const v4 &piece) {
+    Pack8 pk;
+    if constexpr (__is_same(T, _Float16)) pk.h = piece;
+    else pk.b = piece;
+    *(u32x2 *)(scr_frag + sb * 64 + g * 16) = pk.u;
+  };
+
+  // ---- dropped, normalised probabilities in the element type: second operand and saved output.
+  // (The dropout rows are the last loads to arrive; nothing is stored before they are consumed, so
+  // that waiting for them never waits for a store.)
+  if (DROPT) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *(u32x4 *)(scr_row + 4 * i * PITCH) = dreg[i];
+    scratch_turn();
+  }
+  v8 pfrag[NSB][2];
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float keep[4] = {a.drop_scale, a.drop_scale, a.drop_scale, a.drop_scale};
+      if (DROPT) {
+        const v4 dm = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) keep[t] = (float)dm[t] * a.drop_scale;
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)((x[sb][4 * g + t] * inv) * keep[t]);
+    }
+  scratch_turn();
+
+  if (SAVE && a.save_softmax) {
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        v4 s4;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) s4[t] = (T)(x[sb][4 * g + t] * inv);
+        put_piece(sb, g, s4);
+      }
+    scratch_turn();
+    store_rows(a.save_softmax);
+    scratch_turn();
+  }
+  if (SAVE && a.save_dropout) {
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        v4 d4;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) d4[t] = pfrag[sb][g >> 1][4 * (g & 1) + t];
+        put_piece(sb, g, d4);
+      }
+    scratch_turn();
+    store_rows(a.save_dropout);
+  }
+
+  // ---- O^T = V^T . P^T
+  f32x16 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb) {
+    if (sb * 32 < a.sk) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          o[db] = E::mfma(panel_read_transposed<T, C::BT>(lds + (2 + (sb >> 1)) * TILEB, pl, sb & 1, db, c),
+                          pfrag[sb][c], o[db]);
+    }
+  }
+
+  const int q = q0w + ql;
+  if (q < a.sq) {
+    T *Ob = (T *)a.o + ((size_t)bh * a.sq + q) * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + db * 32, o[db], 1.f, h);
+    if (a.lse && h == 0) a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
+  }
+}
+
+} // namespace fmha

@@ -16,6 +16,7 @@ struct FwdVariant {
   bool causal;
   int drop;     // 0 none, 1 Philox, 2 tensor / save-intermediates
   bool saving;  // drop == 2: the save-intermediates pass is wanted (plain kernel only)
+  bool short_keys; // sk <= 128 under an aligned full mask tensor: the one-pass kernel (head dim 64, folded layout)
 };
 
 // Return 0 on success, 1 if the variant is not built, 2 if the launch failed.

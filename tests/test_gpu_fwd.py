@@ -149,6 +149,67 @@ def test_train_ops_and_saved_intermediates():
     assert torch.equal(o2, o)  # the save pass does not disturb O
 
 
+# Key ranges of at most 128 keys under a full mask tensor whose rows start on 16-byte boundaries run on a
+# one-pass kernel of their own (exact row maximum, whole-row accesses to the [.., sq, sk] tensors): the
+# reference's three operators at their own shape.  FMHA_FWD_SHORT=0 keeps the same calls on the general
+# kernels; both must meet the oracle.
+SHORT = [
+    # bh, sq, sk, dtype, mode
+    (4, 128, 128, "fp16", "infer"),     # the reference's inference operator (0/1 mask -> (1-m) * -10000)
+    (4, 128, 40, "fp16", "infer"),      # one partly filled key block
+    (6, 33, 64, "fp16", "train"),       # ragged query rows, dropout tensor
+    (5, 200, 96, "fp16", "save"),       # two query tiles, three key blocks
+    (3, 77, 8, "fp16", "save"),         # a single 16-byte chunk per row
+    (4, 300, 128, "bf16", "save"),
+    (600, 128, 128, "fp16", "train"),   # more workgroups than the device holds at once
+    (6, 160, 128, "fp16", "bcast"),     # [B,1,sq,sk] mask shared by the heads of a batch entry, -inf entries, LSE
+]
+
+
+@pytest.mark.parametrize("short", ["1", "0"])
+@pytest.mark.parametrize("bh,sq,sk,dtype,mode", SHORT)
+def test_short_key_ranges_under_full_masks(bh, sq, sk, dtype, mode, short, monkeypatch):
+    monkeypatch.setenv("FMHA_FWD_SHORT", short)
+    q, k, v = make_qkv(bh, sq, sk, 64, seed=bh + sk, dtype=dtype)
+    g = torch.Generator().manual_seed(sq + sk)
+    tol = TOL[dtype]
+    if mode == "infer":
+        m = torch.empty(bh, sq, sk).random_(2, generator=g).to(TDT[dtype])
+        o, lse, _, _ = _run(q, k, v, mask=m.cuda(), mask_kind=capi.MASK_KEEP01, want_lse=True)
+        ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), mask_kind="keep01", want=("o", "lse"))
+        assert np.abs(f32(o.cpu()) - ref["o"]).max() <= tol
+        assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= LSE_TOL[dtype]
+        return
+    if mode == "bcast":
+        m = torch.randn(bh // 3, 1, sq, sk, generator=g) * 2
+        m[:, :, :, 5::7] = float("-inf")
+        m[0, 0, 3, :] = float("-inf")          # a query that sees no key at all: O = 0, LSE = -inf
+        m = m.to(TDT[dtype])
+        o, lse, _, _ = _run(q, k, v, mask=m.cuda(), want_lse=True)
+        ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), want=("o", "lse"))
+        assert np.abs(f32(o.cpu()) - ref["o"]).max() <= tol
+        got = lse.cpu().numpy()
+        dead = np.isneginf(ref["lse"])
+        assert dead.any() and np.array_equal(np.isneginf(got), dead)
+        assert np.abs(got[~dead] - ref["lse"][~dead]).max() <= LSE_TOL[dtype]
+        assert (f32(o.cpu())[dead] == 0).all()
+        return
+    pm = (torch.empty(bh, sq, sk).random_(2, generator=g) * -1000).to(TDT[dtype])
+    dm = torch.empty(bh, sq, sk).random_(2, generator=g).to(TDT[dtype])
+    o, _, sm, dr = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0,
+                        save=(mode == "save"))
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(pm), drop_mask=f32(dm), drop_scale=2.0,
+                           want=("o", "softmax", "dropout"))
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= 2 * tol   # O is up to 2x larger here (x2 scaling)
+    if mode == "save":
+        assert np.abs(f32(sm.cpu()) - ref["softmax"]).max() <= tol / 2
+        assert np.abs(f32(dr.cpu()) - ref["dropout"]).max() <= tol
+        live = ref["softmax"] > 1e-6
+        assert np.array_equal((f32(dr.cpu()) == 0)[live], (f32(dm) == 0)[live])
+        o2, _, _, _ = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0)
+        assert torch.equal(o2, o)  # saving does not disturb O
+
+
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,mask", [
     (6, 200, 333, 64, "fp16", "pad"),        # ragged tiles, per-key mask
     (4, 192, 192, 64, "bf16", "add_full"),   # full mask tensor and dropout tensor together
