@@ -280,15 +280,37 @@ void set_mask_and_dropout(P &p, MaskLayout &m, const c10::optional<at::Tensor> &
   }
 }
 
+
+// Head dims the kernels are not built for (anything but 64 and 128, up to 128) run zero-padded to
+// the next built size: zero columns add nothing to Q.K^T, the padded columns of V give zero columns
+// of O (and zero columns of dO leave the other gradients untouched), so results are those of the
+// original head dim.  Costs a copy of every operand and the arithmetic on the padding.
+int64_t padded_head_dim(int64_t d) {
+  TORCH_CHECK(d >= 1 && d <= 128, "mha_manual: head dim must be in [1, 128], got ", d);
+  return d <= 64 ? 64 : 128;
+}
+at::Tensor pad_head_dim(const at::Tensor &x, int64_t to) {
+  return at::constant_pad_nd(x, {0, to - x.size(-1)}, 0);
+}
+
 // q, k, v: [B*H,S,D] contiguous (the reference's layout) or [B,H,S,D] views of any batch / head /
 // row strides (e.g. x.view(B,S,H,D).transpose(1,2), or a slice of a packed QKV projection), read
-// in place.  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
+// in place (D = 64 or 128; other head dims up to 128 are padded, see above).  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
 // (seed, offset); p_drop == 0 disables dropout.  Returns (O, LSE fp32): O in q's shape and
 // dimension order, LSE [B*H,Sq] or [B,H,Sq].
 std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,
                                             const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
                                             double p_drop, int64_t seed, int64_t offset,
                                             const c10::optional<at::Tensor> &kv_len) {
+  TORCH_CHECK(q_.dim() >= 3 && k_.dim() == q_.dim() && v_.dim() == q_.dim() && k_.size(-1) == q_.size(-1) &&
+                  v_.size(-1) == q_.size(-1),
+              "mha_manual: q, k, v must be [B*H,S,D] or [B,H,S,D] with one head dim");
+  if (const int64_t d = q_.size(-1), dp = padded_head_dim(d); dp != d) {
+    auto [o, lse] = fmha_fwd(pad_head_dim(q_, dp), pad_head_dim(k_, dp), pad_head_dim(v_, dp), mask,
+                             scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(d)), is_causal, p_drop, seed,
+                             offset, kv_len);
+    return std::make_tuple(o.narrow(-1, 0, d).contiguous(), lse);
+  }
   const RowsOf q = rows_of(q_, "q");
   RowsOf k = rows_of(k_, "k"), v = rows_of(v_, "v");
   same_row_pitch(k, v);
@@ -331,6 +353,17 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor>
 fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,
          const at::Tensor &o_, const at::Tensor &lse, const c10::optional<at::Tensor> &mask, double scale,
          bool is_causal, double p_drop, int64_t seed, int64_t offset, const c10::optional<at::Tensor> &kv_len) {
+  TORCH_CHECK(q_.dim() >= 3 && k_.dim() == q_.dim() && v_.dim() == q_.dim() && k_.size(-1) == q_.size(-1) &&
+                  v_.size(-1) == q_.size(-1) && dout_.sizes() == q_.sizes() && o_.sizes() == q_.sizes(),
+              "mha_manual: q, k, v must be [B*H,S,D] or [B,H,S,D] with one head dim, dout and o shaped like q");
+  if (const int64_t d = q_.size(-1), dp = padded_head_dim(d); dp != d) {
+    auto [dq, dk, dv] = fmha_bwd(pad_head_dim(dout_, dp), pad_head_dim(q_, dp), pad_head_dim(k_, dp),
+                                 pad_head_dim(v_, dp), pad_head_dim(o_, dp), lse, mask,
+                                 scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(d)), is_causal, p_drop, seed,
+                                 offset, kv_len);
+    return std::make_tuple(dq.narrow(-1, 0, d).contiguous(), dk.narrow(-1, 0, d).contiguous(),
+                           dv.narrow(-1, 0, d).contiguous());
+  }
   const RowsOf q = rows_of(q_, "q");
   RowsOf k = rows_of(k_, "k"), v = rows_of(v_, "v");
   same_row_pitch(k, v);
