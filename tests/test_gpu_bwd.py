@@ -140,3 +140,53 @@ def test_causal_tile_pairing_is_bit_identical(bh, sq, sk, d, dtype, p, monkeypat
         torch.cuda.synchronize()
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+FULL_SIZE = [
+    # B, H, S, D, dtype, causal, p_drop, std          (the other train configurations, at full size)
+    (4, 16, 2048, 64, "fp16", False, 0.1, 1.0),       # long sequences, Philox dropout, no mask
+    (16, 32, 1024, 128, "bf16", True, 0.0, 0.5),      # wide heads, bf16, causal
+]
+
+
+@pytest.mark.parametrize("B,H,S,D,dtype,causal,p,std", FULL_SIZE)
+def test_train_step_properties_at_full_size(B, H, S, D, dtype, causal, p, std):
+    """Size-independent checks of forward + backward at the full size of the long-sequence and the
+    wide-head configuration, plus oracle parity on the first two heads (the oracle draws its keep
+    decisions by absolute head index, so heads 0 and 1 of the batch are heads 0 and 1 there)."""
+    bh = B * H
+    tdt = TDT[dtype]
+    q, k, v, do = make_qkv(bh, S, S, D, seed=3, std=std, dtype=dtype, with_dout=True)
+    kw = dict(causal=causal)
+    okw = dict(causal=causal)
+    if p:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=0x1234, offset=0)
+        okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=0x1234, offset=0)
+    qc, kc, vc, dc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o, lse, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    dq, dk, dv = capi.bwd(dc, qc, kc, vc, o, lse, **kw)
+    gtol = 1e-2 if dtype == "fp16" else 3e-2
+    # gradients are linear in dO (doubling is exact in both element types)
+    g2 = capi.bwd((dc.float() * 2).to(tdt), qc, kc, vc, o, lse, **kw)
+    for a, b in zip((dq, dk, dv), g2):
+        assert (b.float() - 2 * a.float()).abs().max().item() <= gtol * b.float().abs().max().item()
+    # sum_q dQ.Q == sum_k dK.K per head (the scores are bilinear in q and k)
+    lhs = (dq.float() * qc.float()).sum((1, 2))
+    rhs = (dk.float() * kc.float()).sum((1, 2))
+    assert (lhs - rhs).abs().max().item() <= 2 * gtol * lhs.abs().max().item()
+    if causal:
+        # the future does not reach the past: new K, V rows at the end leave earlier queries' O bit for bit
+        cut = S - 100
+        k2, v2 = kc.clone(), vc.clone()
+        k2[:, cut:] = 1.0
+        v2[:, cut:] = -3.0
+        o2 = capi.fwd(qc, k2, v2, **kw)[0]
+        assert torch.equal(o2[:, :cut], o[:, :cut])
+        assert not torch.equal(o2[:, cut:], o[:, cut:])
+    torch.cuda.synchronize()
+    heads = [0, 1]
+    ref = oracle.attention(f32(q[heads]), f32(k[heads]), f32(v[heads]), dout=f32(do[heads]),
+                           want=("o", "dq", "dk", "dv"), **okw)
+    assert np.abs(f32(o[heads].cpu()) - ref["o"]).max() <= (2e-3 if dtype == "fp16" else 2e-2)
+    for name, t in zip(("dq", "dk", "dv"), (dq, dk, dv)):
+        assert rel_to_max(f32(t[heads].cpu()), ref[name]) <= gtol, name
