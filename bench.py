@@ -181,6 +181,40 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
     return legs
 
 
+def operator_legs(torch, steps, warmup):
+    """The reference's three operators as a caller sees them (torch.ops.mha_manual.*, outputs
+    allocated per call) at the reference's shape, timed per call on the host clock: called eagerly
+    back to back, and replayed from a captured HIP graph.  One input set (the point is the host's
+    share, not HBM): a launch lasts 15-25 us here, about what dispatching an operator costs."""
+    from nvfuserexamples_amd import load_ops
+    ops = load_ops()
+    bh, s, d = 512, 128, 64
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = (torch.randn((bh, s, d), dtype=torch.float16, device="cuda", generator=g) for _ in range(3))
+    amask = torch.empty((bh, s, s), device="cuda").random_(2, generator=g).half()
+    pad = torch.empty((bh, s, s), device="cuda").random_(2, generator=g).half() * -1000
+    dm = torch.empty((bh, s, s), device="cuda").random_(2, generator=g).half()
+    calls = {"fmha_nvfuser": lambda: ops.fmha_nvfuser(q, k, v, amask),
+             "fmha_train_nvfuser": lambda: ops.fmha_train_nvfuser(q, k, v, pad, dm),
+             "fmha_train_saveim_nvfuser": lambda: ops.fmha_train_saveim_nvfuser(q, k, v, pad, dm)}
+    legs = {}
+    for name, fn in calls.items():
+        _, eager_ms = time_steps(torch, lambda i: fn(), steps, warmup)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep = fn()
+        _, graph_ms = time_steps(torch, lambda i: graph.replay(), steps, warmup)
+        legs[name] = {"eager_us_per_call": round(eager_ms * 1e3, 2), "graph_replay_us_per_call": round(graph_ms * 1e3, 2)}
+        del graph, keep
+    return legs
+
+
 def power_probe(torch, step, seconds=2.0):
     """Socket power and graphics clocks as the board's management firmware reports them (amd-smi),
     sampled while `step` runs back to back on a second thread.  The attention kernels are
@@ -413,6 +447,7 @@ def main():
     }
 
     out["short_sequences"] = short_sequence_legs(torch, capi, L, stream, args.steps, args.warmup)
+    out["operators_BH512_S128_D64"] = operator_legs(torch, args.steps, args.warmup)
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
