@@ -162,6 +162,46 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
         "6 sets rotated")
     del keep, infer, train, save
 
+    # train step at the same short shape (the reference has no backward): [B,1,1,S] padding mask, Philox
+    # dropout; forward with LSE, then the one-launch short-sequence backward
+    bb = 32
+    tkeep, tsteps = [], []
+    for _ in range(6):
+        t = {n: torch.randn(bh, s, d, generator=g).to(torch.float16).cuda() for n in ("q", "k", "v", "dout")}
+        for n in ("o", "dq", "dk", "dv"):
+            t[n] = torch.empty_like(t["q"])
+        t["lse"], t["delta"] = (torch.empty(bh, s, dtype=torch.float32, device="cuda") for _ in range(2))
+        m = torch.zeros(bb, 1, 1, s)
+        for i in range(bb):
+            m[i, 0, 0, 64 + 2 * i:] = -10000.0
+        t["mask"] = m.to(torch.float16).cuda()
+        F, Bp = capi.FwdParams(), capi.BwdParams()
+        for P in (F, Bp):
+            P.q, P.k, P.v, P.o, P.lse = (t[n].data_ptr() for n in ("q", "k", "v", "o", "lse"))
+            P.bh, P.sq, P.sk, P.d = bh, s, s, d
+            P.dtype, P.scale = capi.F16, 0.125
+            P.mask, P.mask_kind = t["mask"].data_ptr(), capi.MASK_ADDITIVE
+            P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = bh // bb, s, 0
+            P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, 0.1, 1.0 / 0.9, 0x1234, 0
+        Bp.dout, Bp.delta, Bp.dq, Bp.dk, Bp.dv = (t[n].data_ptr() for n in ("dout", "delta", "dq", "dk", "dv"))
+        tkeep.append(t)
+        tsteps.append((F, Bp))
+
+    def train_step(i):
+        F, Bp = tsteps[i % len(tsteps)]
+        L.fmha_fwd_launch(C.byref(F), stream)
+        L.fmha_bwd_launch(C.byref(Bp), stream)
+    capi.check(L.fmha_fwd_launch(C.byref(tsteps[0][0]), stream))
+    capi.check(L.fmha_bwd_launch(C.byref(tsteps[0][1]), stream))
+    ms, _ = time_steps(torch, train_step, steps, warmup)
+    nbytes = 12 * bh * s * d * 2 + 3 * bh * s * 4 + bb * s * 2 * 2
+    legs["train_step_BH512_S128_D64_pad_mask_dropout"] = {
+        "us": round(ms * 1e3, 2), "algorithmic_MB": round(nbytes / 1e6, 2),
+        "hbm_GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+        "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+        "tflops": round(14.0 * bh * s * s * d / (ms * 1e-3) / 1e12, 2), "inputs": "6 sets rotated"}
+    del tkeep, tsteps
+
     b1, h1 = 8, 12   # BERT-base forward: the configuration of the CPU baseline
     q1, k1, v1 = (torch.randn(b1 * h1, s, d, generator=g).to(torch.float16).cuda() for _ in range(3))
     o1 = torch.empty_like(q1)

@@ -1,6 +1,15 @@
 // Instantiates the backward kernels for one (element type, head dim, row layout kind) triple, chosen
 // with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1}, and exports their dispatcher.
 #include "fmha_launch.h"
+#ifndef FMHA_TU_STRIDED
+#define FMHA_TU_STRIDED 0
+#endif
+#if FMHA_TU_D == 64 && !FMHA_TU_STRIDED
+#define FMHA_TU_SHORT 1
+#include "fmha_bwd_short.h"
+#else
+#define FMHA_TU_SHORT 0
+#endif
 
 #if FMHA_TU_BF16
 #define FMHA_TU_T __bf16
@@ -8,9 +17,6 @@
 #else
 #define FMHA_TU_T _Float16
 #define FMHA_TU_TNAME f16
-#endif
-#ifndef FMHA_TU_STRIDED
-#define FMHA_TU_STRIDED 0
 #endif
 #if FMHA_TU_STRIDED
 #define FMHA_CAT3(a, b, c) a##b##_d##c##_strided
@@ -68,6 +74,17 @@ template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipS
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
+#if FMHA_TU_SHORT
+// sq, sk <= 128: one workgroup per head computes dQ, dK and dV from one copy of the head in LDS
+template <int DROP> int launch_short(BwdArgs &a, hipStream_t s) {
+  auto kern = fmha_bwd_short_kernel<FMHA_TU_T, DROP>;
+  static const int attr = set_lds(kern, BwdShortCfg::LDS_BYTES);
+  if (attr) return 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)a.bh), dim3(BwdShortCfg::NW * 64), BwdShortCfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+#endif
+
 template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
   if (v.drop == 0) return launch<MASK, CAUSAL, 0>(a, v.pair, s);
   if (v.drop == 1) return launch<MASK, CAUSAL, 1>(a, v.pair, s);
@@ -77,6 +94,11 @@ template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, const BwdVariant &v, hi
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
+#if FMHA_TU_SHORT
+  if (v.short_seq) return v.drop == 1 ? launch_short<1>(a, s) : launch_short<0>(a, s);
+#else
+  if (v.short_seq) return 1;
+#endif
   if (v.mask == kMaskPerKey)
     return v.causal ? by_drop<kMaskPerKey, true>(a, v, s) : by_drop<kMaskPerKey, false>(a, v, s);
   if (v.mask == kMaskFull)

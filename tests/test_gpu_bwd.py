@@ -190,3 +190,70 @@ def test_train_step_properties_at_full_size(B, H, S, D, dtype, causal, p, std):
     assert np.abs(f32(o[heads].cpu()) - ref["o"]).max() <= (2e-3 if dtype == "fp16" else 2e-2)
     for name, t in zip(("dq", "dk", "dv"), (dq, dk, dv)):
         assert rel_to_max(f32(t[heads].cpu()), ref[name]) <= gtol, name
+
+
+# Heads of at most 128 queries and 128 keys (head dim 64, no causal or full mask) take one launch:
+# the workgroup copies Q, K, V and dO into LDS once and computes dQ, then dK and dV, from that copy.
+# FMHA_BWD_SHORT=0 keeps the same calls on the two general kernels; both must meet the oracle.
+SHORT_SEQ = [
+    # bh, sq, sk, dtype, mask, p_drop, kv_len
+    (4, 128, 128, "fp16", None, 0.0, False),
+    (6, 128, 128, "fp16", "pad", 0.1, False),       # BERT-base train step shape (few heads)
+    (3, 100, 77, "fp16", None, 0.1, False),         # ragged in both directions
+    (5, 33, 128, "bf16", "pad", 0.1, False),        # queries fill one wave and a bit
+    (4, 128, 40, "fp16", "pad", 0.0, False),        # keys fill one wave and a bit: two waves idle in the second phase
+    (4, 64, 64, "fp16", "inf", 0.2, False),         # one LDS tile per matrix; -inf mask entries
+    (2, 1, 1, "fp16", None, 0.0, False),
+    (600, 128, 128, "fp16", "pad", 0.1, False),     # more workgroups than the device holds at once
+    (8, 96, 128, "fp16", None, 0.1, True),          # valid key counts
+]
+
+
+@pytest.mark.parametrize("short", ["1", "0"])
+@pytest.mark.parametrize("bh,sq,sk,dtype,mask,p,use_len", SHORT_SEQ)
+def test_short_sequences_backward(bh, sq, sk, dtype, mask, p, use_len, short, monkeypatch):
+    monkeypatch.setenv("FMHA_BWD_SHORT", short)
+    q, k, v, do = make_qkv(bh, sq, sk, 64, seed=bh + sk, dtype=dtype, with_dout=True)
+    m = None
+    if mask == "pad":
+        m = pad_mask(bh // 2 if bh % 2 == 0 else 1, sk, max(1, sk // 2), sk)
+    elif mask == "inf":
+        m = torch.randn(bh, 1, sk, generator=torch.Generator().manual_seed(sk)) * 2
+        m[:, :, 3::5] = float("-inf")
+    if m is not None:
+        m = m.to(TDT[dtype])
+    kw, okw = {}, {}
+    if p > 0:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=99, offset=12)
+        okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=99, offset=12)
+    mo = None if m is None else f32(m)
+    if use_len:
+        lens = torch.tensor([sk, 1, 5, sk // 2], dtype=torch.int32)
+        kw["kv_len"] = lens.cuda()
+        mo = np.zeros((4, 1, 1, sk), np.float32)
+        for i, n in enumerate(lens.tolist()):
+            mo[i, 0, 0, n:] = -np.inf
+    qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), (None if m is None else m.cuda())
+    o, lse, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, **kw)
+    dq, dk, dv = capi.bwd(do.cuda(), qc, kc, vc, o, lse, mask=mc, **kw)
+    torch.cuda.synchronize()
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=mo, dout=f32(do), want=("dq", "dk", "dv"), **okw)
+    for name, t in (("dq", dq), ("dk", dk), ("dv", dv)):
+        got = f32(t.cpu())
+        assert np.isfinite(got).all(), name
+        assert rel_to_max(got, ref[name], floor=1e-3) <= TOL[dtype], name
+    if use_len:
+        # keys past a sequence's count get no gradient at all, and a sequence without keys none anywhere
+        per = bh // 4
+        for i, n in enumerate(lens.tolist()):
+            sl = slice(i * per, (i + 1) * per)
+            assert not dk[sl, n:].any() and not dv[sl, n:].any()
+        # a sequence without any key: O = 0, LSE = -inf, and no gradient anywhere (nothing non-finite either)
+        lens[1] = 0
+        kw["kv_len"] = lens.cuda()
+        o, lse, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+        g0 = capi.bwd(do.cuda(), qc, kc, vc, o, lse, **kw)
+        torch.cuda.synchronize()
+        sl = slice(per, 2 * per)
+        for t in g0:
+            assert torch.isfinite(t.float()).all() and not t[sl].any()

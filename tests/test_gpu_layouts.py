@@ -48,7 +48,10 @@ CASES = [
 
 
 @pytest.mark.parametrize("b,h,sq,sk,d,dtype,causal,p,masked,packed", CASES)
-def test_strided_layouts_match_oracle_and_folded_path(b, h, sq, sk, d, dtype, causal, p, masked, packed):
+def test_strided_layouts_match_oracle_and_folded_path(b, h, sq, sk, d, dtype, causal, p, masked, packed, monkeypatch):
+    # short folded heads would otherwise take the one-launch backward, whose arithmetic differs in the last
+    # bit from the general kernels that serve strided tensors: compare like with like
+    monkeypatch.setenv("FMHA_BWD_SHORT", "0")
     bh = b * h
     q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
     kw, okw = dict(causal=causal), dict(causal=causal)
