@@ -1,8 +1,8 @@
-// Backward kernel for short sequences (sq <= 128 and sk <= 128, head dim 64): one workgroup per
+// Backward kernel for short sequences (sq and sk <= 128, or <= 256; head dim 64): one workgroup per
 // head, one launch, every tensor crosses HBM once.
 //
-// At these shapes the backward is memory time (BH 512, S 128: 5.4 GFLOP against 67 MB), and a head's
-// Q, K, V and dO fit in LDS together (64 KB).  The general path launches two kernels that each
+// At these shapes the backward is mostly memory time (BH 512, S 128: 5.4 GFLOP against 67 MB), and a head's
+// Q, K, V and dO fit in LDS together (64 KB; 128 KB at 256 rows).  The general path launches two kernels that each
 // read the head again; here the workgroup copies the four matrices into LDS once and then runs the
 // same two computations back to back on them:
 //   phase 1  lane = query (a wave owns 32 queries, walks the key blocks):
@@ -19,28 +19,32 @@
 
 namespace fmha {
 
-struct BwdShortCfg {
+// SMAX_: queries and keys per head, 128 (4 waves, 66 KB of LDS: two workgroups per CU) or 256 (8 waves,
+// 131 KB: one workgroup per CU).
+template <int SMAX_> struct BwdShortCfg {
   static constexpr int D = 64;
-  static constexpr int NW = 4;
-  static constexpr int SMAX = 128;                  // queries and keys per head
+  static constexpr int SMAX = SMAX_;
+  static constexpr int NW = SMAX / 32;              // a wave per 32 queries (phase 1) / 32 keys (phase 2)
+  static constexpr int NB = SMAX / 32;              // 32-row blocks per matrix
   static constexpr int BT = 64;                     // rows per swizzled LDS tile
+  static constexpr int NTL = SMAX / BT;             // tiles per matrix
   static constexpr int TILEB = BT * D * 2;
-  static constexpr int LDS_BYTES = 8 * TILEB + 3 * SMAX * 4; // Q, K, V, dO (two tiles each); delta, LSE, mask term
+  static constexpr int LDS_BYTES = 4 * NTL * TILEB + 3 * SMAX * 4; // Q, K, V, dO; delta, LSE, mask term
 };
 
-template <typename T, int DROP>
-__global__ __launch_bounds__(BwdShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <typename T, int DROP, int SMAX>
+__global__ __launch_bounds__(BwdShortCfg<SMAX>::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void fmha_bwd_short_kernel(const BwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
-  using C = BwdShortCfg;
-  constexpr int D = C::D, KS = D / 16, DB = D / 32, NT = C::NW * 64, TILEB = C::TILEB, BT = C::BT;
+  using C = BwdShortCfg<SMAX>;
+  constexpr int D = C::D, KS = D / 16, DB = D / 32, NT = C::NW * 64, TILEB = C::TILEB, BT = C::BT, NTL = C::NTL;
   constexpr float NEG_INF = -__builtin_inff();
   constexpr float BIG = 3.0e38f;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  char *ldsQ = lds, *ldsK = lds + 2 * TILEB, *ldsV = lds + 4 * TILEB, *ldsDO = lds + 6 * TILEB;
-  float *fD = (float *)(lds + 8 * TILEB); // delta[q]
+  char *ldsQ = lds, *ldsK = lds + NTL * TILEB, *ldsV = lds + 2 * NTL * TILEB, *ldsDO = lds + 3 * NTL * TILEB;
+  float *fD = (float *)(lds + 4 * NTL * TILEB); // delta[q]
   float *fL = fD + C::SMAX;               // LSE[q] in log2 units; +BIG for rows that must give P = 0
   float *fM = fL + C::SMAX;               // mask term of key k in log2 units; -inf past the valid keys
 
@@ -62,17 +66,16 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
   TileCopy<T, D, BT, NT> tcopy;
   tcopy.init(tid, D);
   const uint32_t lds0 = lds_address(lds);
-  tcopy.issue(Qb, 0, a.sq, lds0, tid);
-  tcopy.issue(Kb, 0, a.sk, lds0 + 2 * TILEB, tid);
-  tcopy.issue(Vb, 0, a.sk, lds0 + 4 * TILEB, tid);
-  tcopy.issue(dOb, 0, a.sq, lds0 + 6 * TILEB, tid);
-  if (a.sq > BT) {
-    tcopy.issue(Qb, BT, a.sq, lds0 + TILEB, tid);
-    tcopy.issue(dOb, BT, a.sq, lds0 + 7 * TILEB, tid);
-  }
-  if (a.sk > BT) {
-    tcopy.issue(Kb, BT, a.sk, lds0 + 3 * TILEB, tid);
-    tcopy.issue(Vb, BT, a.sk, lds0 + 5 * TILEB, tid);
+#pragma unroll
+  for (int t = 0; t < NTL; ++t) {
+    if (t * BT < a.sq) {
+      tcopy.issue(Qb, t * BT, a.sq, lds0 + t * TILEB, tid);
+      tcopy.issue(dOb, t * BT, a.sq, lds0 + (3 * NTL + t) * TILEB, tid);
+    }
+    if (t * BT < a.sk) {
+      tcopy.issue(Kb, t * BT, a.sk, lds0 + (NTL + t) * TILEB, tid);
+      tcopy.issue(Vb, t * BT, a.sk, lds0 + (2 * NTL + t) * TILEB, tid);
+    }
   }
   // this lane's part of its query's O row (for delta), in the layout of a B operand
   const int q1 = w * 32 + ql; // phase 1: the lane's query
@@ -123,7 +126,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
       for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb) {
+    for (int sb = 0; sb < C::NB; ++sb) {
       if (sb * 32 < a.sk) {
         const char *tK = ldsK + (sb >> 1) * TILEB, *tV = ldsV + (sb >> 1) * TILEB;
         f32x16 x, g;
@@ -189,7 +192,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
         dv[db][r] = 0.f;
       }
 #pragma unroll
-    for (int qb = 0; qb < 4; ++qb) {
+    for (int qb = 0; qb < C::NB; ++qb) {
       if (qb * 32 < a.sq) {
         const char *tQ = ldsQ + (qb >> 1) * TILEB, *tDO = ldsDO + (qb >> 1) * TILEB;
         f32x16 x, g;

@@ -44,7 +44,8 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 
 // Tuning overrides for experiments and tests: FMHA_FWD_QB=1|2 forces the query blocks per wave of
 // the forward, FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
-// one-pass kernels, FMHA_BWD_PAIR=0|1 sets the pairing of causal tiles in the backward.
+// one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
+// pairing of causal tiles in the backward.
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
   return e ? std::atoi(e) : dflt;
@@ -318,9 +319,11 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   v.causal = p->causal != 0;
   v.drop = p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0;
   v.pair = env_int("FMHA_BWD_PAIR", -1); // tuning / test override: 0 or 1
-  // Heads whose Q, K, V and dO fit in LDS together take one launch instead of two.
-  v.short_seq = !strided && p->d == 64 && p->sq <= 128 && p->sk <= 128 && !v.causal && v.mask != kMaskFull &&
-                env_int("FMHA_BWD_SHORT", 1) != 0;
+  // Heads whose Q, K, V and dO fit in LDS together (up to 256 queries and keys) take one launch instead of two.
+  int short_rows = env_int("FMHA_BWD_SHORT", 1); // 0: never; 1: up to 256 rows; other values: that many rows
+  if (short_rows == 1) short_rows = 256;
+  v.short_seq = !strided && p->d == 64 && p->sq <= short_rows && p->sk <= short_rows && p->sq <= 256 && p->sk <= 256 &&
+                !v.causal && v.mask != kMaskFull;
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;
   if (strided) {

@@ -192,7 +192,7 @@ def test_train_step_properties_at_full_size(B, H, S, D, dtype, causal, p, std):
         assert rel_to_max(f32(t[heads].cpu()), ref[name]) <= gtol, name
 
 
-# Heads of at most 128 queries and 128 keys (head dim 64, no causal or full mask) take one launch:
+# Heads of at most 256 queries and 256 keys (head dim 64, no causal or full mask) take one launch:
 # the workgroup copies Q, K, V and dO into LDS once and computes dQ, then dK and dV, from that copy.
 # FMHA_BWD_SHORT=0 keeps the same calls on the two general kernels; both must meet the oracle.
 SHORT_SEQ = [
@@ -206,6 +206,12 @@ SHORT_SEQ = [
     (2, 1, 1, "fp16", None, 0.0, False),
     (600, 128, 128, "fp16", "pad", 0.1, False),     # more workgroups than the device holds at once
     (8, 96, 128, "fp16", None, 0.1, True),          # valid key counts
+    # up to 256 rows: the same kernel with eight waves and 128 KB of LDS
+    (4, 256, 256, "fp16", "pad", 0.1, False),
+    (6, 197, 197, "fp16", None, 0.1, False),        # ViT-B/16 sequence length
+    (3, 130, 250, "bf16", "pad", 0.0, False),       # five query blocks against eight key blocks
+    (300, 200, 250, "fp16", "pad", 0.1, False),     # more workgroups than the device holds at once
+    (8, 256, 200, "fp16", None, 0.0, True),         # valid key counts
 ]
 
 
