@@ -76,9 +76,9 @@ template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipS
 
 #if FMHA_TU_SHORT
 // sq, sk <= 128: one workgroup per head computes dQ, dK and dV from one copy of the head in LDS
-template <int DROP, int SMAX> int launch_short(BwdArgs &a, hipStream_t s) {
+template <int DROP, int SMAX, bool CAUSAL> int launch_short(BwdArgs &a, hipStream_t s) {
   using Cfg = BwdShortCfg<SMAX>;
-  auto kern = fmha_bwd_short_kernel<FMHA_TU_T, DROP, SMAX>;
+  auto kern = fmha_bwd_short_kernel<FMHA_TU_T, DROP, SMAX, CAUSAL>;
   static const int attr = set_lds(kern, Cfg::LDS_BYTES);
   if (attr) return 2;
   hipLaunchKernelGGL(kern, dim3((unsigned)a.bh), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, a);
@@ -97,8 +97,13 @@ template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, const BwdVariant &v, hi
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
 #if FMHA_TU_SHORT
   if (v.short_seq) {
-    if (a.sq <= 128 && a.sk <= 128) return v.drop == 1 ? launch_short<1, 128>(a, s) : launch_short<0, 128>(a, s);
-    return v.drop == 1 ? launch_short<1, 256>(a, s) : launch_short<0, 256>(a, s);
+    const bool small = a.sq <= 128 && a.sk <= 128;
+    if (v.causal) {
+      if (small) return v.drop == 1 ? launch_short<1, 128, true>(a, s) : launch_short<0, 128, true>(a, s);
+      return v.drop == 1 ? launch_short<1, 256, true>(a, s) : launch_short<0, 256, true>(a, s);
+    }
+    if (small) return v.drop == 1 ? launch_short<1, 128, false>(a, s) : launch_short<0, 128, false>(a, s);
+    return v.drop == 1 ? launch_short<1, 256, false>(a, s) : launch_short<0, 256, false>(a, s);
   }
 #else
   if (v.short_seq) return 1;

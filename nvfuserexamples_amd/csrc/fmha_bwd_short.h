@@ -1,4 +1,5 @@
-// Backward kernel for short sequences (sq and sk <= 128, or <= 256; head dim 64): one workgroup per
+// Backward kernel for short sequences (sq and sk <= 128, or <= 256; head dim 64; no mask, a per-key mask
+// and / or the causal mask): one workgroup per
 // head, one launch, every tensor crosses HBM once.
 //
 // At these shapes the backward is mostly memory time (BH 512, S 128: 5.4 GFLOP against 67 MB), and a head's
@@ -32,7 +33,7 @@ template <int SMAX_> struct BwdShortCfg {
   static constexpr int LDS_BYTES = 4 * NTL * TILEB + 3 * SMAX * 4; // Q, K, V, dO; delta, LSE, mask term
 };
 
-template <typename T, int DROP, int SMAX>
+template <typename T, int DROP, int SMAX, bool CAUSAL>
 __global__ __launch_bounds__(BwdShortCfg<SMAX>::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void fmha_bwd_short_kernel(const BwdArgs a) {
   using E = Elem<T>;
@@ -127,7 +128,8 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
 
 #pragma unroll
     for (int sb = 0; sb < C::NB; ++sb) {
-      if (sb * 32 < a.sk) {
+      // causal (key <= query): key blocks above the wave's queries contribute nothing
+      if (sb * 32 < a.sk && (!CAUSAL || sb <= w)) {
         const char *tK = ldsK + (sb >> 1) * TILEB, *tV = ldsV + (sb >> 1) * TILEB;
         f32x16 x, g;
 #pragma unroll
@@ -148,7 +150,8 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
           const f32x4 mk = *(const f32x4 *)(fM + sb * 32 + 8 * gq + 4 * h);
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
-            const float p = fast_exp2(fmaf(x[4 * gq + t], a.scale_l2, mk[t]) - lq);
+            float p = fast_exp2(fmaf(x[4 * gq + t], a.scale_l2, mk[t]) - lq);
+            if (CAUSAL) p = (sb * 32 + 8 * gq + 4 * h + t <= q1) ? p : 0.f;
             float gv = g[4 * gq + t] - delta;
             if (DROP == 1)
               gv = drop_keep_byte(wd[gq], t, a.drop.thr) ? fmaf(g[4 * gq + t], a.drop_scale, -delta) : -delta;
@@ -193,7 +196,8 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
       }
 #pragma unroll
     for (int qb = 0; qb < C::NB; ++qb) {
-      if (qb * 32 < a.sq) {
+      // causal: query blocks below the wave's keys see none of them
+      if (qb * 32 < a.sq && (!CAUSAL || qb >= w)) {
         const char *tQ = ldsQ + (qb >> 1) * TILEB, *tDO = ldsDO + (qb >> 1) * TILEB;
         f32x16 x, g;
 #pragma unroll
@@ -216,7 +220,8 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
           const f32x4 Ll = *(const f32x4 *)(fL + qq);
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
-            const float p = fast_exp2(fmaf(x[4 * gq + t], a.scale_l2, mk) - Ll[t]);
+            float p = fast_exp2(fmaf(x[4 * gq + t], a.scale_l2, mk) - Ll[t]);
+            if (CAUSAL) p = (key <= qq + t) ? p : 0.f;
             float gv = g[4 * gq + t] - Dl[t];
             float pz = p;
             if (DROP == 1) {

@@ -192,32 +192,38 @@ def test_train_step_properties_at_full_size(B, H, S, D, dtype, causal, p, std):
         assert rel_to_max(f32(t[heads].cpu()), ref[name]) <= gtol, name
 
 
-# Heads of at most 256 queries and 256 keys (head dim 64, no causal or full mask) take one launch:
+# Heads of at most 256 queries and 256 keys (head dim 64, no full mask tensor) take one launch:
 # the workgroup copies Q, K, V and dO into LDS once and computes dQ, then dK and dV, from that copy.
 # FMHA_BWD_SHORT=0 keeps the same calls on the two general kernels; both must meet the oracle.
 SHORT_SEQ = [
-    # bh, sq, sk, dtype, mask, p_drop, kv_len
-    (4, 128, 128, "fp16", None, 0.0, False),
-    (6, 128, 128, "fp16", "pad", 0.1, False),       # BERT-base train step shape (few heads)
-    (3, 100, 77, "fp16", None, 0.1, False),         # ragged in both directions
-    (5, 33, 128, "bf16", "pad", 0.1, False),        # queries fill one wave and a bit
-    (4, 128, 40, "fp16", "pad", 0.0, False),        # keys fill one wave and a bit: two waves idle in the second phase
-    (4, 64, 64, "fp16", "inf", 0.2, False),         # one LDS tile per matrix; -inf mask entries
-    (2, 1, 1, "fp16", None, 0.0, False),
-    (600, 128, 128, "fp16", "pad", 0.1, False),     # more workgroups than the device holds at once
-    (8, 96, 128, "fp16", None, 0.1, True),          # valid key counts
+    # bh, sq, sk, dtype, mask, p_drop, kv_len, causal
+    (4, 128, 128, "fp16", None, 0.0, False, False),
+    (6, 128, 128, "fp16", "pad", 0.1, False, False),       # BERT-base train step shape (few heads)
+    (3, 100, 77, "fp16", None, 0.1, False, False),         # ragged in both directions
+    (5, 33, 128, "bf16", "pad", 0.1, False, False),        # queries fill one wave and a bit
+    (4, 128, 40, "fp16", "pad", 0.0, False, False),        # keys fill one wave and a bit: two waves idle in the second phase
+    (4, 64, 64, "fp16", "inf", 0.2, False, False),         # one LDS tile per matrix; -inf mask entries
+    (2, 1, 1, "fp16", None, 0.0, False, False),
+    (600, 128, 128, "fp16", "pad", 0.1, False, False),     # more workgroups than the device holds at once
+    (8, 96, 128, "fp16", None, 0.1, True, False),          # valid key counts
     # up to 256 rows: the same kernel with eight waves and 128 KB of LDS
-    (4, 256, 256, "fp16", "pad", 0.1, False),
-    (6, 197, 197, "fp16", None, 0.1, False),        # ViT-B/16 sequence length
-    (3, 130, 250, "bf16", "pad", 0.0, False),       # five query blocks against eight key blocks
-    (300, 200, 250, "fp16", "pad", 0.1, False),     # more workgroups than the device holds at once
-    (8, 256, 200, "fp16", None, 0.0, True),         # valid key counts
+    (4, 256, 256, "fp16", "pad", 0.1, False, False),
+    (6, 197, 197, "fp16", None, 0.1, False, False),        # ViT-B/16 sequence length
+    (3, 130, 250, "bf16", "pad", 0.0, False, False),       # five query blocks against eight key blocks
+    (300, 200, 250, "fp16", "pad", 0.1, False, False),     # more workgroups than the device holds at once
+    (8, 256, 200, "fp16", None, 0.0, True, False),         # valid key counts
+    # causal (key <= query): blocks above the diagonal are skipped in both phases
+    (4, 128, 128, "fp16", None, 0.0, False, True),
+    (6, 200, 200, "fp16", "pad", 0.1, False, True),
+    (3, 77, 250, "bf16", None, 0.1, False, True),   # more keys than queries: the last key blocks see no query
+    (3, 250, 100, "fp16", None, 0.0, False, True),  # more queries than keys
+    (8, 256, 256, "fp16", None, 0.1, True, True),   # causal with valid key counts
 ]
 
 
 @pytest.mark.parametrize("short", ["1", "0"])
-@pytest.mark.parametrize("bh,sq,sk,dtype,mask,p,use_len", SHORT_SEQ)
-def test_short_sequences_backward(bh, sq, sk, dtype, mask, p, use_len, short, monkeypatch):
+@pytest.mark.parametrize("bh,sq,sk,dtype,mask,p,use_len,causal", SHORT_SEQ)
+def test_short_sequences_backward(bh, sq, sk, dtype, mask, p, use_len, causal, short, monkeypatch):
     monkeypatch.setenv("FMHA_BWD_SHORT", short)
     q, k, v, do = make_qkv(bh, sq, sk, 64, seed=bh + sk, dtype=dtype, with_dout=True)
     m = None
@@ -228,7 +234,7 @@ def test_short_sequences_backward(bh, sq, sk, dtype, mask, p, use_len, short, mo
         m[:, :, 3::5] = float("-inf")
     if m is not None:
         m = m.to(TDT[dtype])
-    kw, okw = {}, {}
+    kw, okw = dict(causal=causal), dict(causal=causal)
     if p > 0:
         kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=99, offset=12)
         okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=99, offset=12)
