@@ -360,26 +360,28 @@ FMHA_DEV void drop_block(const DropCtx &c, uint32_t bh, uint32_t q4, uint32_t k4
 // ---- sharing one Philox call per 4x4 block among the four lanes that need it
 // (v_mov_b32 with a DPP quad permutation; lanes 4n..4n+3 form a quad)
 template <int CTRL> FMHA_DEV uint32_t quad_perm(uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, false);
+  // every lane of a quad is a valid source, so the previous value of the destination never shows:
+  // leave it undefined instead of clearing it first
+  return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, CTRL, 0xf, 0xf, true);
 }
 
 // 4x4 transpose inside a quad: on entry lane i holds a[0..3]; on exit a[g] is what lane g held
-// in a[i].  Two butterfly stages (partner lane ^1, then ^2).
+// in a[i].  Two butterfly stages (partner lane ^1, then ^2), written as selects so that they
+// compile to v_cndmask rather than to moves under a narrowed exec mask.
 FMHA_DEV void quad_transpose4(uint32_t a[4], int lane) {
   const bool odd = lane & 1;
   // stage 1: exchange a[1]<->a[0] and a[3]<->a[2] with the lane ^ 1
-  uint32_t s0 = odd ? a[0] : a[1];
-  uint32_t s1 = odd ? a[2] : a[3];
-  s0 = quad_perm<0xB1>(s0);
-  s1 = quad_perm<0xB1>(s1);
-  if (odd) { a[0] = s0; a[2] = s1; } else { a[1] = s0; a[3] = s1; }
-  // stage 2: exchange the (a[2],a[3]) pair of lanes 0,1 with the (a[0],a[1]) pair of lanes 2,3
+  const uint32_t s0 = quad_perm<0xB1>(odd ? a[0] : a[1]);
+  const uint32_t s1 = quad_perm<0xB1>(odd ? a[2] : a[3]);
+  const uint32_t b0 = odd ? s0 : a[0], b1 = odd ? a[1] : s0, b2 = odd ? s1 : a[2], b3 = odd ? a[3] : s1;
+  // stage 2: exchange the (2,3) pair of lanes 0,1 with the (0,1) pair of lanes 2,3
   const bool hi = lane & 2;
-  uint32_t u0 = hi ? a[0] : a[2];
-  uint32_t u1 = hi ? a[1] : a[3];
-  u0 = quad_perm<0x4E>(u0);
-  u1 = quad_perm<0x4E>(u1);
-  if (hi) { a[0] = u0; a[1] = u1; } else { a[2] = u0; a[3] = u1; }
+  const uint32_t u0 = quad_perm<0x4E>(hi ? b0 : b2);
+  const uint32_t u1 = quad_perm<0x4E>(hi ? b1 : b3);
+  a[0] = hi ? u0 : b0;
+  a[1] = hi ? u1 : b1;
+  a[2] = hi ? b2 : u0;
+  a[3] = hi ? b3 : u1;
 }
 
 // Lane = query layout.  The lane owns query q and, in one 32-key block starting at key kb32, the
