@@ -4,7 +4,7 @@
 #ifndef FMHA_TU_STRIDED
 #define FMHA_TU_STRIDED 0
 #endif
-#if FMHA_TU_D == 64 && !FMHA_TU_STRIDED
+#if FMHA_TU_D == 64
 #define FMHA_TU_SHORT 1
 #include "fmha_bwd_short.h"
 #else
@@ -78,7 +78,7 @@ template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipS
 // sq, sk <= 128: one workgroup per head computes dQ, dK and dV from one copy of the head in LDS
 template <int DROP, int SMAX, bool CAUSAL> int launch_short(BwdArgs &a, hipStream_t s) {
   using Cfg = BwdShortCfg<SMAX>;
-  auto kern = fmha_bwd_short_kernel<FMHA_TU_T, DROP, SMAX, CAUSAL>;
+  auto kern = fmha_bwd_short_kernel<FMHA_TU_T, DROP, SMAX, CAUSAL, kStrided>;
   static const int attr = set_lds(kern, Cfg::LDS_BYTES);
   if (attr) return 2;
   hipLaunchKernelGGL(kern, dim3((unsigned)a.bh), dim3(Cfg::NW * 64), Cfg::LDS_BYTES, s, a);

@@ -33,9 +33,10 @@ template <int SMAX_> struct BwdShortCfg {
   static constexpr int LDS_BYTES = 4 * NTL * TILEB + 3 * SMAX * 4; // Q, K, V, dO; delta, LSE, mask term
 };
 
-template <typename T, int DROP, int SMAX, bool CAUSAL>
+template <typename T, int DROP, int SMAX, bool CAUSAL, bool STRIDED>
 __global__ __launch_bounds__(BwdShortCfg<SMAX>::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void fmha_bwd_short_kernel(const BwdArgs a) {
+  using RW = Rows<STRIDED, BwdShortCfg<SMAX>::D>;
   using E = Elem<T>;
   using v8 = typename E::v8;
   using C = BwdShortCfg<SMAX>;
@@ -57,25 +58,27 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
   const int bh = blockIdx.x;
   const int kend = bwd_valid_keys(a, bh);
 
-  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
-  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
-  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
-  const T *Ob = (const T *)a.o + (size_t)bh * a.sq * D;
-  const T *dOb = (const T *)a.dout + (size_t)bh * a.sq * D;
+  const T *Qb = (const T *)a.q + RW::head(a.mq, bh, a.sq);
+  const T *Kb = (const T *)a.k + RW::head(a.mk, bh, a.sk);
+  const T *Vb = (const T *)a.v + RW::head(a.mv, bh, a.sk);
+  const T *Ob = (const T *)a.o + RW::head(a.mo, bh, a.sq);
+  const T *dOb = (const T *)a.dout + RW::head(a.mdo, bh, a.sq);
 
   // ---- the head's four matrices: global -> LDS, all requests up front
-  TileCopy<T, D, BT, NT> tcopy;
-  tcopy.init(tid, D);
+  TileCopy<T, D, BT, NT> cq, ck, cdo; // rows of Q, of K and V (equally far apart), of dO
+  cq.init(tid, RW::ss(a.mq));
+  ck.init(tid, RW::ss(a.mk));
+  cdo.init(tid, RW::ss(a.mdo));
   const uint32_t lds0 = lds_address(lds);
 #pragma unroll
   for (int t = 0; t < NTL; ++t) {
     if (t * BT < a.sq) {
-      tcopy.issue(Qb, t * BT, a.sq, lds0 + t * TILEB, tid);
-      tcopy.issue(dOb, t * BT, a.sq, lds0 + (3 * NTL + t) * TILEB, tid);
+      cq.issue(Qb, t * BT, a.sq, lds0 + t * TILEB, tid);
+      cdo.issue(dOb, t * BT, a.sq, lds0 + (3 * NTL + t) * TILEB, tid);
     }
     if (t * BT < a.sk) {
-      tcopy.issue(Kb, t * BT, a.sk, lds0 + (NTL + t) * TILEB, tid);
-      tcopy.issue(Vb, t * BT, a.sk, lds0 + (2 * NTL + t) * TILEB, tid);
+      ck.issue(Kb, t * BT, a.sk, lds0 + (NTL + t) * TILEB, tid);
+      ck.issue(Vb, t * BT, a.sk, lds0 + (2 * NTL + t) * TILEB, tid);
     }
   }
   // this lane's part of its query's O row (for delta), in the layout of a B operand
@@ -84,7 +87,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
   {
     const int q = q1 < a.sq ? q1 : a.sq - 1;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) oreg[ks] = as_v8<T>(*(const u32x4 *)(Ob + (size_t)q * D + ks * 16 + h * 8));
+    for (int ks = 0; ks < KS; ++ks) oreg[ks] = as_v8<T>(*(const u32x4 *)(Ob + (size_t)q * RW::ss(a.mo) + ks * 16 + h * 8));
   }
   if (tid < C::SMAX) {
     float lq = BIG; // rows past the end and rows that saw no key: P = 0
@@ -166,7 +169,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
       }
     }
     if (q1 < a.sq) {
-      T *dQr = (T *)a.dq + ((size_t)bh * a.sq + q1) * D;
+      T *dQr = (T *)a.dq + RW::head(a.mdq, bh, a.sq) + (size_t)q1 * RW::ss(a.mdq);
 #pragma unroll
       for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQr + db * 32, dq[db], a.scale, h);
       if (h == 0) a.delta[(size_t)bh * a.sq + q1] = delta;
@@ -243,8 +246,8 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
       }
     }
     if (key < a.sk) {
-      T *dKr = (T *)a.dk + ((size_t)bh * a.sk + key) * D;
-      T *dVr = (T *)a.dv + ((size_t)bh * a.sk + key) * D;
+      T *dKr = (T *)a.dk + RW::head(a.mdk, bh, a.sk) + (size_t)key * RW::ss(a.mdk);
+      T *dVr = (T *)a.dv + RW::head(a.mdv, bh, a.sk) + (size_t)key * RW::ss(a.mdv);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         store_acc_block_row<T>(dKr + db * 32, dk[db], a.scale, h);

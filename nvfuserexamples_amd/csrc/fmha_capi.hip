@@ -322,7 +322,7 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   // Heads whose Q, K, V and dO fit in LDS together (up to 256 queries and keys) take one launch instead of two.
   int short_rows = env_int("FMHA_BWD_SHORT", 1); // 0: never; 1: up to 256 rows; other values: that many rows
   if (short_rows == 1) short_rows = 256;
-  v.short_seq = !strided && p->d == 64 && p->sq <= short_rows && p->sk <= short_rows && p->sq <= 256 && p->sk <= 256 &&
+  v.short_seq = p->d == 64 && p->sq <= short_rows && p->sk <= short_rows && p->sq <= 256 && p->sk <= 256 &&
                 v.mask != kMaskFull;
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;

@@ -34,7 +34,7 @@ struct BwdVariant {
   bool causal;
   int drop; // 0 none, 1 Philox
   int pair; // causal tile pairing: -1 decide from the amount of work, 0 off, 1 on
-  bool short_seq; // sq, sk <= 256 without a full mask tensor: the one-launch kernel (head dim 64, folded layout)
+  bool short_seq; // sq, sk <= 256 without a full mask tensor: the one-launch kernel (head dim 64)
 };
 
 int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);

@@ -44,14 +44,14 @@ CASES = [
     (2, 3, 320, 320, 64, "fp16", True, 0.0, False, True),    # causal, packed projection
     (2, 2, 256, 256, 128, "bf16", True, 0.0, False, True),
     (40, 16, 128, 192, 64, "fp16", False, 0.0, True, False),  # more items than resident workgroups
+    # short heads: the one-launch backward reads and writes the same layouts
+    (3, 4, 197, 197, 64, "fp16", False, 0.1, False, True),    # ViT-B/16 length, packed projection
+    (2, 3, 100, 128, 64, "bf16", True, 0.0, True, False),
 ]
 
 
 @pytest.mark.parametrize("b,h,sq,sk,d,dtype,causal,p,masked,packed", CASES)
-def test_strided_layouts_match_oracle_and_folded_path(b, h, sq, sk, d, dtype, causal, p, masked, packed, monkeypatch):
-    # short folded heads would otherwise take the one-launch backward, whose arithmetic differs in the last
-    # bit from the general kernels that serve strided tensors: compare like with like
-    monkeypatch.setenv("FMHA_BWD_SHORT", "0")
+def test_strided_layouts_match_oracle_and_folded_path(b, h, sq, sk, d, dtype, causal, p, masked, packed):
     bh = b * h
     q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
     kw, okw = dict(causal=causal), dict(causal=causal)
@@ -126,8 +126,7 @@ def test_bad_strides_are_refused():
         capi.fwd(q3, k, k)
 
 
-def test_operators_and_autograd_take_strided_tensors(monkeypatch):
-    monkeypatch.setenv("FMHA_BWD_SHORT", "0")   # like with like, as above
+def test_operators_and_autograd_take_strided_tensors():
     from nvfuserexamples_amd import load_ops
     from nvfuserexamples_amd.autograd import attention
     ops = load_ops()
