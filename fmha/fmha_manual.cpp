@@ -153,7 +153,10 @@ std::vector<at::Tensor> train_forward(const at::Tensor &input, const at::Tensor 
   p.drop_mask = dm.data_ptr();
   p.drop_scale = 2.0f;
   std::vector<at::Tensor> out{o};
+  at::Tensor lse; // scratch: with it the library derives the saved outputs from one forward launch
   if (save) {
+    lse = at::empty({bh, sq}, input.options().dtype(at::kFloat));
+    p.lse = lse.data_ptr<float>();
     at::Tensor sm = at::empty({bh, sq, sk}, input.options());
     at::Tensor dr = at::empty({bh, sq, sk}, input.options());
     p.save_softmax = sm.data_ptr();

@@ -209,6 +209,10 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
                       device=q.device) if want_lse else None
     P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
     P.lse = lse.data_ptr() if lse is not None else None
+    lse_scratch = None
+    if save and lse is None:   # with an LSE buffer the library takes the faster route to the saved outputs
+        lse_scratch = torch.empty((bh, sq), dtype=torch.float32, device=q.device)
+        P.lse = lse_scratch.data_ptr()
     P.bh, P.sq, P.sk, P.d = bh, sq, sk, d
     P.scale = float(scale) if scale is not None else d ** -0.5
     P.causal = int(bool(causal))

@@ -209,6 +209,14 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  (!a.drop_mask || aligned16(a.drop_mask)) && (!a.save_softmax || aligned16(a.save_softmax)) &&
                  (!a.save_dropout || aligned16(a.save_dropout)) && (!saving || a.drop_mask) &&
                  env_int("FMHA_FWD_SHORT", 1) != 0;
+  // Longer key ranges: where the caller provides an LSE buffer, the save-intermediates operator is the forward
+  // launch followed by a streaming kernel that derives both saved outputs from that LSE (instead of a second
+  // sweep inside a slower forward).  Same alignment needs as above.
+  v.save_split = saving && !v.short_keys && !strided && p->d == 64 && p->lse && (p->sk % 8) == 0 &&
+                 v.mask == kMaskFull && !v.causal && a.drop_mask && aligned16(a.mask) && (a.mask_sb % 8) == 0 &&
+                 (a.mask_sq % 8) == 0 && aligned16(a.drop_mask) && (!a.save_softmax || aligned16(a.save_softmax)) &&
+                 (!a.save_dropout || aligned16(a.save_dropout)) && env_int("FMHA_FWD_SAVE_SPLIT", 1) != 0;
+  if (v.save_split) v.saving = false; // the forward launch itself saves nothing
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
   // flop.  That pays (4-6 % measured) for the unmasked variant at head dim 64 on long key
   // ranges when there is enough work for every resident workgroup to get several 256-query

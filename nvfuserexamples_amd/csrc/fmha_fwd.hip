@@ -8,6 +8,7 @@
 #if FMHA_TU_D == 64 && !FMHA_TU_STRIDED
 #define FMHA_TU_SHORT 1
 #include "fmha_fwd_short.h"
+#include "fmha_fwd_save.h"
 #else
 #define FMHA_TU_SHORT 0
 #endif
@@ -85,6 +86,18 @@ template <bool DROPT, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
 }
 #endif
 
+#if FMHA_TU_SHORT
+// the saved outputs of the save-intermediates operator, from the row log-sum-exp of a forward launch
+int launch_save(FwdArgs &a, hipStream_t s) {
+  auto kern = fmha_fwd_save_kernel<FMHA_TU_T>;
+  a.nqt = (a.sq + SaveCfg::QT - 1) / SaveCfg::QT;
+  const long long nblk = (long long)a.bh * a.nqt;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(SaveCfg::NW * 64), SaveCfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+#endif
+
 template <int QB, int MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<QB, MASK, CAUSAL, 0>(a, s);
   if (drop == 1) return launch<QB, MASK, CAUSAL, 1>(a, s);
@@ -122,8 +135,12 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
     if (v.saving) return launch_short<true, true>(a, s);
     return v.drop == 2 ? launch_short<true, false>(a, s) : launch_short<false, false>(a, s);
   }
+  if (v.save_split) { // forward with LSE on the pipelined kernel, then the saved outputs from that LSE
+    const int rc = launch<1, kMaskFull, false, 2, true>(a, s);
+    return rc ? rc : launch_save(a, s);
+  }
 #else
-  if (v.short_keys) return 1;
+  if (v.short_keys || v.save_split) return 1;
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;

@@ -210,6 +210,42 @@ def test_short_key_ranges_under_full_masks(bh, sq, sk, dtype, mode, short, monke
         assert torch.equal(o2, o)  # saving does not disturb O
 
 
+# Beyond 128 keys the saved outputs come from a streaming kernel that follows the forward launch and
+# derives them from its row log-sum-exp (FMHA_FWD_SAVE_SPLIT=0: from a second sweep inside a plain forward
+# kernel, which is also what serves rows that do not start on 16-byte boundaries and head dim 128).
+SAVE_LONG = [
+    # bh, sq, sk, d, dtype
+    (6, 200, 264, 64, "fp16"),     # ragged query tiles, a partly filled last key tile
+    (3, 128, 512, 64, "fp16"),
+    (4, 192, 320, 64, "bf16"),
+    (300, 128, 192, 64, "fp16"),   # more workgroups than the device holds at once
+    (3, 100, 333, 64, "fp16"),     # rows not 16-byte aligned: the plain kernel either way
+    (2, 160, 256, 128, "fp16"),    # head dim 128: the plain kernel either way
+]
+
+
+@pytest.mark.parametrize("split", ["1", "0"])
+@pytest.mark.parametrize("bh,sq,sk,d,dtype", SAVE_LONG)
+def test_saved_intermediates_beyond_128_keys(bh, sq, sk, d, dtype, split, monkeypatch):
+    monkeypatch.setenv("FMHA_FWD_SAVE_SPLIT", split)
+    q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype)
+    g = torch.Generator().manual_seed(sq + sk)
+    pm = (torch.empty(bh, sq, sk).random_(2, generator=g) * -1000).to(TDT[dtype])
+    dm = torch.empty(bh, sq, sk).random_(2, generator=g).to(TDT[dtype])
+    o, _, sm, dr = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0,
+                        save=True)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(pm), drop_mask=f32(dm), drop_scale=2.0,
+                           want=("o", "softmax", "dropout"))
+    tol = TOL[dtype]
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= 2 * tol
+    assert np.abs(f32(sm.cpu()) - ref["softmax"]).max() <= tol / 2
+    assert np.abs(f32(dr.cpu()) - ref["dropout"]).max() <= tol
+    live = ref["softmax"] > 1e-6
+    assert np.array_equal((f32(dr.cpu()) == 0)[live], (f32(dm) == 0)[live])
+    o2, _, _, _ = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0)
+    assert torch.equal(o2, o)  # saving does not disturb O
+
+
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,mask", [
     (6, 200, 333, 64, "fp16", "pad"),        # ragged tiles, per-key mask
     (4, 192, 192, 64, "bf16", "add_full"),   # full mask tensor and dropout tensor together
