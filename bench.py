@@ -113,11 +113,12 @@ def time_launches(torch, step, steps, warmup):
 
 def short_sequence_legs(torch, capi, L, stream, steps, warmup):
     """The bandwidth-bound shapes: the reference's own operators at the reference's fixed shape
-    (BH 512, S 128, D 64 with full [BH,S,S] mask tensors: fmha/fmha_manual.cpp:24-29, test.py:20-23)
-    and the BERT-base configuration that the CPU baseline is timed on.  Reported as time and as
-    algorithmic bytes per second against the HBM peak, beside the headline, never as `value`.
-    The reference-shape legs rotate six input sets (302 to 604 MB, more than the 256 MB last-level
-    cache); the BERT-base leg is 6 MB and stays cache-resident whatever is rotated."""
+    (BH 512, S 128, D 64 with full [BH,S,S] mask tensors: fmha/fmha_manual.cpp:24-29, test.py:20-23),
+    the same operators with their full mask tensors at the headline sequence length (S 512), a train
+    step at the short shape, and the BERT-base configuration that the CPU baseline is timed on.
+    Reported as time and as algorithmic bytes per second against the HBM peak, beside the headline,
+    never as `value`.  The legs rotate input sets that together exceed the 256 MB last-level cache;
+    the BERT-base leg is 6 MB and stays cache-resident whatever is rotated."""
     legs = {}
 
     def run(name, Ps, nbytes, note):
@@ -161,6 +162,34 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
     run("fmha_train_saveim_nvfuser_BH512_S128_D64_full_masks", save, 4 * bh * s * d * 2 + 4 * bh * s * s * 2,
         "6 sets rotated")
     del keep, infer, train, save
+
+    # the same two operators at the headline sequence length (S 512): 403 / 671 MB per call, two sets rotated
+    s5 = 512
+    keep5, infer5, train5 = [], [], []
+    for _ in range(2):
+        q, k, v = (torch.randn(bh, s5, d, generator=g).to(torch.float16).cuda() for _ in range(3))
+        o = torch.empty_like(q)
+        amask = (torch.rand(bh, s5, s5, generator=g) > 0.1).to(torch.float16).cuda()
+        pad = (torch.rand(bh, s5, s5, generator=g) > 0.9).to(torch.float16).mul_(-1000.0).cuda()
+        dm = (torch.rand(bh, s5, s5, generator=g) > 0.5).to(torch.float16).cuda()
+        keep5.append((q, k, v, o, amask, pad, dm))
+        for kind in ("infer", "train"):
+            P = capi.FwdParams()
+            P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+            P.bh, P.sq, P.sk, P.d = bh, s5, s5, d
+            P.dtype, P.scale = capi.F16, 0.125
+            P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = 1, s5 * s5, s5
+            if kind == "infer":
+                P.mask, P.mask_kind, P.mask_neg = amask.data_ptr(), capi.MASK_KEEP01, -10000.0
+                infer5.append(P)
+            else:
+                P.mask, P.mask_kind = pad.data_ptr(), capi.MASK_ADDITIVE
+                P.drop_kind, P.drop_mask, P.drop_scale = capi.DROP_TENSOR, dm.data_ptr(), 2.0
+                train5.append(P)
+    run("fmha_nvfuser_BH512_S512_D64_full_mask", infer5, 4 * bh * s5 * d * 2 + bh * s5 * s5 * 2, "2 sets rotated")
+    run("fmha_train_nvfuser_BH512_S512_D64_full_masks", train5, 4 * bh * s5 * d * 2 + 2 * bh * s5 * s5 * 2,
+        "2 sets rotated")
+    del keep5, infer5, train5
 
     # train step at the same short shape (the reference has no backward): [B,1,1,S] padding mask, Philox
     # dropout; forward with LSE, then the one-launch short-sequence backward

@@ -43,7 +43,8 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 }
 
 // Tuning overrides for experiments and tests: FMHA_FWD_QB=1|2 forces the query blocks per wave of
-// the forward, FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
+// the forward, FMHA_FWD_STREAM=0 keeps full-mask forwards on the pipelined kernel,
+// FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
 // one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
 // pairing of causal tiles in the backward.
 int env_int(const char *name, int dflt) {
@@ -217,6 +218,12 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  (a.mask_sq % 8) == 0 && aligned16(a.drop_mask) && (!a.save_softmax || aligned16(a.save_softmax)) &&
                  (!a.save_dropout || aligned16(a.save_dropout)) && env_int("FMHA_FWD_SAVE_SPLIT", 1) != 0;
   if (v.save_split) v.saving = false; // the forward launch itself saves nothing
+  // Other forwards under an aligned full mask tensor (with or without a dropout tensor) are memory time at
+  // head dim 64: the streaming kernel.
+  v.stream = !v.short_keys && !v.saving && !strided && p->d == 64 && (p->sk % 8) == 0 && v.mask == kMaskFull &&
+             !v.causal && v.drop != 1 && !p->kv_len && aligned16(a.mask) && (a.mask_sb % 8) == 0 &&
+             (a.mask_sq % 8) == 0 && (v.drop != 2 || (a.drop_mask && aligned16(a.drop_mask))) &&
+             env_int("FMHA_FWD_STREAM", 1) != 0;
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
   // flop.  That pays (4-6 % measured) for the unmasked variant at head dim 64 on long key
   // ranges when there is enough work for every resident workgroup to get several 256-query

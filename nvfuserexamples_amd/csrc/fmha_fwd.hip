@@ -9,6 +9,7 @@
 #define FMHA_TU_SHORT 1
 #include "fmha_fwd_short.h"
 #include "fmha_fwd_save.h"
+#include "fmha_fwd_stream.h"
 #else
 #define FMHA_TU_SHORT 0
 #endif
@@ -98,6 +99,18 @@ int launch_save(FwdArgs &a, hipStream_t s) {
 }
 #endif
 
+#if FMHA_TU_SHORT
+// long key ranges under a full mask tensor (and a dropout tensor): the streaming forward
+template <bool DROPT> int launch_stream(FwdArgs &a, hipStream_t s) {
+  auto kern = fmha_fwd_stream_kernel<FMHA_TU_T, DROPT>;
+  a.nqt = (a.sq + StreamCfg::QT - 1) / StreamCfg::QT;
+  const long long nblk = (long long)a.bh * a.nqt;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(StreamCfg::NW * 64), StreamCfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+#endif
+
 template <int QB, int MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<QB, MASK, CAUSAL, 0>(a, s);
   if (drop == 1) return launch<QB, MASK, CAUSAL, 1>(a, s);
@@ -135,12 +148,13 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
     if (v.saving) return launch_short<true, true>(a, s);
     return v.drop == 2 ? launch_short<true, false>(a, s) : launch_short<false, false>(a, s);
   }
-  if (v.save_split) { // forward with LSE on the pipelined kernel, then the saved outputs from that LSE
-    const int rc = launch<1, kMaskFull, false, 2, true>(a, s);
+  if (v.save_split) { // forward with LSE, then the saved outputs from that LSE
+    const int rc = v.stream ? launch_stream<true>(a, s) : launch<1, kMaskFull, false, 2, true>(a, s);
     return rc ? rc : launch_save(a, s);
   }
+  if (v.stream) return v.drop == 2 ? launch_stream<true>(a, s) : launch_stream<false>(a, s);
 #else
-  if (v.short_keys || v.save_split) return 1;
+  if (v.short_keys || v.save_split || v.stream) return 1;
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;

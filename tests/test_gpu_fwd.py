@@ -163,6 +163,15 @@ SHORT = [
     (4, 300, 128, "bf16", "save"),
     (600, 128, 128, "fp16", "train"),   # more workgroups than the device holds at once
     (6, 160, 128, "fp16", "bcast"),     # [B,1,sq,sk] mask shared by the heads of a batch entry, -inf entries, LSE
+    # beyond 128 keys the same operators run on a streaming kernel (whole-row accesses, online softmax over
+    # 64-key tiles); FMHA_FWD_STREAM=0 keeps them on the pipelined kernel
+    (4, 512, 512, "fp16", "infer"),
+    (3, 200, 264, "fp16", "train"),     # ragged query tile, partly filled last key tile
+    (4, 128, 320, "bf16", "train"),
+    (2, 33, 1024, "fp16", "infer"),     # sixteen key tiles
+    (300, 128, 192, "fp16", "train"),   # more workgroups than the device holds at once
+    (6, 160, 256, "fp16", "bcast"),
+    (3, 100, 136, "fp16", "save"),      # saved outputs from the streaming forward's LSE
 ]
 
 
@@ -170,6 +179,7 @@ SHORT = [
 @pytest.mark.parametrize("bh,sq,sk,dtype,mode", SHORT)
 def test_short_key_ranges_under_full_masks(bh, sq, sk, dtype, mode, short, monkeypatch):
     monkeypatch.setenv("FMHA_FWD_SHORT", short)
+    monkeypatch.setenv("FMHA_FWD_STREAM", short)
     q, k, v = make_qkv(bh, sq, sk, 64, seed=bh + sk, dtype=dtype)
     g = torch.Generator().manual_seed(sq + sk)
     tol = TOL[dtype]
@@ -228,6 +238,9 @@ SAVE_LONG = [
 @pytest.mark.parametrize("bh,sq,sk,d,dtype", SAVE_LONG)
 def test_saved_intermediates_beyond_128_keys(bh, sq, sk, d, dtype, split, monkeypatch):
     monkeypatch.setenv("FMHA_FWD_SAVE_SPLIT", split)
+    # without the split the saving forward is the plain kernel, whose O is bit-identical to the pipelined
+    # kernel's, not to the streaming kernel's: keep the non-saving call on the same family
+    monkeypatch.setenv("FMHA_FWD_STREAM", split)
     q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype)
     g = torch.Generator().manual_seed(sq + sk)
     pm = (torch.empty(bh, sq, sk).random_(2, generator=g) * -1000).to(TDT[dtype])
