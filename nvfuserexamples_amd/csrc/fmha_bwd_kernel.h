@@ -152,19 +152,26 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int q = q0w + qb * 32 + ql;
+    // Rows past the end re-read the last row (nothing of theirs is stored and their P is forced to 0).
+    // The loads are unconditional on purpose: a load under a lane condition is merged with its "else"
+    // value right behind it, so the compiler waits for it on the spot and the twelve loads below would
+    // take four round trips to memory instead of one.
+    const int qc = q < a.sq ? q : a.sq - 1;
+    u32x4 tq[KS], td[KS], to[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const size_t col = ks * 16 + h * 8;
+      tq[ks] = *(const u32x4 *)(Qb + (size_t)qc * RW::ss(a.mq) + col);
+      td[ks] = *(const u32x4 *)(dOb + (size_t)qc * RW::ss(a.mdo) + col);
+      to[ks] = *(const u32x4 *)(Ob + (size_t)qc * RW::ss(a.mo) + col);
+    }
+    const float lse_q = a.lse[(size_t)bh * a.sq + qc];
     float dsum = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      u32x4 tq = {0u, 0u, 0u, 0u}, td = {0u, 0u, 0u, 0u}, to = {0u, 0u, 0u, 0u};
-      if (q < a.sq) {
-        const size_t col = ks * 16 + h * 8;
-        tq = *(const u32x4 *)(Qb + (size_t)q * RW::ss(a.mq) + col);
-        td = *(const u32x4 *)(dOb + (size_t)q * RW::ss(a.mdo) + col);
-        to = *(const u32x4 *)(Ob + (size_t)q * RW::ss(a.mo) + col);
-      }
-      const v8 qraw = as_v8<T>(tq);
-      const v8 doraw = as_v8<T>(td);
-      const v8 ov = as_v8<T>(to);
+      const v8 qraw = as_v8<T>(tq[ks]);
+      const v8 doraw = as_v8<T>(td[ks]);
+      const v8 ov = as_v8<T>(to[ks]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         qreg[qb][ks][j] = (T)((float)qraw[j] * a.scale_l2);
@@ -176,8 +183,7 @@ __global__ __launch_bounds__(NW * 64)
     delta[qb] = dsum;
     float nl = BIGNEG; // rows past the end and fully masked rows get P = 0
     if (q < a.sq) {
-      const float v = a.lse[(size_t)bh * a.sq + q];
-      if (v != NEG_INF) nl = -v * FMHA_LOG2E;
+      if (lse_q != NEG_INF) nl = -lse_q * FMHA_LOG2E;
       if (h == 0) a.delta[(size_t)bh * a.sq + q] = dsum;
     }
 #pragma unroll
@@ -471,16 +477,23 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
   for (int kb = 0; kb < KB; ++kb) {
     const int key = k0w + kb * 32 + kl;
+    // Unconditional loads (a load under a lane condition makes the compiler wait for it on the spot:
+    // four round trips to memory instead of one).  Keys past the end re-read the last row; invalid keys
+    // get P = dS = 0 through their mask term, whatever their K and V rows hold.
+    const int kc = key < a.sk ? key : a.sk - 1;
+    u32x4 tk[KS], tv[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      u32x4 tk = {0u, 0u, 0u, 0u}, tv = {0u, 0u, 0u, 0u};
-      if (key < skv) {
-        const size_t col = ks * 16 + h * 8;
-        tk = *(const u32x4 *)(Kb + (size_t)key * RW::ss(a.mk) + col);
-        tv = *(const u32x4 *)(Vb + (size_t)key * RW::ss(a.mv) + col);
-      }
-      const v8 kraw = as_v8<T>(tk);
-      const v8 vraw = as_v8<T>(tv);
+      const size_t col = ks * 16 + h * 8;
+      tk[ks] = *(const u32x4 *)(Kb + (size_t)kc * RW::ss(a.mk) + col);
+      tv[ks] = *(const u32x4 *)(Vb + (size_t)kc * RW::ss(a.mv) + col);
+    }
+    T mraw_key = (T)0.f;
+    if (MASK == kMaskPerKey) mraw_key = ((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + kc];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const v8 kraw = as_v8<T>(tk[ks]);
+      const v8 vraw = as_v8<T>(tv[ks]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         kreg[kb][ks][j] = (T)((float)kraw[j] * a.scale_l2);
@@ -488,8 +501,7 @@ __global__ __launch_bounds__(NW * 64)
       }
     }
     float mk = 0.f;
-    if (MASK == kMaskPerKey && key < skv)
-      mk = fmaf((float)((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + key], a.mask_a, a.mask_b);
+    if (MASK == kMaskPerKey) mk = fmaf((float)mraw_key, a.mask_a, a.mask_b);
     if (key >= skv) mk = BIGNEG;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {

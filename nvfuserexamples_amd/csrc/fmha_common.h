@@ -296,6 +296,49 @@ template <typename T> FMHA_DEV void store_acc_block_row(T *dst_row, const f32x16
   }
 }
 
+// ---------------------------------------------------------------- row <-> accumulator layout
+// A wave's 32 x KEYS block of a [.., sq, sk] tensor (mask, dropout tensor, saved outputs) moves
+// to and from global memory as whole row segments: 16 bytes (8 keys) per lane, KEYS/8 lanes per
+// row, so instruction i of KEYS/16 covers rows RPI*i .. RPI*i + RPI-1 (RPI = 512/KEYS).  The MFMA
+// accumulators hold the block the other way round: lane = row (l % 32), and for each 32-key
+// sub-block sb four 8-byte pieces g at keys 32 sb + 8 g + 4 (l / 32) .. +3.  As a global access that
+// layout touches 32 different cache lines per instruction; instead a wave-private LDS scratch
+// (row pitch = row + 16 bytes) is written in one layout and read in the other.  The scratch belongs
+// to one wave, whose LDS accesses execute in order: turn() only keeps the compiler from moving
+// accesses across the change of layout.
+template <int KEYS> struct RowScratch {
+  static constexpr int LPR = KEYS / 8;    // lanes per row
+  static constexpr int RPI = 64 / LPR;    // rows per instruction
+  static constexpr int NI = 32 / RPI;     // instructions per block
+  static constexpr int PITCH = KEYS * 2 + 16;
+  static constexpr int BYTES = 32 * PITCH;
+  char *row;  // this lane's 16 bytes of instruction 0 (+ RPI * i * PITCH for instruction i)
+  char *frag; // this lane's piece (0, 0) (+ 64 sb + 16 g)
+  int rsub, chunk; // the lane's row within an instruction's rows, and its 8-key chunk of the row
+  FMHA_DEV void init(char *base, int l) {
+    rsub = l / LPR;
+    chunk = l % LPR;
+    row = base + rsub * PITCH + chunk * 16;
+    frag = base + (l & 31) * PITCH + (l >> 5) * 8;
+  }
+  static FMHA_DEV void turn() {
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+  }
+  FMHA_DEV void rows_in(const u32x4 (&r)[NI]) const {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) *(u32x4 *)(row + RPI * i * PITCH) = r[i];
+  }
+  FMHA_DEV u32x4 row_out(int i) const { return *(const u32x4 *)(row + RPI * i * PITCH); }
+  FMHA_DEV u32x2 piece(int sb, int g) const { return *(const u32x2 *)(frag + sb * 64 + g * 16); }
+  template <typename T> FMHA_DEV void put_piece(int sb, int g, const typename Elem<T>::v4 &v) const {
+    Pack8 pk;
+    if constexpr (__is_same(T, _Float16)) pk.h = v;
+    else pk.b = v;
+    *(u32x2 *)(frag + sb * 64 + g * 16) = pk.u;
+  }
+};
+
 FMHA_DEV float max3(float a, float b, float c) { return __builtin_fmaxf(__builtin_fmaxf(a, b), c); }
 FMHA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 FMHA_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

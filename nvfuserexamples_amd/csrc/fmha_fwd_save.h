@@ -21,9 +21,8 @@ struct SaveCfg {
   static constexpr int BK = 64;
   static constexpr int ROWB = D * 2 + 16;          // padded K rows: conflict-free 16-byte reads
   static constexpr int KTILEB = BK * ROWB;
-  static constexpr int SCR_PITCH = BK * 2 + 16;
-  static constexpr int SCR_BYTES = 32 * SCR_PITCH;
-  static constexpr int LDS_BYTES = 2 * KTILEB + NW * SCR_BYTES;
+  using Scratch = RowScratch<BK>;                  // wave-private: rows of a [.., sq, sk] tensor <-> accumulator layout
+  static constexpr int LDS_BYTES = 2 * KTILEB + NW * Scratch::BYTES;
 };
 
 template <typename T>
@@ -33,7 +32,7 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = SaveCfg;
-  constexpr int D = C::D, KS = D / 16, BK = C::BK, NSB = BK / 32, NT = C::NW * 64, ROWB = C::ROWB, PITCH = C::SCR_PITCH;
+  constexpr int D = C::D, KS = D / 16, BK = C::BK, NSB = BK / 32, NT = C::NW * 64, ROWB = C::ROWB;
   constexpr int CPR = D / 8, CPT = BK * CPR / NT;
   constexpr float NEG_INF = -__builtin_inff();
 
@@ -68,30 +67,34 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
 
   // ---- staging.  K: global -> registers -> LDS (two stages).  [.., sq, sk] rows: instruction i covers
   // rows 8i .. 8i+7 of the wave's 32, eight lanes per row, 8 keys (16 bytes) per lane.
-  const int rsub = l >> 3, chunk = l & 7;
+  typename C::Scratch scr;
+  scr.init(lds + 2 * C::KTILEB + w * C::Scratch::BYTES, l);
+  const int rsub = scr.rsub, chunk = scr.chunk;
   int qrow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int q = q0w + 8 * i + rsub;
     qrow[i] = q < a.sq ? q : a.sq - 1;
   }
-  const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + chunk * 8;
-  const T *db_ = (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk + chunk * 8;
+  const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb;
+  const T *db_ = (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk;
   u32x4 kst[CPT], mreg[4], dreg[4];
+  // Every load is unconditional (a load under a lane condition makes the compiler wait for it on the
+  // spot): rows past the end re-read the last row, chunks past sk re-read the row's first chunk; neither
+  // is ever used (those keys get P = 0 and are not stored).
   auto gload = [&](int k0, u32x4 (&kd)[CPT], u32x4 (&md)[4], u32x4 (&dd)[4]) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * NT;
-      const int kr = k0 + c / CPR;
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      kd[i] = kr < a.sk ? *(const u32x4 *)(Kb + (size_t)kr * D + (c % CPR) * 8) : z;
+      int kr = k0 + c / CPR;
+      kr = kr < a.sk ? kr : a.sk - 1;
+      kd[i] = *(const u32x4 *)(Kb + (size_t)kr * D + (c % CPR) * 8);
     }
-    const bool cvalid = k0 + chunk * 8 < a.sk;
+    const int koff = k0 + chunk * 8 < a.sk ? k0 + chunk * 8 : 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      md[i] = cvalid ? *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq + k0) : z;
-      dd[i] = cvalid ? *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk + k0) : z;
+      md[i] = *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq + koff);
+      dd[i] = *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk + koff);
     }
   };
   auto lstore = [&](int stage, const u32x4 (&kd)[CPT]) {
@@ -102,32 +105,15 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
     }
   };
 
-  char *scr = lds + 2 * C::KTILEB + w * C::SCR_BYTES;
-  char *scr_row = scr + (rsub * PITCH + chunk * 16); // + 8i rows
-  char *scr_frag = scr + (ql * PITCH + h * 8);       // + 64 sb + 16 g
-  auto scratch_turn = [] {
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("" ::: "memory");
-  };
-  auto rows_in = [&](const u32x4 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4 *)(scr_row + 8 * i * PITCH) = r[i];
-  };
   auto rows_out = [&](void *out, int k0) {
     const bool cvalid = k0 + chunk * 8 < a.sk;
     T *ob = (T *)out + (size_t)bh * a.sq * a.sk + k0 + chunk * 8;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int q = q0w + 8 * i + rsub;
-      const u32x4 t = *(const u32x4 *)(scr_row + 8 * i * PITCH);
+      const u32x4 t = scr.row_out(i);
       if (cvalid && q < a.sq) *(u32x4 *)(ob + (size_t)q * a.sk) = t;
     }
-  };
-  auto put_piece = [&](int sb, int g, const v4 &piece) {
-    Pack8 pk;
-    if constexpr (__is_same(T, _Float16)) pk.h = piece;
-    else pk.b = piece;
-    *(u32x2 *)(scr_frag + sb * 64 + g * 16) = pk.u;
   };
 
   const int nkt = (a.sk + BK - 1) / BK;
@@ -152,13 +138,13 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
       for (int ks = 0; ks < KS; ++ks)
         x[sb] = E::mfma(as_v8<T>(*(const u32x4 *)(ldsK + (sb * 32 + ql) * ROWB + ks * 32 + h * 16)), qreg[ks], x[sb]);
     }
-    rows_in(mreg);
-    scratch_turn();
+    scr.rows_in(mreg);
+    scr.turn();
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const v4 mv = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+        const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int kk = k0 + sb * 32 + 8 * g + 4 * h + i;
@@ -166,7 +152,7 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
           x[sb][4 * g + i] = kk < a.sk ? fast_exp2(s) : 0.f;
         }
       }
-    scratch_turn();
+    scr.turn();
 
     // ---- softmax out
     if (a.save_softmax) {
@@ -177,34 +163,34 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
           v4 s4;
 #pragma unroll
           for (int i = 0; i < 4; ++i) s4[i] = (T)x[sb][4 * g + i];
-          put_piece(sb, g, s4);
+          scr.template put_piece<T>(sb, g, s4);
         }
-      scratch_turn();
+      scr.turn();
       rows_out(a.save_softmax, k0);
-      scratch_turn();
+      scr.turn();
     }
 
     // ---- dropped, scaled copy out
     if (a.save_dropout) {
-      rows_in(dreg);
-      scratch_turn();
+      scr.rows_in(dreg);
+      scr.turn();
       v4 d4[NSB][4];
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const v4 dm = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+          const v4 dm = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
           for (int i = 0; i < 4; ++i) d4[sb][g][i] = (T)(x[sb][4 * g + i] * ((float)dm[i] * a.drop_scale));
         }
-      scratch_turn();
+      scr.turn();
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) put_piece(sb, g, d4[sb][g]);
-      scratch_turn();
+        for (int g = 0; g < 4; ++g) scr.template put_piece<T>(sb, g, d4[sb][g]);
+      scr.turn();
       rows_out(a.save_dropout, k0);
-      scratch_turn();
+      scr.turn();
     }
 
     if (more) {

@@ -31,9 +31,8 @@ struct ShortCfg {
   static constexpr int NSB = SKMAX / 32;            // 32-key accumulator blocks
   static constexpr int BT = 64;                     // rows per swizzled LDS tile
   static constexpr int TILEB = BT * D * 2;
-  static constexpr int SCR_PITCH = SKMAX * 2 + 16;  // scratch row pitch: 16 bytes of padding per row
-  static constexpr int SCR_BYTES = 32 * SCR_PITCH;
-  static constexpr int LDS_BYTES = 4 * TILEB + NW * SCR_BYTES; // K, V (two tiles each) + one scratch per wave
+  using Scratch = RowScratch<SKMAX>;              // wave-private: rows of a [.., sq, sk] tensor <-> accumulator layout
+  static constexpr int LDS_BYTES = 4 * TILEB + NW * Scratch::BYTES; // K, V (two tiles each) + one scratch per wave
 };
 
 template <typename T, bool DROPT, bool SAVE>
@@ -44,7 +43,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   using v4 = typename E::v4;
   using C = ShortCfg;
   constexpr int D = C::D, KS = D / 16, DB = D / 32, NSB = C::NSB, NT = C::NW * 64;
-  constexpr int TILEB = C::TILEB, PITCH = C::SCR_PITCH;
+  constexpr int TILEB = C::TILEB;
   constexpr float NEG_INF = -__builtin_inff();
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -87,14 +86,18 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 
   // [.., sq, sk] rows as the wave reads and writes them: instruction i covers rows 4i .. 4i+3 of the
   // wave's 32, sixteen lanes per row, 8 keys (16 bytes) per lane
-  const int rsub = l >> 4;
-  const int chunk = l & 15;
+  typename C::Scratch scr;
+  scr.init(lds + 4 * TILEB + w * C::Scratch::BYTES, l);
+  const int rsub = scr.rsub, chunk = scr.chunk;
   const bool cvalid = chunk * 8 < a.sk;
   u32x4 mreg[8], dreg[8];
   {
-    const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + chunk * 8;
-    const T *db_ = DROPT ? (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk + chunk * 8 : nullptr;
-    const u32x4 z = {0u, 0u, 0u, 0u};
+    // Lanes whose chunk lies past sk read chunk 0 instead (their values are never used: those keys'
+    // scores are forced to -inf).  Unconditional loads matter: a load under a lane condition is merged
+    // with its "else" value right behind it, which makes the compiler wait for it on the spot.
+    const int ch8 = cvalid ? chunk * 8 : 0;
+    const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + ch8;
+    const T *db_ = DROPT ? (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk + ch8 : nullptr;
     int qrow[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -102,32 +105,21 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
       qrow[i] = q < a.sq ? q : a.sq - 1;
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) mreg[i] = cvalid ? *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq) : z;
+    for (int i = 0; i < 8; ++i) mreg[i] = *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq);
     if (DROPT) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dreg[i] = cvalid ? *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk) : z;
+      for (int i = 0; i < 8; ++i) dreg[i] = *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk);
     }
   }
   // Loads complete in the order they were requested.  The K and V copies went out first: once at most
   // the 4 Q, 8 mask and 8 dropout-row loads requested after them are outstanding, they have landed;
-  // the first product then runs while the [.., sq, sk] rows are still on their way.  (Lanes whose
-  // chunk lies past sk skip their row loads together, as a branch around all of them or as a masked
-  // load that is still counted; either way no more than these loads follow the copies.)
+  // the first product then runs while the [.., sq, sk] rows are still on their way.  (A test compiles
+  // this kernel to assembly and checks that count.)
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + 8 + (DROPT ? 8 : 0)) : "memory");
   __syncthreads();
 
   PanelLane pl;
   pl.init(l);
-  char *scr = lds + 4 * TILEB + w * C::SCR_BYTES;
-  char *scr_row = scr + (rsub * PITCH + chunk * 16); // + 4i rows: this lane's 16 bytes of instruction i
-  char *scr_frag = scr + (ql * PITCH + h * 8);       // + 64 sb + 16 g: this lane's 8-byte piece (sb, g)
-  // The scratch belongs to one wave, whose LDS accesses execute in order: between the two layouts
-  // it is enough to keep the compiler from moving accesses across.
-  auto scratch_turn = [] {
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("" ::: "memory");
-  };
-
   // ---- x^T = K . Q^T for all keys (lane = query, registers = keys 32 sb + 8g + 4h + t)
   f32x16 x[NSB];
 #pragma unroll
@@ -142,15 +134,14 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   }
 
   // ---- scale and mask (log2 units); keys past the end drop out
-#pragma unroll
-  for (int i = 0; i < 8; ++i) *(u32x4 *)(scr_row + 4 * i * PITCH) = mreg[i];
-  scratch_turn();
+  scr.rows_in(mreg);
+  scr.turn();
   float mx = NEG_INF;
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const v4 mv = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+      const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int kk = sb * 32 + 8 * g + 4 * h + t;
@@ -160,7 +151,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
         mx = fmaxf(mx, xv);
       }
     }
-  scratch_turn();
+  scr.turn();
   mx = xhalf_max(mx);
   const float mref = mx == NEG_INF ? 0.f : mx;
 
@@ -183,24 +174,16 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int q = q0w + 4 * i + rsub;
-      const u32x4 t = *(const u32x4 *)(scr_row + 4 * i * PITCH);
+      const u32x4 t = scr.row_out(i);
       if (cvalid && q < a.sq) *(u32x4 *)(ob + (size_t)q * a.sk) = t;
     }
   };
-  auto put_piece = [&](int sb, int g, const v4 &piece) {
-    Pack8 pk;
-    if constexpr (__is_same(T, _Float16)) pk.h = piece;
-    else pk.b = piece;
-    *(u32x2 *)(scr_frag + sb * 64 + g * 16) = pk.u;
-  };
-
   // ---- dropped, normalised probabilities in the element type: second operand and saved output.
   // (The dropout rows are the last loads to arrive; nothing is stored before they are consumed, so
   // that waiting for them never waits for a store.)
   if (DROPT) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *(u32x4 *)(scr_row + 4 * i * PITCH) = dreg[i];
-    scratch_turn();
+    scr.rows_in(dreg);
+    scr.turn();
   }
   v8 pfrag[NSB][2];
 #pragma unroll
@@ -209,14 +192,14 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
     for (int g = 0; g < 4; ++g) {
       float keep[4] = {a.drop_scale, a.drop_scale, a.drop_scale, a.drop_scale};
       if (DROPT) {
-        const v4 dm = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+        const v4 dm = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
         for (int t = 0; t < 4; ++t) keep[t] = (float)dm[t] * a.drop_scale;
       }
 #pragma unroll
       for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)((x[sb][4 * g + t] * inv) * keep[t]);
     }
-  scratch_turn();
+  scr.turn();
 
   if (SAVE && a.save_softmax) {
 #pragma unroll
@@ -226,11 +209,11 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
         v4 s4;
 #pragma unroll
         for (int t = 0; t < 4; ++t) s4[t] = (T)(x[sb][4 * g + t] * inv);
-        put_piece(sb, g, s4);
+        scr.template put_piece<T>(sb, g, s4);
       }
-    scratch_turn();
+    scr.turn();
     store_rows(a.save_softmax);
-    scratch_turn();
+    scr.turn();
   }
   if (SAVE && a.save_dropout) {
 #pragma unroll
@@ -240,9 +223,9 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
         v4 d4;
 #pragma unroll
         for (int t = 0; t < 4; ++t) d4[t] = pfrag[sb][g >> 1][4 * (g & 1) + t];
-        put_piece(sb, g, d4);
+        scr.template put_piece<T>(sb, g, d4);
       }
-    scratch_turn();
+    scr.turn();
     store_rows(a.save_dropout);
   }
 

@@ -22,9 +22,8 @@ struct StreamCfg {
   static constexpr int BK = 64;
   static constexpr int ROWB = D * 2 + 16;          // padded K / V rows: conflict-free 16-byte and transpose reads
   static constexpr int TILEB = BK * ROWB;
-  static constexpr int SCR_PITCH = BK * 2 + 16;
-  static constexpr int SCR_BYTES = 32 * SCR_PITCH;
-  static constexpr int LDS_BYTES = 4 * TILEB + NW * SCR_BYTES; // {K, V} x 2 stages + one scratch per wave
+  using Scratch = RowScratch<BK>;                  // wave-private: rows of a [.., sq, sk] tensor <-> accumulator layout
+  static constexpr int LDS_BYTES = 4 * TILEB + NW * Scratch::BYTES; // {K, V} x 2 stages + one scratch per wave
 };
 
 template <typename T, bool DROPT>
@@ -35,7 +34,7 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
   using v4 = typename E::v4;
   using C = StreamCfg;
   constexpr int D = C::D, KS = D / 16, DB = D / 32, BK = C::BK, NSB = BK / 32, NT = C::NW * 64, ROWB = C::ROWB;
-  constexpr int PITCH = C::SCR_PITCH, TILEB = C::TILEB;
+  constexpr int TILEB = C::TILEB;
   constexpr int CPR = D / 8, CPT = BK * CPR / NT;
   constexpr float NEG_INF = -__builtin_inff();
 
@@ -68,33 +67,37 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
 
   // ---- staging.  K, V: global -> registers -> LDS (two stages).  [.., sq, sk] rows: instruction i covers
   // rows 8i .. 8i+7 of the wave's 32, eight lanes per row, 8 keys (16 bytes) per lane.
-  const int rsub = l >> 3, chunk = l & 7;
+  typename C::Scratch scr;
+  scr.init(lds + 4 * TILEB + w * C::Scratch::BYTES, l);
+  const int rsub = scr.rsub, chunk = scr.chunk;
   int qrow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int q = q0w + 8 * i + rsub;
     qrow[i] = q < a.sq ? q : a.sq - 1;
   }
-  const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + chunk * 8;
-  const T *db_ = DROPT ? (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk + chunk * 8 : nullptr;
+  const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb;
+  const T *db_ = DROPT ? (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk : nullptr;
   struct Stage {
     u32x4 k[CPT], v[CPT], m[4], d[4];
   };
+  // Every load is unconditional (a load under a lane condition makes the compiler wait for it on the
+  // spot): key rows past the end re-read the last row, chunks past sk re-read the row's first chunk;
+  // those keys' scores are forced to -inf, so P = 0 meets finite values of V.
   auto gload = [&](int k0, Stage &st) {
-    const u32x4 z = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * NT;
-      const int kr = k0 + c / CPR;
-      const bool ok = kr < a.sk; // rows past the end: zeros (their scores are set to -inf, and P = 0 meets V = 0)
-      st.k[i] = ok ? *(const u32x4 *)(Kb + (size_t)kr * D + (c % CPR) * 8) : z;
-      st.v[i] = ok ? *(const u32x4 *)(Vb + (size_t)kr * D + (c % CPR) * 8) : z;
+      int kr = k0 + c / CPR;
+      kr = kr < a.sk ? kr : a.sk - 1;
+      st.k[i] = *(const u32x4 *)(Kb + (size_t)kr * D + (c % CPR) * 8);
+      st.v[i] = *(const u32x4 *)(Vb + (size_t)kr * D + (c % CPR) * 8);
     }
-    const bool cvalid = k0 + chunk * 8 < a.sk;
+    const int koff = k0 + chunk * 8 < a.sk ? k0 + chunk * 8 : 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      st.m[i] = cvalid ? *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq + k0) : z;
-      if (DROPT) st.d[i] = cvalid ? *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk + k0) : z;
+      st.m[i] = *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq + koff);
+      if (DROPT) st.d[i] = *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk + koff);
     }
   };
   auto lstore = [&](int stage, const Stage &st) {
@@ -104,18 +107,6 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
       *(u32x4 *)(lds + stage * 2 * TILEB + (c / CPR) * ROWB + (c % CPR) * 16) = st.k[i];
       *(u32x4 *)(lds + stage * 2 * TILEB + TILEB + (c / CPR) * ROWB + (c % CPR) * 16) = st.v[i];
     }
-  };
-
-  char *scr = lds + 4 * TILEB + w * C::SCR_BYTES;
-  char *scr_row = scr + (rsub * PITCH + chunk * 16); // + 8i rows
-  char *scr_frag = scr + (ql * PITCH + h * 8);       // + 64 sb + 16 g
-  auto scratch_turn = [] {
-    __builtin_amdgcn_wave_barrier();
-    asm volatile("" ::: "memory");
-  };
-  auto rows_in = [&](const u32x4 (&r)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4 *)(scr_row + 8 * i * PITCH) = r[i];
   };
 
   // ---- running state: row maximum m (log2 units), this lane's part of the row sum, unnormalised O^T
@@ -150,14 +141,14 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
       for (int ks = 0; ks < KS; ++ks)
         x[sb] = E::mfma(as_v8<T>(*(const u32x4 *)(ldsK + (sb * 32 + ql) * ROWB + ks * 32 + h * 16)), qreg[ks], x[sb]);
     }
-    rows_in(cur.m);
-    scratch_turn();
+    scr.rows_in(cur.m);
+    scr.turn();
     float tmax = NEG_INF;
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const v4 mv = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+        const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int kk = k0 + sb * 32 + 8 * g + 4 * h + i;
@@ -167,7 +158,7 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
           tmax = fmaxf(tmax, s);
         }
       }
-    scratch_turn();
+    scr.turn();
 
     // ---- online softmax: raise the maximum, rescale what has been accumulated under the old one
     tmax = xhalf_max(tmax);
@@ -192,8 +183,8 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
 
     // ---- (dropped) probabilities in the element type: B operand of the second product
     if (DROPT) {
-      rows_in(cur.d);
-      scratch_turn();
+      scr.rows_in(cur.d);
+      scr.turn();
     }
     v8 pfrag[NSB][2];
 #pragma unroll
@@ -202,14 +193,14 @@ void fmha_fwd_stream_kernel(const FwdArgs a) {
       for (int g = 0; g < 4; ++g) {
         float keep[4] = {1.f, 1.f, 1.f, 1.f};
         if (DROPT) {
-          const v4 dm = as_v4<T>(*(const u32x2 *)(scr_frag + sb * 64 + g * 16));
+          const v4 dm = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
           for (int i = 0; i < 4; ++i) keep[i] = (float)dm[i];
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) pfrag[sb][g >> 1][4 * (g & 1) + i] = (T)(x[sb][4 * g + i] * keep[i]);
       }
-    if (DROPT) scratch_turn();
+    if (DROPT) scr.turn();
 
     // ---- O^T += V^T . P^T
 #pragma unroll
