@@ -146,8 +146,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     const int q = q0w + qb * 32 + ql;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      u32x4 t = {0u, 0u, 0u, 0u};
-      if (q < a.sq) t = *(const u32x4 *)(Qb + (size_t)q * RW::ss(a.mq) + ks * 16 + h * 8);
+      // rows past the end re-read the last row (never stored); unconditional loads do not stall on each other
+      const int qc = q < a.sq ? q : a.sq - 1;
+      const u32x4 t = *(const u32x4 *)(Qb + (size_t)qc * RW::ss(a.mq) + ks * 16 + h * 8);
       const v8 raw = as_v8<T>(t);
 #pragma unroll
       for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
@@ -172,19 +173,17 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * NT;
       const int row = c / CPR, col = c % CPR;
-      const int kr = k0 + row;
-      u32x4 kk = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-      if (kr < a.sk) {
-        kk = *(const u32x4 *)(Kb + (size_t)kr * RW::ss(a.mk) + col * 8);
-        vv = *(const u32x4 *)(Vb + (size_t)kr * RW::ss(a.mv) + col * 8);
-      }
-      kst[i] = kk;
-      vst[i] = vv;
+      // keys past the end re-read the last row: their scores get -inf through the extra step, so P = 0
+      // meets finite values of V (unconditional loads do not stall on each other)
+      int kr = k0 + row;
+      kr = kr < a.sk ? kr : a.sk - 1;
+      kst[i] = *(const u32x4 *)(Kb + (size_t)kr * RW::ss(a.mk) + col * 8);
+      vst[i] = *(const u32x4 *)(Vb + (size_t)kr * RW::ss(a.mv) + col * 8);
     }
-    if (tid < BK) {
-      const int kr = k0 + tid;
+    {
+      const int kr = k0 + (tid & (BK - 1));
       mvalid = kr < a.sk;
-      if (MASK == kMaskPerKey && mvalid) mraw = mkey[kr];
+      if (MASK == kMaskPerKey) mraw = mkey[mvalid ? kr : a.sk - 1];
     }
   };
   auto lstore = [&](int stage) {
