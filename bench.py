@@ -284,6 +284,41 @@ def operator_legs(torch, steps, warmup):
     return legs
 
 
+def torch_sdpa_context(torch, steps, warmup):
+    """For scale only: PyTorch's own fused attention (torch.nn.functional.scaled_dot_product_attention,
+    whichever backend it selects) on the same GPU at the headline shape, [B,H,S,D] fp16 tensors -- the
+    same padding mask for the forward, and a forward + backward with dropout 0.1 (no mask, which its
+    fastest backend requires).  Not a baseline of the reference and not part of `value`."""
+    import torch.nn.functional as F
+    out = {}
+    try:
+        g = torch.Generator(device="cuda").manual_seed(5)
+        q, k, v = (torch.randn((B, H, S, D), dtype=torch.float16, device="cuda", generator=g) for _ in range(3))
+        m = torch.zeros(B, 1, 1, S, dtype=torch.float16, device="cuda")
+        for i in range(B):
+            m[i, 0, 0, 256 + 8 * i:] = -10000.0
+        with torch.no_grad():
+            ms, _ = time_steps(torch, lambda i: F.scaled_dot_product_attention(q, k, v, attn_mask=m), steps, warmup)
+            ms_nomask, _ = time_steps(torch, lambda i: F.scaled_dot_product_attention(q, k, v), steps, warmup)
+        out["fwd_pad_mask_us"] = round(ms * 1e3, 1)
+        out["fwd_no_mask_us"] = round(ms_nomask * 1e3, 1)
+        out["fwd_no_mask_tflops"] = round(4.0 * B * H * S * S * D / (ms_nomask * 1e-3) / 1e12, 1)
+        qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+        do = torch.randn_like(q)
+
+        def step(i):
+            o = F.scaled_dot_product_attention(qg, kg, vg, dropout_p=0.1)
+            o.backward(do)
+        n = max(10, steps // 10)
+        ms_t, _ = time_steps(torch, step, n, max(2, warmup // 10))
+        out["train_step_dropout_us"] = round(ms_t * 1e3, 1)
+        out["train_step_tflops"] = round(14.0 * B * H * S * S * D / (ms_t * 1e-3) / 1e12, 1)
+        out["torch"] = torch.__version__
+    except Exception as e:  # a context figure must never break the benchmark
+        out["unavailable"] = repr(e)[:200]
+    return out
+
+
 def power_probe(torch, step, seconds=2.0):
     """Socket power and graphics clocks as the board's management firmware reports them (amd-smi),
     sampled while `step` runs back to back on a second thread.  The attention kernels are
@@ -517,6 +552,7 @@ def main():
 
     out["short_sequences"] = short_sequence_legs(torch, capi, L, stream, args.steps, args.warmup)
     out["operators_BH512_S128_D64"] = operator_legs(torch, args.steps, args.warmup)
+    out["torch_sdpa_same_gpu"] = torch_sdpa_context(torch, args.steps, args.warmup)
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
