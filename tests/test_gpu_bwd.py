@@ -305,3 +305,34 @@ def test_large_scores_stay_finite_and_accurate(bh, sq, sk, mask, p, std):
         got = f32(t.cpu())
         assert np.isfinite(got).all(), name
         assert rel_to_max(got, ref[name]) <= 3e-2, name
+
+
+@pytest.mark.parametrize("bh,s,d,dtype", [(8, 8192, 64, "fp16"), (4, 4096, 128, "bf16")])
+def test_long_sequences_split_over_keys(bh, s, d, dtype):
+    """Sequences far beyond what the oracle finishes in seconds (128 key tiles), checked by an identity
+    instead: attention over all keys is the LSE-weighted merge of attention over the two halves of the
+    keys, and, given the full O and LSE, the backward over half the keys yields that half's dK and dV
+    and a dQ that sums to the full one."""
+    tdt = TDT[dtype]
+    q, k, v, do = (t.cuda() for t in make_qkv(bh, s, s, d, seed=s, std=0.5 if d == 128 else 1.0, dtype=dtype,
+                                              with_dout=True))
+    o, lse, _, _ = capi.fwd(q, k, v, want_lse=True)
+    h = s // 2
+    halves = [(k[:, :h].contiguous(), v[:, :h].contiguous()), (k[:, h:].contiguous(), v[:, h:].contiguous())]
+    parts = [capi.fwd(q, kk, vv, want_lse=True)[:2] for kk, vv in halves]
+    l1, l2 = parts[0][1].double(), parts[1][1].double()
+    lm = torch.logaddexp(l1, l2)
+    merged = parts[0][0].double() * (l1 - lm).exp().unsqueeze(-1) + parts[1][0].double() * (l2 - lm).exp().unsqueeze(-1)
+    otol = 2e-3 if dtype == "fp16" else 2e-2
+    assert (merged - o.double()).abs().max().item() <= otol
+    assert (lm - lse.double()).abs().max().item() <= 2e-3
+    # backward: the same O and LSE, half of the keys at a time
+    dq, dk, dv = capi.bwd(do, q, k, v, o, lse)
+    g = [capi.bwd(do, q, kk, vv, o, lse) for kk, vv in halves]
+    gtol = 1e-2 if dtype == "fp16" else 3e-2
+    for full, a, b in ((dk, g[0][1], g[1][1]), (dv, g[0][2], g[1][2])):
+        cat = torch.cat([a, b], dim=1).float()
+        assert (cat - full.float()).abs().max().item() <= gtol * full.float().abs().max().item()
+    dq_sum = g[0][0].float() + g[1][0].float()
+    assert (dq_sum - dq.float()).abs().max().item() <= gtol * dq.float().abs().max().item()
+    assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
