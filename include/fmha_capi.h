@@ -44,6 +44,13 @@ enum {
   FMHA_DROP_TENSOR = 2   /* caller supplies a multiplicative [bh,sq,sk] tensor (fmha_manual.cpp:478-480) */
 };
 
+/* fmha_fwd_params.flags.
+ * A [.., 1, sk] mask whose tail is hard-masked (mask term <= -9000, e.g. the -10000 or -inf of a
+ * padded batch) lets the forward skip the key tiles that hold nothing else; the skipped keys' weights
+ * are exactly zero unless a masked key's score exceeds every visible key's by more than 8800.
+ * FMHA_FLAG_NO_MASK_TRIM makes it visit every tile regardless. */
+enum { FMHA_FLAG_NO_MASK_TRIM = 1 };
+
 /* return codes */
 enum {
   FMHA_OK = 0,
@@ -100,7 +107,7 @@ typedef struct fmha_fwd_params {
   int32_t bh, sq, sk, d;
   int32_t dtype;
   float scale; /* > 0; 1/8 in the reference (fmha_manual.cpp:68) */
-  int32_t flags; /* reserved, pass 0 */
+  int32_t flags; /* 0 or FMHA_FLAG_NO_MASK_TRIM */
 
   /* Optional valid key counts (the "padded version" the reference leaves as a TODO,
    * fmha_manual.cpp:110,178): head b attends keys [0, kv_len[b / kv_len_bh_div]) only, exactly

@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfmha_hip.so")
 
 F16, BF16 = 0, 1
 MASK_NONE, MASK_ADDITIVE, MASK_KEEP01 = 0, 1, 2
+FLAG_NO_MASK_TRIM = 1  # fwd(flags=...): visit every key tile even where a per-key mask hard-masks the tail
 DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_philox_keep_mask", "fmha_drop_threshold",

@@ -68,6 +68,9 @@ struct FwdArgs {
   RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
 };
 
+// FwdArgs::flags
+enum { kFwdFlagNoTrim = 1 }; // visit every key tile even where a per-key mask hard-masks the tail
+
 // how the mask tensor is read
 enum { kMaskNone = 0, kMaskPerKey = 1, kMaskFull = 2 };
 

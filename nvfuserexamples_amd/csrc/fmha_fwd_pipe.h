@@ -49,7 +49,8 @@ template <int D, int QB> struct PipeCfg {
   // workgroups per CU; otherwise Q is loaded from global memory when the item starts.
   static constexpr bool QLDS = (D == 64);
   static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * XROWB; // {K,V} x 2 stages + extra rows x 2 stages
-  static constexpr int lds_bytes(int nw) { return LDS_BYTES + (QLDS ? nw * QB * 32 * D * 2 : 0); }
+  static constexpr int TRIM_BYTES = 128; // per-item key counts derived from a per-key mask, at the very end
+  static constexpr int lds_bytes(int nw) { return LDS_BYTES + (QLDS ? nw * QB * 32 * D * 2 : 0) + TRIM_BYTES; }
 };
 
 // The LDS operands of one steady-state iteration in issue order.  kind 0: V^T block of the
@@ -130,6 +131,53 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   int lb = blockIdx.x;
   if ((G & 7) == 0) lb = (lb & 7) * (G >> 3) + (lb >> 3);
 
+  // A per-key mask that ends in "hard" masked keys (a padded batch: -10000 or -inf on the tail of
+  // every sequence) leaves those keys with a weight of exactly zero, so the key tiles that hold
+  // nothing else need not be visited -- the same saving as valid key counts, for callers who only
+  // have the mask.  The workgroup looks at the mask rows of its (few) items once, in its prologue,
+  // sharing the trip to memory with the first item's Q and K tiles: one wave per row loads the
+  // whole row up front, a ballot per 64-key chunk gives the last key that is not hard-masked.  A row without any such key keeps its full range (a
+  // fully masked row is a plain softmax over all keys, reference fmha/fmha_manual.cpp:70).
+  // "Hard" means a mask term of -9000 or below (-10000 is -9984 in bf16): such a key's weight is
+  // exactly zero in fp32 unless its score exceeds every visible key's by more than 8800, a spread
+  // at which a -10000 mask would not mask in the reference either.  kFwdFlagNoTrim turns it off.
+  constexpr bool TRIM = MASK == kMaskPerKey;
+  constexpr int kTrimSlots = 4, kTrimChunks = 16; // items per workgroup (one wave each), 64-key chunks per row
+  static_assert(NW >= kTrimSlots, "one wave per item looks at its mask row");
+  constexpr float kHardMask = -9000.f * FMHA_LOG2E;
+  static_assert(kTrimSlots * 4 <= C::TRIM_BYTES, "key counts do not fit their LDS area");
+  int *trim_kend = (int *)(lds + C::lds_bytes(NW) - C::TRIM_BYTES); // exchanged through the dynamic LDS block
+  // The counts of the workgroup's items, by their order (item lb + n * G has ordinal n), as scalars:
+  // with one wave per SIMD an LDS read or a division per item would be paid in full.  They start
+  // at "no trimming" and are set by the workgroup prologue once the mask rows have been looked at.
+  int trim_n[kTrimSlots];
+#pragma unroll
+  for (int i = 0; i < kTrimSlots; ++i) trim_n[i] = a.sk;
+  // The mask rows are requested first of all (wave n: the row of the workgroup's n-th item, 64 keys
+  // per instruction), so that the item set-up and the first copies below run in their shadow.
+  const int ws = __builtin_amdgcn_readfirstlane(w);
+  const bool trim = TRIM && lb < nitems && lb + kTrimSlots * G >= nitems && a.sk > 0 && a.sk <= 64 * kTrimChunks &&
+                    !(a.flags & kFwdFlagNoTrim); // workgroup-uniform
+  T trim_mv[kTrimChunks];
+#pragma unroll
+  for (int c = 0; c < kTrimChunks; ++c) trim_mv[c] = (T)0.f;
+  if (TRIM && trim && ws < kTrimSlots) {
+    const int idx = lb + ws * G < nitems ? lb + ws * G : lb;
+    const T *mk = (const T *)a.mask + (size_t)(idx / (a.nqt * a.mask_div)) * a.mask_sb; // (idx / nqt) / mask_div
+#pragma unroll
+    for (int c = 0; c < kTrimChunks / 2; ++c) {
+      const int key = c * 64 + l;
+      trim_mv[c] = mk[key < a.sk ? key : a.sk - 1];
+    }
+    if (a.sk > 64 * kTrimChunks / 2) {
+#pragma unroll
+      for (int c = kTrimChunks / 2; c < kTrimChunks; ++c) {
+        const int key = c * 64 + l;
+        trim_mv[c] = mk[key < a.sk ? key : a.sk - 1];
+      }
+    }
+  }
+
   // Everything that depends on the item.  Keys: tiles [0, nkt), keys [0, kend); the tile count
   // is padded to even (nkt2) with an all-masked phantom tile so that the two x / P buffers and
   // the two LDS stages alternate with fixed roles across items as well.
@@ -166,6 +214,20 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     it.Kb = (const T *)a.k + RW::head(a.mk, it.bh, a.sk);
     it.Vb = (const T *)a.v + RW::head(a.mv, it.bh, a.sk);
     it.mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(it.bh / a.mask_div) * a.mask_sb : nullptr;
+    return it;
+  };
+  // The mask's own trailing hard-masked keys shorten an item after the fact: with n >= 1 live keys
+  // the range becomes [0, min(kend, n)) and the tile count follows from it (kend always lies in
+  // the item's last tile).
+  auto trim_count = [&](int ord) { return ord == 0 ? trim_n[0] : ord == 1 ? trim_n[1] : ord == 2 ? trim_n[2] : trim_n[3]; };
+  auto trimmed = [&](Item it, int ord) {
+    if (TRIM) {
+      const int n = trim_count(ord);
+      if (n < it.kend) {
+        it.kend = n;
+        it.nkt2 = ((n + BK - 1) / BK + 1) & ~1;
+      }
+    }
     return it;
   };
   Item cur = make_item(lb);
@@ -218,8 +280,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   XStage xs; // extra rows of the tile after next, in flight across iterations
   int nn_kend = cur.kend;      // key range and per-key mask of the item after next
   const T *nn_mkey = cur.mkey;
-  auto set_after_next = [&](int idx) {
-    const Item it = make_item(idx + 2 * G < nitems ? idx + 2 * G : idx);
+  auto set_after_next = [&](int idx, int ord) {
+    const bool has = idx + 2 * G < nitems;
+    const Item it = trimmed(make_item(has ? idx + 2 * G : idx), has ? ord + 2 : ord);
     nn_kend = it.kend;
     nn_mkey = it.mkey;
   };
@@ -649,7 +712,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   auto diag = [&](int t) { return CAUSAL && (t * BK + BK - 1 > q0w); };
 
   // ---- workgroup prologue: the first item's Q, K(0), K(1) and extra rows
-  set_after_next(lb);
   if (C::QLDS) dmaQ(cur);
   dmaK(0);
   dmaK(1);
@@ -657,16 +719,63 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     XStage x0, x1;
     gloadX(0, x0);
     gloadX(1, x1);
-    gloadX(2, xs);
+    // The third tile of the stream is the first item's tile 2 or, if trimming leaves it only two
+    // tiles, the next item's tile 0: both candidates are requested now, so that the choice does
+    // not cost a second trip to memory.
+    T xs_here = (T)0.f, xs_next = (T)0.f;
+    set_after_next(lb, 0);
+    if (TRIM) {
+      const int last = a.sk > 0 ? a.sk - 1 : 0;
+      const int ka = 2 * BK + (tid & (BK - 1)), kb = tid & (BK - 1);
+      xs_here = cur.mkey[ka < last ? ka : last];
+      xs_next = nxt.mkey[kb < last ? kb : last];
+    } else {
+      gloadX(2, xs);
+    }
+    // Up to here the items had their untrimmed key ranges: the tiles just requested hold real
+    // rows where a trimmed range would repeat its last row, which makes no difference to keys
+    // that are marked as past the end below.
+    if (TRIM) {
+      if (trim) {
+        if (ws < kTrimSlots) {
+          int last = -1;
+          auto chunk = [&](int c) {
+            const int key = c * 64 + l;
+            const bool live = key < a.sk && fmaf((float)trim_mv[c], a.mask_a, a.mask_b) > kHardMask;
+            const unsigned long long bal = __builtin_amdgcn_ballot_w64(live);
+            if (bal) last = c * 64 + 63 - __builtin_clzll(bal); // chunks ascend: the last hit wins
+          };
+#pragma unroll
+          for (int c = 0; c < kTrimChunks / 2; ++c) chunk(c);
+          if (a.sk > 64 * kTrimChunks / 2) {
+#pragma unroll
+            for (int c = kTrimChunks / 2; c < kTrimChunks; ++c) chunk(c);
+          }
+          if (l == 0) trim_kend[ws] = last < 0 ? a.sk : last + 1;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < kTrimSlots; ++i) trim_n[i] = __builtin_amdgcn_readfirstlane(trim_kend[i]);
+        cur = trimmed(cur, 0);
+        nxt = trimmed(nxt, lb + G < nitems ? 1 : 0);
+        const int nn = trim_count(lb + 2 * G < nitems ? 2 : 0);
+        nn_kend = nn < nn_kend ? nn : nn_kend;
+        x0.mvalid = (tid & (BK - 1)) < cur.kend;
+        x1.mvalid = BK + (tid & (BK - 1)) < cur.kend;
+      }
+      const bool here = 2 < cur.nkt2;
+      xs.mraw = here ? xs_here : xs_next;
+      xs.mvalid = here ? 2 * BK + (tid & (BK - 1)) < cur.kend : (tid & (BK - 1)) < nxt.kend;
+    }
     lstoreX(0, x0);
     lstoreX(1, x1);
   }
 
-  for (int idx = lb;;) {
+  for (int idx = lb, ord = 0;;) {
     const int nidx = idx + G;
     const bool more = nidx < nitems;
-    nxt = make_item(more ? nidx : idx);
-    set_after_next(idx);
+    nxt = trimmed(make_item(more ? nidx : idx), more ? ord + 1 : ord);
+    set_after_next(idx, ord);
     bh = cur.bh;
     q0w = cur.qt * QT + w * (QB * 32);
     if (DROP == 2) {
@@ -777,6 +886,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     }
     if (!more) break;
     idx = nidx;
+    ++ord;
     cur = nxt;
   }
   if (probe) {

@@ -344,3 +344,78 @@ def test_golden_fixture():
                         seed=int(f["seed"]), offset=int(f["offset"]), want_lse=True)
     assert np.abs(f32(o.cpu()) - f["o"]).max() <= 2e-3
     assert np.abs(lse.cpu().numpy() - f["lse"]).max() <= 1e-3
+
+
+# A [B,1,1,sk] mask that ends in hard-masked keys (-10000 or -inf on the tail of every padded
+# sequence) lets the pipelined forward skip the key tiles that hold nothing else.  The skipped
+# keys' weights are exactly zero either way, so the result must equal, bit for bit, that of a
+# launch which visits every tile (FLAG_NO_MASK_TRIM), and match the oracle like any other forward.
+def _tail_mask(kind, b, sk, seed):
+    g = torch.Generator().manual_seed(seed)
+    m = torch.zeros(b, 1, 1, sk)
+    lens = torch.randint(1, sk + 1, (b,), generator=g)
+    for i in range(b):
+        n = int(lens[i])
+        if kind == "tail":
+            m[i, ..., n:] = -10000.0
+        elif kind == "inf":
+            m[i, ..., n:] = float("-inf")
+        elif kind == "holes":                       # masked keys inside the live range as well
+            m[i, ..., n:] = -10000.0
+            m[i, 0, 0, torch.rand(sk, generator=g) < 0.3] = -10000.0
+        elif kind == "soft":                        # a tail that is NOT hard: nothing may be skipped
+            m[i, ..., n:] = -100.0
+        elif kind == "last_live":                   # only the very last key is visible
+            m[i, ..., : sk - 1] = -10000.0
+        elif kind == "some_rows_all_masked":        # a fully masked row is a softmax over all keys
+            m[i] = -10000.0 if i % 2 else 0.0
+            if not i % 2:
+                m[i, ..., n:] = -10000.0
+    return m
+
+
+TRIM = [
+    # bh, sq, sk, d, dtype, kind, causal, extra
+    (8, 512, 512, 64, "fp16", "tail", False, None),
+    (8, 512, 512, 64, "fp16", "inf", False, None),
+    (8, 512, 512, 64, "fp16", "holes", False, None),
+    (8, 512, 512, 64, "fp16", "soft", False, None),
+    (8, 256, 512, 64, "fp16", "last_live", False, None),
+    (8, 512, 512, 64, "fp16", "some_rows_all_masked", False, None),
+    (6, 300, 333, 64, "bf16", "tail", False, None),          # ragged; -10000 is -9984 in bf16
+    (4, 256, 1024, 64, "fp16", "tail", False, None),         # the longest rows that are looked at
+    (4, 128, 1100, 64, "fp16", "tail", False, None),         # beyond: not looked at
+    (4, 256, 320, 128, "bf16", "tail", False, None),
+    (4, 384, 384, 64, "fp16", "tail", True, None),           # causal: both limits apply
+    (8, 512, 512, 64, "fp16", "tail", False, "philox"),      # keep decisions depend on positions only
+    (8, 512, 512, 64, "fp16", "holes", False, "kv_len"),     # valid key counts on top of the mask
+    (600, 128, 256, 64, "fp16", "tail", False, None),        # several items per workgroup
+    (2400, 128, 256, 64, "fp16", "tail", False, None),       # more than are looked at: no trimming
+]
+
+
+@pytest.mark.parametrize("qb", [1, 2])
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,kind,causal,extra", TRIM)
+def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kind, causal, extra, qb, monkeypatch):
+    monkeypatch.setenv("FMHA_FWD_QB", str(qb))
+    b = bh // 2
+    q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype)
+    m = _tail_mask(kind, b, sk, seed=sk + bh).to(TDT[dtype])
+    kw = dict(mask=m.cuda(), causal=causal, want_lse=True)
+    kv = None
+    if extra == "philox":
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=0.1, seed=7, offset=3)
+    elif extra == "kv_len":
+        kv = torch.randint(0, sk + 1, (b,), generator=torch.Generator().manual_seed(5), dtype=torch.int32)
+        kw.update(kv_len=kv.cuda())
+    o, lse, _, _ = _run(q, k, v, **kw)
+    o_all, lse_all, _, _ = _run(q, k, v, flags=capi.FLAG_NO_MASK_TRIM, **kw)
+    assert torch.equal(o, o_all)
+    assert torch.equal(lse, lse_all)
+    if extra is None and bh <= 8:
+        ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), causal=causal, want=("o", "lse"))
+        assert np.abs(f32(o.cpu()) - ref["o"]).max() <= TOL[dtype]
+        # one visible key: the LSE is that key's score, whose rounding (Q is rounded once after scaling)
+        # goes with sum |q_i k_i| rather than with the score itself
+        slack = 4.0 if kind == "last_live" else 1.0
+        assert (np.abs(lse.cpu().numpy() - ref["lse"]) <= slack * LSE_TOL[dtype] + LSE_REL[dtype] * np.abs(ref["lse"])).all()
