@@ -44,11 +44,12 @@ enum {
   FMHA_DROP_TENSOR = 2   /* caller supplies a multiplicative [bh,sq,sk] tensor (fmha_manual.cpp:478-480) */
 };
 
-/* fmha_fwd_params.flags.
+/* fmha_fwd_params.flags, fmha_bwd_params.flags.
  * A [.., 1, sk] mask whose tail is hard-masked (mask term <= -9000, e.g. the -10000 or -inf of a
- * padded batch) lets the forward skip the key tiles that hold nothing else; the skipped keys' weights
- * are exactly zero unless a masked key's score exceeds every visible key's by more than 8800.
- * FMHA_FLAG_NO_MASK_TRIM makes it visit every tile regardless. */
+ * padded batch; rows of up to 1024 keys are looked at) lets forward and backward skip the key tiles
+ * that hold nothing else; the skipped keys' weights are exactly zero unless a masked key's score
+ * exceeds every visible key's by more than 8800.  FMHA_FLAG_NO_MASK_TRIM makes them visit every tile
+ * regardless. */
 enum { FMHA_FLAG_NO_MASK_TRIM = 1 };
 
 /* return codes */
@@ -171,7 +172,7 @@ typedef struct fmha_bwd_params {
   int32_t bh, sq, sk, d;
   int32_t dtype;
   float scale;
-  int32_t flags; /* reserved, pass 0 */
+  int32_t flags; /* 0 or FMHA_FLAG_NO_MASK_TRIM */
 
   const int32_t *kv_len; /* as in fmha_fwd_params; dk and dv rows at or past the count are zero */
   int32_t kv_len_bh_div;

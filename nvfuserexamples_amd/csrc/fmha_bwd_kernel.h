@@ -88,6 +88,54 @@ FMHA_DEV int bwd_valid_keys(const BwdArgs &a, int bh) {
   return n < 0 ? 0 : (n < a.sk ? n : a.sk);
 }
 
+// BwdArgs::flags
+enum { kBwdFlagNoTrim = 1 }; // visit every key tile even where a per-key mask hard-masks the tail
+
+// The mask's own say on how many keys a head sees.  A per-key mask that ends in hard-masked keys
+// (mask term of -9000 or below: the -10000 or -inf tail of a padded sequence) gives those keys
+// P = exp(score + mask - LSE) = 0 exactly, hence dS = 0: their tiles need not be visited and their
+// dK, dV rows are zero.  A workgroup loads its head's mask row when it starts (`issue`, NT threads,
+// rows of up to 1024 keys) and turns it into a key count once its own operand loads, issued behind
+// it, have been consumed (`finish`), so that the row costs no trip to memory of its own.  A row
+// without any live key keeps all its keys (its softmax is a plain one over all of them).
+template <typename T, int NT> struct MaskTail {
+  static constexpr int kMaxKeys = 1024, NCH = kMaxKeys / NT;
+  T v[NCH];
+  FMHA_DEV static bool enabled(const BwdArgs &a) { return a.sk > 0 && a.sk <= kMaxKeys && !(a.flags & kBwdFlagNoTrim); }
+  FMHA_DEV void issue(const BwdArgs &a, const T *mkey, int tid) {
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) v[c] = (T)0.f;
+    if (enabled(a)) { // uniform
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int key = c * NT + tid;
+        v[c] = mkey[key < a.sk ? key : a.sk - 1];
+      }
+    }
+  }
+  // `red`: NT / 64 ints of LDS that nothing else uses until this returns (two barriers inside)
+  FMHA_DEV int finish(const BwdArgs &a, int *red, int tid) {
+    if (!enabled(a)) return a.sk;
+    constexpr float kHardMask = -9000.f * FMHA_LOG2E;
+    int last = -1;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int key = c * NT + tid;
+      const bool live = key < a.sk && fmaf((float)v[c], a.mask_a, a.mask_b) > kHardMask;
+      const unsigned long long bal = __builtin_amdgcn_ballot_w64(live);
+      if (bal) last = c * NT + (tid & ~63) + 63 - __builtin_clzll(bal); // chunks ascend: the last hit wins
+    }
+    if ((tid & 63) == 0) red[tid >> 6] = last;
+    __syncthreads();
+    int top = -1;
+#pragma unroll
+    for (int ww = 0; ww < NT / 64; ++ww) top = red[ww] > top ? red[ww] : top;
+    top = __builtin_amdgcn_readfirstlane(top);
+    __syncthreads();
+    return top < 0 ? a.sk : top + 1;
+  }
+};
+
 // A value as hi + lo in the element type (|error| ~ 2^-2p relative), clamped to a large finite
 // negative number so that it may be multiplied by zero.
 template <typename T> FMHA_DEV void split_hi_lo(float v, T &hi, T &lo) {
@@ -134,6 +182,9 @@ __global__ __launch_bounds__(NW * 64)
   const int bh = bid / npair;
   const int pi = bid - bh * npair;
   const int npass = (paired && a.ntile - 1 - pi != pi) ? 2 : 1;
+  MaskTail<T, NT> tail;
+  int live_keys = a.sk; // the mask's own count of keys worth visiting
+  if (MASK == kMaskPerKey) tail.issue(a, (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb, tid);
   for (int pass = 0; pass < npass; ++pass) {
   const int qt = CAUSAL ? (pass == 0 ? a.ntile - 1 - pi : pi) : pi;
   const int q0w = qt * QT + w * (QB * 32);
@@ -209,7 +260,10 @@ __global__ __launch_bounds__(NW * 64)
     }
   }
 
-  const int skv = bwd_valid_keys(a, bh);
+  // (the tile area of LDS is idle here in the first pass: nothing has been copied yet)
+  if (MASK == kMaskPerKey && pass == 0) live_keys = tail.finish(a, (int *)lds, tid);
+  int skv = bwd_valid_keys(a, bh);
+  skv = live_keys < skv ? live_keys : skv;
   int nkt = (skv + BK - 1) / BK;
   if (nkt < 1) nkt = 1; // no valid key at all: one tile of keys that are all "past the end"
   if (CAUSAL) {
@@ -459,6 +513,9 @@ __global__ __launch_bounds__(NW * 64)
   const int bh = bid / npair;
   const int pi = bid - bh * npair;
   const int npass = (paired && a.ntile - 1 - pi != pi) ? 2 : 1;
+  MaskTail<T, NT> tail;
+  int live_keys = a.sk; // the mask's own count of keys worth visiting
+  if (MASK == kMaskPerKey) tail.issue(a, (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb, tid);
   for (int pass = 0; pass < npass; ++pass) {
   const int ktile = pass == 0 ? pi : a.ntile - 1 - pi;
   const int k0w = ktile * KT + w * (KB * 32);
@@ -537,7 +594,10 @@ __global__ __launch_bounds__(NW * 64)
 
   const int nqt = (a.sq + BQ - 1) / BQ;
   // first query tile that sees any of these keys; none at all if the whole key tile is invalid
-  const int qt0 = ktile * KT >= skv ? nqt : (CAUSAL ? (ktile * KT) / BQ : 0);
+  // (hard-masked keys already have P = 0 through their mask term; the count only decides whether the
+  // whole key tile can be left out.  LDS is idle here in the first pass.)
+  if (MASK == kMaskPerKey && pass == 0) live_keys = tail.finish(a, (int *)lds, tid);
+  const int qt0 = ktile * KT >= (live_keys < skv ? live_keys : skv) ? nqt : (CAUSAL ? (ktile * KT) / BQ : 0);
 
   // ---- staging: Q and dO tiles copied straight into LDS (rows past the end repeat the last
   // valid row); the per-query extra rows take the register path one tile further ahead, as in

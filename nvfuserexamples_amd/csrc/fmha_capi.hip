@@ -46,8 +46,8 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // the forward, FMHA_FWD_STREAM=0 keeps full-mask forwards on the pipelined kernel,
 // FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
 // one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
-// pairing of causal tiles in the backward, FMHA_FWD_TRIM=0 makes the forward visit key tiles that a
-// per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call).
+// pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
+// that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call).
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
   return e ? std::atoi(e) : dflt;
@@ -187,7 +187,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
-  if (!env_int("FMHA_FWD_TRIM", 1)) a.flags |= kFwdFlagNoTrim;
+  if (!env_int("FMHA_MASK_TRIM", 1)) a.flags |= kFwdFlagNoTrim;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
   a.clock_probe = (unsigned long long *)p->clock_probe;
@@ -317,6 +317,7 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   if (!(a.drop_scale > 0.f)) return FMHA_E_ARG;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
+  if (!env_int("FMHA_MASK_TRIM", 1)) a.flags |= kBwdFlagNoTrim;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
   int mrc;

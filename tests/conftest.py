@@ -41,6 +41,33 @@ def pad_mask(b, sk, lo, hi, seed=0, neg=-10000.0):
     return m
 
 
+def tail_mask(kind, b, sk, seed):
+    """[B,1,1,sk] additive masks with a (mostly hard-masked) tail per row, for the tests of key tiles
+    that are skipped because the mask leaves nothing in them."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    m = torch.zeros(b, 1, 1, sk)
+    lens = torch.randint(1, sk + 1, (b,), generator=g)
+    for i in range(b):
+        n = int(lens[i])
+        if kind == "tail":
+            m[i, ..., n:] = -10000.0
+        elif kind == "inf":
+            m[i, ..., n:] = float("-inf")
+        elif kind == "holes":                       # masked keys inside the live range as well
+            m[i, ..., n:] = -10000.0
+            m[i, 0, 0, torch.rand(sk, generator=g) < 0.3] = -10000.0
+        elif kind == "soft":                        # a tail that is NOT hard: nothing may be skipped
+            m[i, ..., n:] = -100.0
+        elif kind == "last_live":                   # only the very last key is visible
+            m[i, ..., : sk - 1] = -10000.0
+        elif kind == "some_rows_all_masked":        # a fully masked row is a softmax over all keys
+            m[i] = -10000.0 if i % 2 else 0.0
+            if not i % 2:
+                m[i, ..., n:] = -10000.0
+    return m
+
+
 def f32(t):
     return t.float().numpy()
 

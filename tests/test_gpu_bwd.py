@@ -9,7 +9,7 @@ import torch
 
 import oracle
 from nvfuserexamples_amd import capi
-from conftest import make_qkv, pad_mask, f32, rel_to_max
+from conftest import make_qkv, pad_mask, tail_mask, f32, rel_to_max
 
 pytestmark = pytest.mark.gpu
 
@@ -336,3 +336,50 @@ def test_long_sequences_split_over_keys(bh, s, d, dtype):
     dq_sum = g[0][0].float() + g[1][0].float()
     assert (dq_sum - dq.float()).abs().max().item() <= gtol * dq.float().abs().max().item()
     assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
+
+
+# A [B,1,1,sk] mask that ends in hard-masked keys lets the dQ kernel stop at the last live key tile
+# and the dK/dV kernel leave out key tiles past it.  Those keys have P = 0 exactly either way, so the
+# gradients must equal, bit for bit, those of launches that visit every tile (FLAG_NO_MASK_TRIM).
+BWD_TRIM = [
+    # bh, sq, sk, d, dtype, kind, causal, p, kv_len
+    (8, 512, 512, 64, "fp16", "tail", False, 0.0, False),
+    (8, 512, 512, 64, "fp16", "tail", False, 0.1, False),     # headline train-step shape (few heads)
+    (8, 512, 512, 64, "fp16", "inf", False, 0.0, False),
+    (8, 512, 512, 64, "fp16", "holes", False, 0.1, False),
+    (8, 512, 512, 64, "fp16", "soft", False, 0.0, False),
+    (8, 300, 512, 64, "fp16", "last_live", False, 0.0, False),
+    (8, 512, 512, 64, "fp16", "some_rows_all_masked", False, 0.1, False),
+    (6, 300, 333, 64, "bf16", "tail", False, 0.1, False),
+    (4, 300, 1024, 64, "fp16", "tail", False, 0.0, False),    # the longest rows that are looked at
+    (4, 300, 1100, 64, "fp16", "tail", False, 0.0, False),    # beyond: not looked at
+    (4, 320, 320, 128, "bf16", "tail", False, 0.1, False),
+    (4, 384, 384, 64, "fp16", "tail", True, 0.1, False),      # causal: tile pairs, both limits apply
+    (8, 512, 512, 64, "fp16", "holes", False, 0.0, True),     # valid key counts on top of the mask
+]
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,kind,causal,p,use_len", BWD_TRIM)
+def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kind, causal, p, use_len):
+    b = bh // 2
+    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
+    m = tail_mask(kind, b, sk, seed=sk + bh).to(TDT[dtype])
+    kw = dict(mask=m.cuda(), causal=causal)
+    okw = dict(causal=causal)
+    if p > 0:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=5, offset=1)
+        okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=5, offset=1)
+    if use_len:
+        kv = torch.randint(0, sk + 1, (b,), generator=torch.Generator().manual_seed(5), dtype=torch.int32)
+        kw.update(kv_len=kv.cuda())
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o, lse, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    grads = capi.bwd(doc, qc, kc, vc, o, lse, **kw)
+    grads_all = capi.bwd(doc, qc, kc, vc, o, lse, flags=capi.FLAG_NO_MASK_TRIM, **kw)
+    torch.cuda.synchronize()
+    for name, t, t_all in zip(("dq", "dk", "dv"), grads, grads_all):
+        assert torch.equal(t, t_all), name
+    if not use_len:
+        ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), dout=f32(do), want=("dq", "dk", "dv"), **okw)
+        for name, t in zip(("dq", "dk", "dv"), grads):
+            assert rel_to_max(f32(t.cpu()), ref[name], floor=1e-3) <= TOL[dtype], name

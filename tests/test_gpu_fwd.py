@@ -11,7 +11,7 @@ import torch
 
 import oracle
 from nvfuserexamples_amd import capi
-from conftest import make_qkv, pad_mask, f32
+from conftest import make_qkv, pad_mask, tail_mask, f32
 
 pytestmark = pytest.mark.gpu
 
@@ -350,30 +350,6 @@ def test_golden_fixture():
 # sequence) lets the pipelined forward skip the key tiles that hold nothing else.  The skipped
 # keys' weights are exactly zero either way, so the result must equal, bit for bit, that of a
 # launch which visits every tile (FLAG_NO_MASK_TRIM), and match the oracle like any other forward.
-def _tail_mask(kind, b, sk, seed):
-    g = torch.Generator().manual_seed(seed)
-    m = torch.zeros(b, 1, 1, sk)
-    lens = torch.randint(1, sk + 1, (b,), generator=g)
-    for i in range(b):
-        n = int(lens[i])
-        if kind == "tail":
-            m[i, ..., n:] = -10000.0
-        elif kind == "inf":
-            m[i, ..., n:] = float("-inf")
-        elif kind == "holes":                       # masked keys inside the live range as well
-            m[i, ..., n:] = -10000.0
-            m[i, 0, 0, torch.rand(sk, generator=g) < 0.3] = -10000.0
-        elif kind == "soft":                        # a tail that is NOT hard: nothing may be skipped
-            m[i, ..., n:] = -100.0
-        elif kind == "last_live":                   # only the very last key is visible
-            m[i, ..., : sk - 1] = -10000.0
-        elif kind == "some_rows_all_masked":        # a fully masked row is a softmax over all keys
-            m[i] = -10000.0 if i % 2 else 0.0
-            if not i % 2:
-                m[i, ..., n:] = -10000.0
-    return m
-
-
 TRIM = [
     # bh, sq, sk, d, dtype, kind, causal, extra
     (8, 512, 512, 64, "fp16", "tail", False, None),
@@ -400,7 +376,7 @@ def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kin
     monkeypatch.setenv("FMHA_FWD_QB", str(qb))
     b = bh // 2
     q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype)
-    m = _tail_mask(kind, b, sk, seed=sk + bh).to(TDT[dtype])
+    m = tail_mask(kind, b, sk, seed=sk + bh).to(TDT[dtype])
     kw = dict(mask=m.cuda(), causal=causal, want_lse=True)
     kv = None
     if extra == "philox":
