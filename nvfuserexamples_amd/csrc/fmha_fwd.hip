@@ -67,6 +67,24 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
   long long nblk = (long long)a.bh * a.nqt;
   if (nblk > 0x7fffffffLL) return 2;
   if (kPipe && nblk > resident) nblk = resident;
+  a.bal_rows = 0;
+  if (kPipe && MASK == kMaskPerKey && !CAUSAL && a.mask_div > 0 && a.bh % a.mask_div == 0) {
+    // shapes whose mask rows can be dealt to the workgroups by length (see FwdArgs::bal_rows): an
+    // additive mask (its values are compared as they are), rows of whole 16-byte pieces, at most 64
+    // pieces of 512 keys in all
+    const long long items = (long long)a.bh * a.nqt, ipr = (long long)a.mask_div * a.nqt, rows = a.bh / a.mask_div;
+    const bool shape = nblk % ipr == 0 && items % nblk == 0 && items / nblk >= 2 && items / nblk <= 4 &&
+                       rows == items / nblk * (nblk / ipr);
+    const bool mask_ok = a.mask_a == FMHA_LOG2E && a.mask_b == 0.f && a.sk % 8 == 0 && a.sk <= 1024 &&
+                         rows * ((a.sk + 511) / 512) <= 64 && a.mask_sb % 8 == 0 &&
+                         (reinterpret_cast<uintptr_t>(a.mask) & 15) == 0;
+    if (shape && mask_ok && !a.kv_len && !(a.flags & kFwdFlagNoTrim)) {
+      a.bal_rows = (int32_t)rows;
+      a.bal_ipr = (int32_t)ipr;
+      a.bal_R = (int32_t)(nblk / ipr);
+      a.bal_inv_ipr = 1.f / (float)ipr;
+    }
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(kNW * 64), kLds, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }

@@ -66,6 +66,15 @@ struct FwdArgs {
   int32_t kv_div;
   unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
   RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
+  // Balanced dealing of a per-key mask's rows over the persistent workgroups (pipelined kernel; set
+  // by its launch code, 0 rows = off).  It applies when every workgroup has the same number of items
+  // (2 to 4), one per round, and a round's items of one mask row (bal_ipr = heads per row x query
+  // tiles) fill whole groups of bal_ipr workgroups: round n of workgroup g * bal_ipr + r is item r of
+  // row g + n * bal_R.  Then the rows can be dealt to the groups by length without breaking that shape.
+  int32_t bal_rows;   // mask rows (= bh / mask_div)
+  int32_t bal_ipr;    // items per mask row
+  int32_t bal_R;      // rows per round = grid size / bal_ipr
+  float bal_inv_ipr;  // 1 / bal_ipr
 };
 
 // FwdArgs::flags

@@ -49,7 +49,7 @@ template <int D, int QB> struct PipeCfg {
   // workgroups per CU; otherwise Q is loaded from global memory when the item starts.
   static constexpr bool QLDS = (D == 64);
   static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * XROWB; // {K,V} x 2 stages + extra rows x 2 stages
-  static constexpr int TRIM_BYTES = 128; // per-item key counts derived from a per-key mask, at the very end
+  static constexpr int TRIM_BYTES = 256; // per-item key counts derived from a per-key mask, at the very end
   static constexpr int lds_bytes(int nw) { return LDS_BYTES + (QLDS ? nw * QB * 32 * D * 2 : 0) + TRIM_BYTES; }
 };
 
@@ -156,8 +156,41 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // The mask rows are requested first of all (wave n: the row of the workgroup's n-th item, 64 keys
   // per instruction), so that the item set-up and the first copies below run in their shadow.
   const int ws = __builtin_amdgcn_readfirstlane(w);
-  const bool trim = TRIM && lb < nitems && lb + kTrimSlots * G >= nitems && a.sk > 0 && a.sk <= 64 * kTrimChunks &&
-                    !(a.flags & kFwdFlagNoTrim); // workgroup-uniform
+  // Balanced mode (set up by the host when the shape allows it, see FwdArgs::bal_rows): every
+  // workgroup looks at ALL mask rows (16 bytes per lane and instruction, wave n takes every NW-th
+  // row or half row of 512 keys), so that all workgroups know every row's key count and can agree,
+  // without talking to each other, on a dealing of the rows that evens out their work: a
+  // workgroup's items come from one mask row per round; the first round keeps its row (its copies
+  // start before the counts are known), the later rounds hand the remaining rows out by their
+  // length, longest to the least loaded, in alternating order.
+  const bool bal = TRIM && !CAUSAL && a.bal_rows > 0 && lb < nitems;
+  const bool trim = TRIM && !bal && lb < nitems && lb + kTrimSlots * G >= nitems && a.sk > 0 &&
+                    a.sk <= 64 * kTrimChunks && !(a.flags & kFwdFlagNoTrim); // workgroup-uniform
+  constexpr int kBalSlots = 16; // (half) rows per wave
+  static_assert(kBalSlots * NW * 4 <= C::TRIM_BYTES, "row counts do not fit their LDS area");
+  u32x4 bal_mv[kBalSlots];
+  const int bal_halves = a.sk > 512 ? 2 : 1; // 512-key pieces per row
+  if (TRIM && bal) {
+    auto bal_load = [&](int sidx) {
+      const int gs = sidx * NW + ws; // which (row, half) this wave's slot covers
+      int row = bal_halves == 2 ? gs >> 1 : gs;
+      const int half = bal_halves == 2 ? gs & 1 : 0;
+      row = row < a.bal_rows ? row : a.bal_rows - 1;
+      int key0 = half * 512 + l * 8;
+      key0 = key0 < a.sk ? key0 : 0;
+      bal_mv[sidx] = *(const u32x4 *)((const T *)a.mask + (size_t)row * a.mask_sb + key0);
+    };
+#pragma unroll
+    for (int i = 0; i < kBalSlots / 2; ++i) bal_load(i);
+    if (a.bal_rows * bal_halves > kBalSlots / 2 * NW) {
+#pragma unroll
+      for (int i = kBalSlots / 2; i < kBalSlots; ++i) bal_load(i);
+    }
+  }
+  int bal_row[kTrimSlots]; // balanced mode: the mask row (= group of bal_ipr items) of the n-th item
+  int bal_r0 = 0;          // ... and the item's place within its row
+#pragma unroll
+  for (int i = 0; i < kTrimSlots; ++i) bal_row[i] = 0;
   T trim_mv[kTrimChunks];
 #pragma unroll
   for (int c = 0; c < kTrimChunks; ++c) trim_mv[c] = (T)0.f;
@@ -185,8 +218,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     int bh, qt, nkt2, kend;
     const T *Kb, *Vb, *mkey;
   };
-  auto make_item = [&](int idx) {
+  auto make_item = [&](int idx, int ord) {
     Item it;
+    if (TRIM && bal) { // the dealing decides which row's item this is
+      const int row = ord == 0 ? bal_row[0] : ord == 1 ? bal_row[1] : ord == 2 ? bal_row[2] : bal_row[3];
+      idx = row * a.bal_ipr + bal_r0;
+    }
     it.bh = idx / a.nqt;
     it.qt = idx - it.bh * a.nqt;
     // Causal items grow with the query tile.  A workgroup's items are G apart, which is often a
@@ -230,8 +267,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     }
     return it;
   };
-  Item cur = make_item(lb);
-  Item nxt = make_item(lb + G < nitems ? lb + G : lb); // without a successor the streams harmlessly re-read the item
+  if (TRIM && bal) { // until the dealing is known: every round keeps its own row
+    const int grp = (int)(((float)lb + 0.5f) * a.bal_inv_ipr);
+    bal_r0 = lb - grp * a.bal_ipr;
+#pragma unroll
+    for (int i = 0; i < kTrimSlots; ++i) bal_row[i] = grp + i * a.bal_R;
+  }
+  Item cur = make_item(lb, 0);
+  Item nxt = make_item(lb + G < nitems ? lb + G : lb, lb + G < nitems ? 1 : 0); // without a successor the streams harmlessly re-read the item
   int bh = cur.bh, q0w = cur.qt * QT + w * (QB * 32); // of the current item
 
   // ---- staging
@@ -282,7 +325,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   const T *nn_mkey = cur.mkey;
   auto set_after_next = [&](int idx, int ord) {
     const bool has = idx + 2 * G < nitems;
-    const Item it = trimmed(make_item(has ? idx + 2 * G : idx), has ? ord + 2 : ord);
+    const Item it = trimmed(make_item(has ? idx + 2 * G : idx, has ? ord + 2 : ord), has ? ord + 2 : ord);
     nn_kend = it.kend;
     nn_mkey = it.mkey;
   };
@@ -735,7 +778,85 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     // Up to here the items had their untrimmed key ranges: the tiles just requested hold real
     // rows where a trimmed range would repeat its last row, which makes no difference to keys
     // that are marked as past the end below.
-    if (TRIM) {
+    if (TRIM && bal) {
+      // ---- every row's count: a lane's eight keys are all hard-masked iff the smallest of their bit
+      // patterns, read as unsigned, is not below that of the threshold (negative numbers grow with
+      // their magnitude; anything non-negative is smaller)
+      const unsigned hard = __builtin_bit_cast(unsigned short, (T)(-9000.f));
+      int *part = trim_kend; // [kBalSlots * NW] keys up to the last live one, per (half) row
+      auto bal_count = [&](int sidx) {
+        const int gs = sidx * NW + ws;
+        const int half = bal_halves == 2 ? gs & 1 : 0;
+        const u32x4 r = bal_mv[sidx];
+        unsigned lo = 0xffffu;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned e0 = r[j] & 0xffffu, e1 = r[j] >> 16;
+          lo = e0 < lo ? e0 : lo;
+          lo = e1 < lo ? e1 : lo;
+        }
+        const bool live = half * 512 + l * 8 < a.sk && lo < hard;
+        const unsigned long long bl = __builtin_amdgcn_ballot_w64(live);
+        const int n = bl ? half * 512 + (64 - __builtin_clzll(bl)) * 8 : 0; // rounded up to the lane's 8 keys
+        if (l == 0) part[gs] = n;
+      };
+#pragma unroll
+      for (int i = 0; i < kBalSlots / 2; ++i) bal_count(i);
+      if (a.bal_rows * bal_halves > kBalSlots / 2 * NW) {
+#pragma unroll
+        for (int i = kBalSlots / 2; i < kBalSlots; ++i) bal_count(i);
+      }
+      __syncthreads();
+      // ---- lane i: row i.  (Every wave does the same arithmetic and arrives at the same scalars.)
+      const bool row_ok = l < a.bal_rows;
+      int len = 0;
+      if (row_ok) {
+        len = bal_halves == 2 ? (part[2 * l + 1] ? part[2 * l + 1] : part[2 * l]) : part[l];
+        len = len == 0 || len > a.sk ? a.sk : len; // no live key: a plain softmax over all keys
+      }
+      const int cls = (len + 2 * BK - 1) / (2 * BK); // work of an item: its tile pairs (1 .. 8)
+      const int R = a.bal_R;
+      const int grp = bal_row[0];
+      // position of each lane's row among the first round's rows (l < R) / the other rows, longest first
+      const unsigned long long below = l ? ~0ull >> (64 - l) : 0ull;
+      int pos = 0, above_first = 0, above_rest = 0;
+#pragma unroll
+      for (int c = kTrimChunks * 64 / (2 * BK); c >= 1; --c) {
+        const unsigned long long bf = __builtin_amdgcn_ballot_w64(row_ok && l < R && cls == c);
+        const unsigned long long br = __builtin_amdgcn_ballot_w64(row_ok && l >= R && cls == c);
+        if (cls == c) pos = l < R ? above_first + __builtin_popcountll(bf & below) : above_rest + __builtin_popcountll(br & below);
+        above_first += __builtin_popcountll(bf);
+        above_rest += __builtin_popcountll(br);
+      }
+      const int my_rank = __builtin_amdgcn_readlane(pos, grp); // 0: the longest first-round row
+      trim_n[0] = __builtin_amdgcn_readlane(len, grp);
+      const int rounds = a.bal_rows / R;
+#pragma unroll
+      for (int n = 1; n < kTrimSlots; ++n) {
+        // round n hands every (rounds-1)-th row of the sorted rest to the groups (so that each round
+        // spans all lengths), the longest to the group with the shortest first-round row in odd
+        // rounds, the other way round in even ones
+        const int want = ((n & 1) ? R - 1 - my_rank : my_rank) * (rounds - 1) + (n - 1);
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(row_ok && l >= R && pos == want);
+        const int row = n < rounds && hit ? __builtin_ctzll(hit) : grp;
+        bal_row[n] = row;
+        trim_n[n] = __builtin_amdgcn_readlane(len, row);
+      }
+      __syncthreads(); // the counts' LDS area is not written again, but keep the waves together as the other path does
+      cur = trimmed(cur, 0);
+      nxt = trimmed(make_item(0, lb + G < nitems ? 1 : 0), lb + G < nitems ? 1 : 0);
+      x0.mvalid = (tid & (BK - 1)) < cur.kend;
+      x1.mvalid = BK + (tid & (BK - 1)) < cur.kend;
+      const bool here = 2 < cur.nkt2;
+      xs.mraw = xs_here;
+      xs.mvalid = 2 * BK + (tid & (BK - 1)) < cur.kend;
+      if (!here) { // (rare: at most two tiles) the stream's third tile is the next item's first, known only now
+        const int kr = tid & (BK - 1);
+        xs.mvalid = kr < nxt.kend;
+        xs.mraw = nxt.mkey[xs.mvalid ? kr : (nxt.kend > 0 ? nxt.kend - 1 : 0)];
+      }
+      set_after_next(lb, 0);
+    } else if (TRIM) {
       if (trim) {
         if (ws < kTrimSlots) {
           int last = -1;
@@ -774,7 +895,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   for (int idx = lb, ord = 0;;) {
     const int nidx = idx + G;
     const bool more = nidx < nitems;
-    nxt = trimmed(make_item(more ? nidx : idx), more ? ord + 1 : ord);
+    nxt = trimmed(make_item(more ? nidx : idx, more ? ord + 1 : ord), more ? ord + 1 : ord);
     set_after_next(idx, ord);
     bh = cur.bh;
     q0w = cur.qt * QT + w * (QB * 32);

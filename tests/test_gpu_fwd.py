@@ -351,30 +351,42 @@ def test_golden_fixture():
 # keys' weights are exactly zero either way, so the result must equal, bit for bit, that of a
 # launch which visits every tile (FLAG_NO_MASK_TRIM), and match the oracle like any other forward.
 TRIM = [
-    # bh, sq, sk, d, dtype, kind, causal, extra
-    (8, 512, 512, 64, "fp16", "tail", False, None),
-    (8, 512, 512, 64, "fp16", "inf", False, None),
-    (8, 512, 512, 64, "fp16", "holes", False, None),
-    (8, 512, 512, 64, "fp16", "soft", False, None),
-    (8, 256, 512, 64, "fp16", "last_live", False, None),
-    (8, 512, 512, 64, "fp16", "some_rows_all_masked", False, None),
-    (6, 300, 333, 64, "bf16", "tail", False, None),          # ragged; -10000 is -9984 in bf16
-    (4, 256, 1024, 64, "fp16", "tail", False, None),         # the longest rows that are looked at
-    (4, 128, 1100, 64, "fp16", "tail", False, None),         # beyond: not looked at
-    (4, 256, 320, 128, "bf16", "tail", False, None),
-    (4, 384, 384, 64, "fp16", "tail", True, None),           # causal: both limits apply
-    (8, 512, 512, 64, "fp16", "tail", False, "philox"),      # keep decisions depend on positions only
-    (8, 512, 512, 64, "fp16", "holes", False, "kv_len"),     # valid key counts on top of the mask
-    (600, 128, 256, 64, "fp16", "tail", False, None),        # several items per workgroup
-    (2400, 128, 256, 64, "fp16", "tail", False, None),       # more than are looked at: no trimming
+    # bh, sq, sk, d, dtype, kind, causal, extra, heads per mask row
+    (8, 512, 512, 64, "fp16", "tail", False, None, 2),
+    (8, 512, 512, 64, "fp16", "inf", False, None, 2),
+    (8, 512, 512, 64, "fp16", "holes", False, None, 2),
+    (8, 512, 512, 64, "fp16", "soft", False, None, 2),
+    (8, 256, 512, 64, "fp16", "last_live", False, None, 2),
+    (8, 512, 512, 64, "fp16", "some_rows_all_masked", False, None, 2),
+    (6, 300, 333, 64, "bf16", "tail", False, None, 2),          # ragged; -10000 is -9984 in bf16
+    (4, 256, 1024, 64, "fp16", "tail", False, None, 2),         # the longest rows that are looked at
+    (4, 128, 1100, 64, "fp16", "tail", False, None, 2),         # beyond: not looked at
+    (4, 256, 320, 128, "bf16", "tail", False, None, 2),
+    (4, 384, 384, 64, "fp16", "tail", True, None, 2),           # causal: both limits apply
+    (8, 512, 512, 64, "fp16", "tail", False, "philox", 2),      # keep decisions depend on positions only
+    (8, 512, 512, 64, "fp16", "holes", False, "kv_len", 2),     # valid key counts on top of the mask
+    (600, 128, 256, 64, "fp16", "tail", False, None, 2),        # several items per workgroup
+    (2400, 128, 256, 64, "fp16", "tail", False, None, 2),       # more than are looked at: no trimming
+    # Shapes at which every workgroup of the persistent kernel has the same number of items (2 to 4)
+    # and the mask has at most 64 rows: there all mask rows are looked at by every workgroup and dealt
+    # to the workgroups by length, which changes which workgroup computes what but not the results.
+    (512, 512, 512, 64, "fp16", "tail", False, None, 16),        # the headline shape
+    (512, 512, 512, 64, "fp16", "holes", False, None, 16),
+    (512, 512, 512, 64, "fp16", "some_rows_all_masked", False, None, 16),
+    (512, 512, 512, 64, "fp16", "last_live", False, None, 16),
+    (512, 512, 512, 64, "fp16", "tail", False, "philox", 16),
+    (256, 512, 512, 64, "bf16", "tail", False, None, 16),        # two items per workgroup
+    (256, 1024, 1024, 64, "fp16", "tail", False, None, 16),      # rows of two 512-key halves
+    (384, 512, 520, 64, "fp16", "tail", False, None, 16),        # three items per workgroup; 520 keys
+    (512, 512, 512, 64, "fp16", "tail", False, None, 8),         # 64 mask rows
 ]
 
 
 @pytest.mark.parametrize("qb", [1, 2])
-@pytest.mark.parametrize("bh,sq,sk,d,dtype,kind,causal,extra", TRIM)
-def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kind, causal, extra, qb, monkeypatch):
+@pytest.mark.parametrize("bh,sq,sk,d,dtype,kind,causal,extra,heads", TRIM)
+def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kind, causal, extra, heads, qb, monkeypatch):
     monkeypatch.setenv("FMHA_FWD_QB", str(qb))
-    b = bh // 2
+    b = bh // heads
     q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype)
     m = tail_mask(kind, b, sk, seed=sk + bh).to(TDT[dtype])
     kw = dict(mask=m.cuda(), causal=causal, want_lse=True)
@@ -395,3 +407,23 @@ def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kin
         # goes with sum |q_i k_i| rather than with the score itself
         slack = 4.0 if kind == "last_live" else 1.0
         assert (np.abs(lse.cpu().numpy() - ref["lse"]) <= slack * LSE_TOL[dtype] + LSE_REL[dtype] * np.abs(ref["lse"])).all()
+
+
+@pytest.mark.parametrize("bh,heads", [(8, 2), (512, 16)])
+def test_skipped_key_tiles_are_never_read(bh, heads):
+    """K and V rows in key tiles that hold only hard-masked keys may hold anything, NaN included: the
+    forward does not visit them (unless told to, which is how this test knows that it tests something)."""
+    s, d, b = 512, 64, bh // heads
+    q, k, v = make_qkv(bh, s, s, d, seed=3)
+    lens = torch.randint(1, s - 128, (b,), generator=torch.Generator().manual_seed(9))
+    m = torch.zeros(b, 1, 1, s)
+    k4, v4 = k.view(b, heads, s, d), v.view(b, heads, s, d)
+    for i in range(b):
+        m[i, ..., lens[i]:] = -10000.0
+        first_unread = (int(lens[i]) + 127) // 128 * 128
+        k4[i, :, first_unread:] = float("nan")
+        v4[i, :, first_unread:] = float("nan")
+    o = _run(q, k, v, mask=m.half().cuda())[0]
+    assert not torch.isnan(o).any()
+    o_all = _run(q, k, v, mask=m.half().cuda(), flags=capi.FLAG_NO_MASK_TRIM)[0]
+    assert torch.isnan(o_all).view(b, -1).any(1).all()
