@@ -101,7 +101,7 @@ enum { kBwdFlagNoTrim = 1 }; // visit every key tile even where a per-key mask h
 template <typename T, int NT> struct MaskTail {
   static constexpr int kMaxKeys = 1024, NCH = kMaxKeys / NT;
   T v[NCH];
-  FMHA_DEV static bool enabled(const BwdArgs &a) { return a.sk > 0 && a.sk <= kMaxKeys && !(a.flags & kBwdFlagNoTrim); }
+  FMHA_DEV static bool enabled(const BwdArgs &a) { return a.sk > 128 && a.sk <= kMaxKeys && !(a.flags & kBwdFlagNoTrim); } // (128 keys or fewer: nothing to leave out)
   FMHA_DEV void issue(const BwdArgs &a, const T *mkey, int tid) {
 #pragma unroll
     for (int c = 0; c < NCH; ++c) v[c] = (T)0.f;

@@ -75,7 +75,7 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
     const long long items = (long long)a.bh * a.nqt, ipr = (long long)a.mask_div * a.nqt, rows = a.bh / a.mask_div;
     const bool shape = nblk % ipr == 0 && items % nblk == 0 && items / nblk >= 2 && items / nblk <= 4 &&
                        rows == items / nblk * (nblk / ipr);
-    const bool mask_ok = a.mask_a == FMHA_LOG2E && a.mask_b == 0.f && a.sk % 8 == 0 && a.sk <= 1024 &&
+    const bool mask_ok = a.mask_a == FMHA_LOG2E && a.mask_b == 0.f && a.sk % 8 == 0 && a.sk > 128 && a.sk <= 1024 &&
                          rows * ((a.sk + 511) / 512) <= 64 && a.mask_sb % 8 == 0 &&
                          (reinterpret_cast<uintptr_t>(a.mask) & 15) == 0;
     if (shape && mask_ok && !a.kv_len && !(a.flags & kFwdFlagNoTrim)) {

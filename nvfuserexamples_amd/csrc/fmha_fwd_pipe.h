@@ -164,7 +164,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // start before the counts are known), the later rounds hand the remaining rows out by their
   // length, longest to the least loaded, in alternating order.
   const bool bal = TRIM && !CAUSAL && a.bal_rows > 0 && lb < nitems;
-  const bool trim = TRIM && !bal && lb < nitems && lb + kTrimSlots * G >= nitems && a.sk > 0 &&
+  const bool trim = TRIM && !bal && lb < nitems && lb + kTrimSlots * G >= nitems && a.sk > 2 * BK && // (two tiles are the least)
                     a.sk <= 64 * kTrimChunks && !(a.flags & kFwdFlagNoTrim); // workgroup-uniform
   constexpr int kBalSlots = 16; // (half) rows per wave
   static_assert(kBalSlots * NW * 4 <= C::TRIM_BYTES, "row counts do not fit their LDS area");
