@@ -136,8 +136,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // nothing else need not be visited -- the same saving as valid key counts, for callers who only
   // have the mask.  The workgroup looks at the mask rows of its (few) items once, in its prologue,
   // sharing the trip to memory with the first item's Q and K tiles: one wave per row loads the
-  // whole row up front, a ballot per 64-key chunk gives the last key that is not hard-masked.  A row without any such key keeps its full range (a
-  // fully masked row is a plain softmax over all keys, reference fmha/fmha_manual.cpp:70).
+  // whole row up front, a ballot per 64-key chunk gives the last key that is not hard-masked.  A
+  // row without any such key keeps its full range (a fully masked row is a plain softmax over all
+  // keys, reference fmha/fmha_manual.cpp:70).
   // "Hard" means a mask term of -9000 or below (-10000 is -9984 in bf16): such a key's weight is
   // exactly zero in fp32 unless its score exceeds every visible key's by more than 8800, a spread
   // at which a -10000 mask would not mask in the reference either.  kFwdFlagNoTrim turns it off.
