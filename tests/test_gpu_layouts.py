@@ -162,3 +162,26 @@ def test_operators_and_autograd_take_strided_tensors():
     gp = packed.grad
     for i, a3 in enumerate(g3):
         assert torch.equal(gp[:, :, i].permute(0, 2, 1, 3).reshape(a3.shape), a3)
+
+
+def test_headline_shape_packed_projection_equals_folded_path():
+    """B32 H16 S512 D64 with a padding mask, read from a packed [B,S,3,H,D] buffer: at this shape the
+    forward deals the mask rows to its workgroups by length, in both layouts alike.  Full size, so the
+    check is bit-equality with the folded path (itself held to the oracle elsewhere), train step included."""
+    b, h, s, d = 32, 16, 512, 64
+    q, k, v, do = make_qkv(b * h, s, s, d, seed=21, with_dout=True)
+    kw = dict(mask=pad_mask(b, s, s // 2, s).half().cuda(), drop_kind=capi.DROP_PHILOX, p_drop=0.1, seed=3, offset=9)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o3, l3, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    g3 = capi.bwd(doc, qc, kc, vc, o3, l3, **kw)
+    q4, k4, v4 = _packed(qc, kc, vc, b, h)
+    o4, l4, _, _ = capi.fwd(q4, k4, v4, want_lse=True, **kw)
+    g4 = capi.bwd(_bshd(doc, b, h), q4, k4, v4, o4, l4, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(o4.reshape(b * h, s, d), o3)
+    assert torch.equal(l4.reshape(b * h, s), l3)
+    for a4, a3 in zip(g4, g3):
+        assert torch.equal(a4.reshape(a3.shape), a3)
+    # and without the dealing and the trimming
+    o0 = capi.fwd(q4, k4, v4, flags=capi.FLAG_NO_MASK_TRIM, **kw)[0]
+    assert torch.equal(o0, o4)
