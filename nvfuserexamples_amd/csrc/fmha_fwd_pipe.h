@@ -189,7 +189,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     }
   }
   int bal_row[kTrimSlots]; // balanced mode: the mask row (= group of bal_ipr items) of the n-th item
-  int bal_r0 = 0;          // ... and the item's place within its row
+  int bal_h0 = 0, bal_qt0 = 0; // ... and the item's head and query tile within its row
 #pragma unroll
   for (int i = 0; i < kTrimSlots; ++i) bal_row[i] = 0;
   T trim_mv[kTrimChunks];
@@ -221,12 +221,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   };
   auto make_item = [&](int idx, int ord) {
     Item it;
-    if (TRIM && bal) { // the dealing decides which row's item this is
-      const int row = ord == 0 ? bal_row[0] : ord == 1 ? bal_row[1] : ord == 2 ? bal_row[2] : bal_row[3];
-      idx = row * a.bal_ipr + bal_r0;
+    int mrow; // the item's mask row
+    if (TRIM && bal) {
+      // the dealing decides which row's item this is; its head and query tile within the row are the
+      // workgroup's own (no division: with one wave per SIMD its latency would be paid in full)
+      mrow = ord == 0 ? bal_row[0] : ord == 1 ? bal_row[1] : ord == 2 ? bal_row[2] : bal_row[3];
+      it.bh = mrow * a.mask_div + bal_h0;
+      it.qt = bal_qt0;
+    } else {
+      it.bh = idx / a.nqt;
+      it.qt = idx - it.bh * a.nqt;
+      mrow = MASK == kMaskPerKey ? it.bh / a.mask_div : 0;
     }
-    it.bh = idx / a.nqt;
-    it.qt = idx - it.bh * a.nqt;
     // Causal items grow with the query tile.  A workgroup's items are G apart, which is often a
     // multiple of the tiles per head, so the order of the tiles is reversed in every other
     // round: long and short items then alternate within each workgroup.  (Within a round the
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     it.nkt2 = (nkt + 1) & ~1;
     it.Kb = (const T *)a.k + RW::head(a.mk, it.bh, a.sk);
     it.Vb = (const T *)a.v + RW::head(a.mv, it.bh, a.sk);
-    it.mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(it.bh / a.mask_div) * a.mask_sb : nullptr;
+    it.mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)mrow * a.mask_sb : nullptr;
     return it;
   };
   // The mask's own trailing hard-masked keys shorten an item after the fact: with n >= 1 live keys
@@ -270,7 +276,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   };
   if (TRIM && bal) { // until the dealing is known: every round keeps its own row
     const int grp = (int)(((float)lb + 0.5f) * a.bal_inv_ipr);
-    bal_r0 = lb - grp * a.bal_ipr;
+    const int r0 = lb - grp * a.bal_ipr; // the item's place within its row: head r0 / nqt, query tile r0 % nqt
+    bal_h0 = r0 / a.nqt;
+    bal_qt0 = r0 - bal_h0 * a.nqt;
 #pragma unroll
     for (int i = 0; i < kTrimSlots; ++i) bal_row[i] = grp + i * a.bal_R;
   }
