@@ -829,8 +829,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       // position of each lane's row among the first round's rows (l < R) / the other rows, longest first
       const unsigned long long below = l ? ~0ull >> (64 - l) : 0ull;
       int pos = 0, above_first = 0, above_rest = 0;
-#pragma unroll
-      for (int c = kTrimChunks * 64 / (2 * BK); c >= 1; --c) {
+      for (int c = (a.sk + 2 * BK - 1) / (2 * BK); c >= 1; --c) { // the classes this key range can have
         const unsigned long long bf = __builtin_amdgcn_ballot_w64(row_ok && l < R && cls == c);
         const unsigned long long br = __builtin_amdgcn_ballot_w64(row_ok && l >= R && cls == c);
         if (cls == c) pos = l < R ? above_first + __builtin_popcountll(bf & below) : above_rest + __builtin_popcountll(br & below);
