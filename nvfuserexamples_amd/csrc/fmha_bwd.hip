@@ -1,5 +1,5 @@
 // Instantiates the backward kernels for one (element type, head dim, row layout kind) triple, chosen
-// with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1}, and exports their dispatcher.
+// with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128,256} -DFMHA_TU_STRIDED={0,1}, and exports their dispatcher.
 #include "fmha_launch.h"
 #ifndef FMHA_TU_STRIDED
 #define FMHA_TU_STRIDED 0
@@ -42,6 +42,7 @@ template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipS
   constexpr int kLdsQ = BwdCfg<FMHA_TU_D, bwd_dq_tile_rows<FMHA_TU_D>()>::LDS_BYTES;
   using CfgK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>;
   constexpr int kLdsK = CfgK::LDS_BYTES + (MASK == kMaskFull ? CfgK::MASK_BYTES : 0);
+  static_assert(kLdsQ <= 160 * 1024 && kLdsK <= 160 * 1024, "tiles do not fit the LDS of a compute unit");
   auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP, kStrided>;
   auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP, kStrided>;
   static const int attr = set_lds(kq, kLdsQ) | set_lds(kk, kLdsK);

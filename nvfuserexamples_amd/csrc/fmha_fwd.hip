@@ -1,5 +1,5 @@
 // Instantiates the forward kernel for one (element type, head dim, row layout kind) triple, chosen
-// with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1}, and exports its dispatcher.
+// with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128,256} -DFMHA_TU_STRIDED={0,1}, and exports its dispatcher.
 #include "fmha_launch.h"
 #include "fmha_fwd_pipe.h"
 #ifndef FMHA_TU_STRIDED
@@ -157,6 +157,25 @@ template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 
 } // namespace
 
+#if FMHA_TU_D == 256
+// Head dim 256: built for coverage, not tuned.  Every variant runs on the plain (not software-pipelined)
+// loop at one wave per SIMD: the output accumulators alone take 128 registers per lane.
+template <int MASK, bool CAUSAL> int plain_by_drop(FwdArgs &a, int drop, hipStream_t s) {
+  if (drop == 0) return launch<1, MASK, CAUSAL, 0, false>(a, s);
+  if (drop == 1) return launch<1, MASK, CAUSAL, 1, false>(a, s);
+  if (drop == 2 && !CAUSAL) return launch<1, MASK, false, 2, false>(a, s);
+  return 1;
+}
+
+int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
+  if (v.qb == 2 || v.short_keys || v.save_split || v.stream || kStrided) return 1;
+  if (v.mask == kMaskPerKey)
+    return v.causal ? plain_by_drop<kMaskPerKey, true>(a, v.drop, s) : plain_by_drop<kMaskPerKey, false>(a, v.drop, s);
+  if (v.mask == kMaskFull)
+    return v.causal ? plain_by_drop<kMaskFull, true>(a, v.drop, s) : plain_by_drop<kMaskFull, false>(a, v.drop, s);
+  return v.causal ? plain_by_drop<kMaskNone, true>(a, v.drop, s) : plain_by_drop<kMaskNone, false>(a, v.drop, s);
+}
+#else
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 #if defined(FMHA_DEV_MINIMAL) || FMHA_TU_STRIDED
   if (v.drop == 2 || v.qb == 2) return 1; // folded layout only
@@ -197,5 +216,6 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
 #endif
   return by_mask<1>(a, v, s);
 }
+#endif
 
 } // namespace fmha

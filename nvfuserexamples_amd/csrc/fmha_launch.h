@@ -1,6 +1,6 @@
 // Internal interface between the C-ABI translation unit and the per-(element type,
 // head dim) kernel translation units.  Each kernel TU is compiled once per
-// combination with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128} -DFMHA_TU_STRIDED={0,1} and exports
+// combination with -DFMHA_TU_BF16={0,1} -DFMHA_TU_D={64,128,256} -DFMHA_TU_STRIDED={0,1} and exports
 // one dispatcher per pass (the _strided ones read the row maps of the argument block; the
 // others assume folded contiguous tensors).
 #pragma once
@@ -26,6 +26,7 @@ int fwd_dispatch_f16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_f16_d256(FwdArgs &a, const FwdVariant &v, hipStream_t s);  // fp16, folded layout only
 int fwd_dispatch_f16_d64_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d128_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d64_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
@@ -43,6 +44,7 @@ int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_f16_d256(BwdArgs &a, const BwdVariant &v, hipStream_t s);  // fp16, folded layout only
 int bwd_dispatch_f16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d128_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);

@@ -44,12 +44,18 @@ CASES = [
     (2, 200, 333, 64, "fp16", None, True, 0.1),
     (2, 333, 200, 64, "fp16", "pad", True, 0.0),
     (2, 640, 640, 128, "bf16", None, True, 0.0),
+    # head dim 256 (fp16 only, built for coverage, not tuned)
+    (2, 256, 256, 256, "fp16", None, False, 0.0),
+    (2, 200, 333, 256, "fp16", "pad", False, 0.1),
+    (2, 130, 257, 256, "fp16", "add_full", False, 0.1),
+    (2, 320, 320, 256, "fp16", None, True, 0.0),
+    (3, 100, 77, 256, "fp16", "pad", True, 0.1),
 ]
 
 
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,mask,causal,p", CASES)
 def test_backward_matches_oracle(bh, sq, sk, d, dtype, mask, causal, p):
-    std = 0.5 if d == 128 else 1.0
+    std = {64: 1.0, 128: 0.5, 256: 0.35}[d]
     q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=std, dtype=dtype, with_dout=True)
     m = None
     if mask == "pad":

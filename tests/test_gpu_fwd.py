@@ -49,6 +49,12 @@ CASES = [
     (2, 256, 256, 128, "fp16", None, False),
     (2, 1024, 1024, 128, "bf16", None, True),         # wide-head bf16 causal
     (4, 192, 192, 64, "bf16", "pad", False),
+    # head dim 256 (fp16 only, built for coverage: plain loop, one wave per SIMD)
+    (2, 256, 256, 256, "fp16", None, False),
+    (2, 200, 333, 256, "fp16", "pad", False),
+    (2, 130, 257, 256, "fp16", "add_full", False),
+    (2, 320, 320, 256, "fp16", None, True),
+    (3, 100, 77, 256, "fp16", "pad", True),
 ]
 
 
@@ -56,7 +62,7 @@ CASES = [
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,mask,causal", CASES)
 def test_forward_matches_oracle(bh, sq, sk, d, dtype, mask, causal, qb, monkeypatch):
     monkeypatch.setenv("FMHA_FWD_QB", str(qb))
-    std = 0.5 if d == 128 else 1.0
+    std = {64: 1.0, 128: 0.5, 256: 0.35}[d]
     q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sq, std=std, dtype=dtype)
     m, mk = None, capi.MASK_ADDITIVE
     g = torch.Generator().manual_seed(sq)
