@@ -284,13 +284,12 @@ void set_mask_and_dropout(P &p, MaskLayout &m, const c10::optional<at::Tensor> &
 }
 
 
-// Head dims the kernels are not built for (anything but 64, 128 and -- fp16 only -- 256) run zero-padded to
+// Head dims the kernels are not built for (anything but 64, 128 and 256) run zero-padded to
 // the next built size: zero columns add nothing to Q.K^T, the padded columns of V give zero columns
 // of O (and zero columns of dO leave the other gradients untouched), so results are those of the
 // original head dim.  Costs a copy of every operand and the arithmetic on the padding.
-int64_t padded_head_dim(int64_t d, at::ScalarType t) {
-  const int64_t top = t == at::kHalf ? 256 : 128; // head dim 256 is built for fp16 only
-  TORCH_CHECK(d >= 1 && d <= top, "mha_manual: head dim must be in [1, ", top, "] for this element type, got ", d);
+int64_t padded_head_dim(int64_t d) {
+  TORCH_CHECK(d >= 1 && d <= 256, "mha_manual: head dim must be in [1, 256], got ", d);
   return d <= 64 ? 64 : d <= 128 ? 128 : 256;
 }
 at::Tensor pad_head_dim(const at::Tensor &x, int64_t to) {
@@ -299,7 +298,7 @@ at::Tensor pad_head_dim(const at::Tensor &x, int64_t to) {
 
 // q, k, v: [B*H,S,D] contiguous (the reference's layout) or [B,H,S,D] views of any batch / head /
 // row strides (e.g. x.view(B,S,H,D).transpose(1,2), or a slice of a packed QKV projection), read
-// in place (D = 64 or 128, fp16 folded tensors also 256; other head dims are padded, see above).  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
+// in place (D = 64 or 128, folded tensors also 256; other head dims are padded, see above).  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
 // (seed, offset); p_drop == 0 disables dropout.  Returns (O, LSE fp32): O in q's shape and
 // dimension order, LSE [B*H,Sq] or [B,H,Sq].
 std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,
@@ -309,7 +308,7 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tens
   TORCH_CHECK(q_.dim() >= 3 && k_.dim() == q_.dim() && v_.dim() == q_.dim() && k_.size(-1) == q_.size(-1) &&
                   v_.size(-1) == q_.size(-1),
               "mha_manual: q, k, v must be [B*H,S,D] or [B,H,S,D] with one head dim");
-  if (const int64_t d = q_.size(-1), dp = padded_head_dim(d, q_.scalar_type()); dp != d) {
+  if (const int64_t d = q_.size(-1), dp = padded_head_dim(d); dp != d) {
     auto [o, lse] = fmha_fwd(pad_head_dim(q_, dp), pad_head_dim(k_, dp), pad_head_dim(v_, dp), mask,
                              scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(d)), is_causal, p_drop, seed,
                              offset, kv_len);
@@ -360,7 +359,7 @@ fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, co
   TORCH_CHECK(q_.dim() >= 3 && k_.dim() == q_.dim() && v_.dim() == q_.dim() && k_.size(-1) == q_.size(-1) &&
                   v_.size(-1) == q_.size(-1) && dout_.sizes() == q_.sizes() && o_.sizes() == q_.sizes(),
               "mha_manual: q, k, v must be [B*H,S,D] or [B,H,S,D] with one head dim, dout and o shaped like q");
-  if (const int64_t d = q_.size(-1), dp = padded_head_dim(d, q_.scalar_type()); dp != d) {
+  if (const int64_t d = q_.size(-1), dp = padded_head_dim(d); dp != d) {
     auto [dq, dk, dv] = fmha_bwd(pad_head_dim(dout_, dp), pad_head_dim(q_, dp), pad_head_dim(k_, dp),
                                  pad_head_dim(v_, dp), pad_head_dim(o_, dp), lse, mask,
                                  scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(d)), is_causal, p_drop, seed,

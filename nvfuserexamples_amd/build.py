@@ -45,10 +45,11 @@ def _tus():
                 defs = [f"-DFMHA_TU_BF16={bf}", f"-DFMHA_TU_D={d}", f"-DFMHA_TU_STRIDED={strided}"]
                 tus.append(("fmha_fwd.hip", f"fmha_fwd_{tag}.o", defs))
                 tus.append(("fmha_bwd.hip", f"fmha_bwd_{tag}.o", defs))
-        if bf == 0:  # head dim 256: fp16, folded layout only
-            defs = ["-DFMHA_TU_BF16=0", "-DFMHA_TU_D=256", "-DFMHA_TU_STRIDED=0"]
-            tus.append(("fmha_fwd.hip", "fmha_fwd_f16_d256.o", defs))
-            tus.append(("fmha_bwd.hip", "fmha_bwd_f16_d256.o", defs))
+        # head dim 256: folded layout only
+        tag = f"{'bf16' if bf else 'f16'}_d256"
+        defs = [f"-DFMHA_TU_BF16={bf}", "-DFMHA_TU_D=256", "-DFMHA_TU_STRIDED=0"]
+        tus.append(("fmha_fwd.hip", f"fmha_fwd_{tag}.o", defs))
+        tus.append(("fmha_bwd.hip", f"fmha_bwd_{tag}.o", defs))
     return tus
 
 

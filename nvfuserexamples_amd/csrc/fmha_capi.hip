@@ -199,10 +199,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if ((mrc = make_row_map(a.mo, p->heads, p->o_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
   if (strided && (saving || p->drop_kind == FMHA_DROP_TENSOR)) return FMHA_E_UNSUPPORTED;
-  // Head dim 256 is built for fp16 and the folded layout only.  (The same kernels instantiated for bf16
-  // at this head dim gave wrong results in testing while fp16 at 256 and bf16 at 128 are right; until
-  // that is understood the combination is refused rather than served.)
-  if (p->d == 256 && (strided || p->dtype != FMHA_DTYPE_F16)) return FMHA_E_UNSUPPORTED;
+  if (p->d == 256 && strided) return FMHA_E_UNSUPPORTED; // head dim 256: folded layout only
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
@@ -264,7 +261,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   } else if (p->dtype == FMHA_DTYPE_F16)
     rc = p->d == 64 ? fwd_dispatch_f16_d64(a, v, s) : p->d == 128 ? fwd_dispatch_f16_d128(a, v, s) : fwd_dispatch_f16_d256(a, v, s);
   else
-    rc = p->d == 64 ? fwd_dispatch_bf16_d64(a, v, s) : fwd_dispatch_bf16_d128(a, v, s);
+    rc = p->d == 64 ? fwd_dispatch_bf16_d64(a, v, s) : p->d == 128 ? fwd_dispatch_bf16_d128(a, v, s) : fwd_dispatch_bf16_d256(a, v, s);
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 
@@ -334,10 +331,7 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   if ((mrc = make_row_map(a.mdq, p->heads, p->dq_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mdk, p->heads, p->dk_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mdv, p->heads, p->dv_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
-  // Head dim 256 is built for fp16 and the folded layout only.  (The same kernels instantiated for bf16
-  // at this head dim gave wrong results in testing while fp16 at 256 and bf16 at 128 are right; until
-  // that is understood the combination is refused rather than served.)
-  if (p->d == 256 && (strided || p->dtype != FMHA_DTYPE_F16)) return FMHA_E_UNSUPPORTED;
+  if (p->d == 256 && strided) return FMHA_E_UNSUPPORTED; // head dim 256: folded layout only
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
 
   BwdVariant v;
@@ -360,7 +354,7 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   } else if (p->dtype == FMHA_DTYPE_F16)
     rc = p->d == 64 ? bwd_dispatch_f16_d64(a, v, s) : p->d == 128 ? bwd_dispatch_f16_d128(a, v, s) : bwd_dispatch_f16_d256(a, v, s);
   else
-    rc = p->d == 64 ? bwd_dispatch_bf16_d64(a, v, s) : bwd_dispatch_bf16_d128(a, v, s);
+    rc = p->d == 64 ? bwd_dispatch_bf16_d64(a, v, s) : p->d == 128 ? bwd_dispatch_bf16_d128(a, v, s) : bwd_dispatch_bf16_d256(a, v, s);
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 

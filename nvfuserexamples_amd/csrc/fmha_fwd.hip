@@ -160,12 +160,14 @@ template <int QB> int by_mask(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 #if FMHA_TU_D == 256
 // Head dim 256: built for coverage, not tuned.  Every variant runs on the plain (not software-pipelined)
 // loop at one wave per SIMD: the output accumulators alone take 128 registers per lane.
+namespace { // (per translation unit: the element type differs between units of the same name)
 template <int MASK, bool CAUSAL> int plain_by_drop(FwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<1, MASK, CAUSAL, 0, false>(a, s);
   if (drop == 1) return launch<1, MASK, CAUSAL, 1, false>(a, s);
   if (drop == 2 && !CAUSAL) return launch<1, MASK, false, 2, false>(a, s);
   return 1;
 }
+} // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
   if (v.qb == 2 || v.short_keys || v.save_split || v.stream || kStrided) return 1;

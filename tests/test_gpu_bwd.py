@@ -44,12 +44,13 @@ CASES = [
     (2, 200, 333, 64, "fp16", None, True, 0.1),
     (2, 333, 200, 64, "fp16", "pad", True, 0.0),
     (2, 640, 640, 128, "bf16", None, True, 0.0),
-    # head dim 256 (fp16 only, built for coverage, not tuned)
+    # head dim 256 (built for coverage, not tuned)
     (2, 256, 256, 256, "fp16", None, False, 0.0),
     (2, 200, 333, 256, "fp16", "pad", False, 0.1),
     (2, 130, 257, 256, "fp16", "add_full", False, 0.1),
-    (2, 320, 320, 256, "fp16", None, True, 0.0),
-    (3, 100, 77, 256, "fp16", "pad", True, 0.1),
+    (2, 320, 320, 256, "bf16", None, True, 0.0),
+    (3, 100, 77, 256, "bf16", "pad", True, 0.1),
+    (2, 192, 192, 256, "fp16", "pad", True, 0.1),
 ]
 
 

@@ -49,12 +49,13 @@ CASES = [
     (2, 256, 256, 128, "fp16", None, False),
     (2, 1024, 1024, 128, "bf16", None, True),         # wide-head bf16 causal
     (4, 192, 192, 64, "bf16", "pad", False),
-    # head dim 256 (fp16 only, built for coverage: plain loop, one wave per SIMD)
+    # head dim 256 (built for coverage: plain loop, one wave per SIMD)
     (2, 256, 256, 256, "fp16", None, False),
     (2, 200, 333, 256, "fp16", "pad", False),
     (2, 130, 257, 256, "fp16", "add_full", False),
-    (2, 320, 320, 256, "fp16", None, True),
-    (3, 100, 77, 256, "fp16", "pad", True),
+    (2, 320, 320, 256, "bf16", None, True),
+    (3, 100, 77, 256, "bf16", "pad", True),
+    (2, 192, 192, 256, "fp16", "pad", True),
 ]
 
 
