@@ -113,7 +113,8 @@ typedef struct fmha_fwd_params {
   /* Optional valid key counts (the "padded version" the reference leaves as a TODO,
    * fmha_manual.cpp:110,178): head b attends keys [0, kv_len[b / kv_len_bh_div]) only, exactly
    * as if the others carried a -inf mask, and whole key tiles past the count are never touched.
-   * Device pointer to int32, or NULL for all sk keys.  Not with FMHA_DROP_TENSOR / the save outputs. */
+   * Device pointer to int32, or NULL for all sk keys.  Not with FMHA_DROP_TENSOR / the save outputs, nor at head dim 256
+   * (forward). */
   const int32_t *kv_len;
   int32_t kv_len_bh_div;
 

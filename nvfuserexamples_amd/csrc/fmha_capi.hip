@@ -153,7 +153,8 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (p->drop_kind == FMHA_DROP_TENSOR && p->causal) return FMHA_E_UNSUPPORTED;
   if (p->kv_len) {
     if (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u)) return FMHA_E_ARG;
-    if (saving || p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED;
+    // (the plain forward loop, which also serves head dim 256, does not read the counts)
+    if (saving || p->drop_kind == FMHA_DROP_TENSOR || p->d == 256) return FMHA_E_UNSUPPORTED;
   }
   if ((uintptr_t)p->clock_probe & 7u) return FMHA_E_ARG;
 

@@ -429,13 +429,16 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
               for (int r = 0; r < 16; r += 2) mx = max3(mx, x[qb][sb][r], x[qb][sb][r + 1]);
             mx = xhalf_max(mx);
             float mnew = mref[qb];
+            const bool had_ref = seen[qb];
             if (mx != NEG_INF) {
               const float cand = (float)(T)(mref[qb] + mx);
               mnew = seen[qb] ? fmaxf(mref[qb], cand) : cand;
               seen[qb] = true;
             }
             const float shift = mref[qb] - mnew;
-            if (shift != 0.f) {
+            // Nothing has been accumulated before the first reference is set, and that first move can be
+            // upwards by thousands (a first tile under a -10000 mask): 0 * 2^shift would be 0 * inf.
+            if (shift != 0.f && had_ref) {
               const float alpha = fast_exp2(shift);
               lsum[qb] *= alpha;
 #pragma unroll

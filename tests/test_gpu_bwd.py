@@ -361,6 +361,7 @@ BWD_TRIM = [
     (4, 300, 1024, 64, "fp16", "tail", False, 0.0, False),    # the longest rows that are looked at
     (4, 300, 1100, 64, "fp16", "tail", False, 0.0, False),    # beyond: not looked at
     (4, 320, 320, 128, "bf16", "tail", False, 0.1, False),
+    (2, 300, 333, 256, "fp16", "holes", False, 0.1, False),   # head dim 256: 32-row tiles
     (4, 384, 384, 64, "fp16", "tail", True, 0.1, False),      # causal: tile pairs, both limits apply
     (8, 512, 512, 64, "fp16", "holes", False, 0.0, True),     # valid key counts on top of the mask
 ]
@@ -369,7 +370,7 @@ BWD_TRIM = [
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,kind,causal,p,use_len", BWD_TRIM)
 def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kind, causal, p, use_len):
     b = bh // 2
-    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
+    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std={64: 1.0, 128: 0.5, 256: 0.35}[d], dtype=dtype, with_dout=True)
     m = tail_mask(kind, b, sk, seed=sk + bh).to(TDT[dtype])
     kw = dict(mask=m.cuda(), causal=causal)
     okw = dict(causal=causal)

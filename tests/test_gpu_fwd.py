@@ -290,6 +290,35 @@ def test_tensor_dropout_matches_oracle(bh, sq, sk, d, dtype, mask):
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= (4e-3 if dtype == "fp16" else 4e-2)   # O is up to 2x larger here
 
 
+@pytest.mark.parametrize("d,dtype", [(128, "fp16"), (128, "bf16"), (256, "fp16"), (256, "bf16")])
+@pytest.mark.parametrize("kind", ["first_tile", "first_key", "all", "all_but_last"])
+def test_plain_loop_under_masks_that_hide_the_first_keys(kind, d, dtype):
+    """The plain (not pipelined) forward loop -- tensor dropout at head dim 128, everything at head dim
+    256 -- sets its reference exponent at the first tile that has a finite score.  Under a -10000 mask
+    that first reference lies thousands below zero and the next one thousands above it; neither move may
+    touch the (still empty) sums.  A fully masked row is a plain softmax (reference fmha/fmha_manual.cpp:70)."""
+    bh, sq, sk = 4, 100, 200
+    q, k, v = make_qkv(bh, sq, sk, d, seed=d + sk, std=0.5 if d == 128 else 0.35, dtype=dtype)
+    m = torch.zeros(2, 1, 1, sk)
+    if kind == "first_tile":
+        m[..., :64] = -10000.0
+    elif kind == "first_key":
+        m[..., 0] = -10000.0
+    elif kind == "all":
+        m[0] = -10000.0
+    elif kind == "all_but_last":
+        m[..., : sk - 1] = -10000.0
+    m = m.to(TDT[dtype])
+    kw, okw = {}, {}
+    if d == 128:  # the dropout tensor (all ones) is what selects the plain loop at this head dim
+        dm = torch.ones(bh, sq, sk).to(TDT[dtype])
+        kw, okw = dict(drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=1.0), dict(drop_mask=f32(dm), drop_scale=1.0)
+    o = _run(q, k, v, mask=m.cuda(), **kw)[0]
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), want=("o",), **okw)
+    assert not torch.isnan(o).any()
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= TOL[dtype]
+
+
 def test_a_caller_built_against_an_older_header_keeps_working():
     """The parameter struct carries its own size: the library reads that many bytes and takes the fields
     beyond them as zero, whatever the memory after a shorter struct holds."""
