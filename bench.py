@@ -284,6 +284,31 @@ def operator_legs(torch, steps, warmup):
     return legs
 
 
+def head_dim_256_leg(torch, capi):
+    """Head dim 256 (built for coverage, not tuned): forward and backward at BH 128, S 2048, fp16, no mask."""
+    bh, s, d = 128, 2048, 256
+    g = torch.Generator().manual_seed(3)
+    q, k, v, do = ((torch.randn(bh, s, d, generator=g) * 0.35).to(torch.float16).cuda() for _ in range(4))
+    o, lse, _, _ = capi.fwd(q, k, v, want_lse=True)
+    grads = capi.bwd(do, q, k, v, o, lse)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    torch.cuda.synchronize()
+    n = 5
+    ev[0].record()
+    for _ in range(n):
+        capi.fwd(q, k, v, want_lse=True, out=o)
+    ev[1].record()
+    for _ in range(n):
+        capi.bwd(do, q, k, v, o, lse, grads=grads)
+    ev[2].record()
+    torch.cuda.synchronize()
+    f_ms, b_ms = ev[0].elapsed_time(ev[1]) / n, ev[1].elapsed_time(ev[2]) / n
+    flops = 4.0 * bh * s * s * d
+    return {"workload": "BH128 S2048 D256 fp16, no mask (includes the wrappers' output allocation where they allocate)",
+            "fwd_us": round(f_ms * 1e3, 1), "fwd_tflops": round(flops / (f_ms * 1e-3) / 1e12, 1),
+            "bwd_us": round(b_ms * 1e3, 1), "bwd_tflops": round(2.5 * flops / (b_ms * 1e-3) / 1e12, 1)}
+
+
 def torch_sdpa_context(torch, steps, warmup):
     """For scale only: PyTorch's own fused attention (torch.nn.functional.scaled_dot_product_attention,
     whichever backend it selects) on the same GPU at the headline shape, [B,H,S,D] fp16 tensors -- the
@@ -578,6 +603,7 @@ def main():
     out["short_sequences"] = short_sequence_legs(torch, capi, L, stream, args.steps, args.warmup)
     out["operators_BH512_S128_D64"] = operator_legs(torch, args.steps, args.warmup)
     out["torch_sdpa_same_gpu"] = torch_sdpa_context(torch, args.steps, args.warmup)
+    out["head_dim_256"] = head_dim_256_leg(torch, capi)
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
