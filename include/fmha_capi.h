@@ -50,7 +50,14 @@ enum {
  * that hold nothing else; the skipped keys' weights are exactly zero unless a masked key's score
  * exceeds every visible key's by more than 8800.  FMHA_FLAG_NO_MASK_TRIM makes them visit every tile
  * regardless. */
-enum { FMHA_FLAG_NO_MASK_TRIM = 1 };
+enum {
+  FMHA_FLAG_NO_MASK_TRIM = 1,
+  /* backward only: take the one-pass kernel where it applies (head dim 64, up to 512 keys, no causal
+   * mask, no [.., sq, sk] mask tensor; beyond 256 keys only with `workspace`).  It forms scores,
+   * exponentials and dropout decisions once instead of once per kernel, and measures level with the
+   * default two-kernel path at best, so it is never chosen unasked. */
+  FMHA_FLAG_BWD_ONE_PASS = 2
+};
 
 /* return codes */
 enum {
@@ -173,7 +180,7 @@ typedef struct fmha_bwd_params {
   int32_t bh, sq, sk, d;
   int32_t dtype;
   float scale;
-  int32_t flags; /* 0 or FMHA_FLAG_NO_MASK_TRIM */
+  int32_t flags; /* 0 or FMHA_FLAG_NO_MASK_TRIM | FMHA_FLAG_BWD_ONE_PASS */
 
   const int32_t *kv_len; /* as in fmha_fwd_params; dk and dv rows at or past the count are zero */
   int32_t kv_len_bh_div;
@@ -182,9 +189,19 @@ typedef struct fmha_bwd_params {
   int32_t heads;
   int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3], do_stride[3];
   int64_t dq_stride[3], dk_stride[3], dv_stride[3];
+
+  /* Optional scratch in device memory (16-byte aligned; contents before and after the call are
+   * meaningless), used with FMHA_FLAG_BWD_ONE_PASS only: with at least
+   * fmha_bwd_workspace_bytes(bh, sq, sk, d) bytes of it, heads of 257 to 512 keys can take the one-pass
+   * kernel, which keeps fp32 partial sums of dq there between the two halves of the key range. */
+  void *workspace;
+  uint64_t workspace_bytes;
 } fmha_bwd_params;
 
 int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);
+
+/* Workspace the backward can make use of for these sizes (0: none). */
+uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d);
 
 /*
  * Materialise the Philox keep decisions the kernels use for (seed, offset, p_drop)
@@ -201,6 +218,11 @@ uint32_t fmha_drop_threshold(float p_drop);
 
 /* Static description of a return code. */
 const char *fmha_strerror(int code);
+
+/* The FMHA_* environment variables (tuning and test overrides of the variant selection, listed in
+ * INTEGRATION.md) are read once per process, on the first launch.  This reads them again; not to be
+ * called while another thread is launching.  (No counterpart in the reference.) */
+void fmha_reload_overrides(void);
 
 /* Library version, "major.minor". */
 const char *fmha_version(void);

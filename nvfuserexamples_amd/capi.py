@@ -13,10 +13,23 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfmha_hip.so")
 F16, BF16 = 0, 1
 MASK_NONE, MASK_ADDITIVE, MASK_KEEP01 = 0, 1, 2
 FLAG_NO_MASK_TRIM = 1  # fwd(flags=...): visit every key tile even where a per-key mask hard-masks the tail
+FLAG_BWD_ONE_PASS = 2  # bwd(flags=...): the one-pass backward kernel where it applies
 DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
-EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_philox_keep_mask", "fmha_drop_threshold",
-           "fmha_strerror", "fmha_version")
+EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
+           "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides")
+# environment overrides the library reads once; the wrappers below make it read them again when they change
+_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB",
+              "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
+_env_seen = None
+
+
+def _sync_env():
+    global _env_seen
+    now = tuple(os.environ.get(n) for n in _ENV_NAMES)
+    if now != _env_seen:
+        lib().fmha_reload_overrides()
+        _env_seen = now
 
 
 class _Params(C.Structure):
@@ -65,6 +78,7 @@ class BwdParams(_Params):
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("o_stride", C.c_int64 * 3), ("do_stride", C.c_int64 * 3),
         ("dq_stride", C.c_int64 * 3), ("dk_stride", C.c_int64 * 3), ("dv_stride", C.c_int64 * 3),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
     ]
 
 
@@ -90,6 +104,8 @@ def lib():
         L.fmha_fwd_launch.restype = C.c_int
         L.fmha_bwd_launch.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         L.fmha_bwd_launch.restype = C.c_int
+        L.fmha_bwd_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+        L.fmha_bwd_workspace_bytes.restype = C.c_uint64
         L.fmha_philox_keep_mask.argtypes = [C.c_uint64, C.c_uint64, C.c_float, C.c_int32, C.c_int32,
                                             C.c_int32, C.c_void_p, C.c_void_p]
         L.fmha_philox_keep_mask.restype = C.c_int
@@ -98,6 +114,8 @@ def lib():
         L.fmha_strerror.argtypes = [C.c_int]
         L.fmha_strerror.restype = C.c_char_p
         L.fmha_version.restype = C.c_char_p
+        L.fmha_reload_overrides.argtypes = []
+        L.fmha_reload_overrides.restype = None
         _lib = L
     return _lib
 
@@ -241,15 +259,19 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
         P.save_softmax, P.save_dropout = sm.data_ptr(), dr.data_ptr()
     P.flags = flags
     _set_kv_len(P, kv_len, bh)
+    _sync_env()
     check(lib().fmha_fwd_launch(C.byref(P), _stream_ptr()))
     return o, lse, sm, dr
 
 
 def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False,
         scale=None, drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
-        flags=0, delta=None, grads=None, kv_len=None):
+        flags=0, delta=None, grads=None, kv_len=None, workspace=True):
     """Launch the backward on the current stream.  Returns (dq, dk, dv).  kv_len and the tensor
-    layouts as in fwd(); each gradient comes back in its input's dimension order."""
+    layouts as in fwd(); each gradient comes back in its input's dimension order.
+
+    workspace: True allocates the scratch that fmha_bwd_workspace_bytes() asks for (if any), a uint8
+    device tensor is passed on as it is, None / False passes none (the two-kernel path beyond 256 keys)."""
     import torch
     bh, sq, d, heads, qs = _rows(q, "q")
     _, sk, _, hk, ks = _rows(k, "k")
@@ -291,6 +313,12 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     P.seed, P.offset = seed, offset
     P.flags = flags
     _set_kv_len(P, kv_len, bh)
+    if workspace is True:
+        need = lib().fmha_bwd_workspace_bytes(bh, sq, sk, d)
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device) if need else None
+    if workspace is not None and workspace is not False:
+        P.workspace, P.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    _sync_env()
     check(lib().fmha_bwd_launch(C.byref(P), _stream_ptr()))
     return dq, dk, dv
 

@@ -53,6 +53,7 @@ struct BwdArgs {
   const int32_t *kv_len; // optional valid key count per group of kv_div heads
   int32_t kv_div;
   RowMap mq, mk, mv, mo, mdo, mdq, mdk, mdv; // row layouts (mk.ss == mv.ss)
+  float *ws; // one-pass kernel only: fp32 partial dQ sums between key chunks
 };
 
 // BT: rows per LDS tile (keys in the dQ kernel, queries in the dK/dV kernel).  The dK/dV kernel

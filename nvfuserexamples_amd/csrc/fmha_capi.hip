@@ -48,9 +48,29 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
 // pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
 // that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call).
+// The environment is read once per process (on the first launch); fmha_reload_overrides() reads it again.
+struct Overrides {
+  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, bwd_pair, bwd_short, bwd_fused;
+};
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
   return e ? std::atoi(e) : dflt;
+}
+Overrides read_overrides() {
+  Overrides o;
+  o.mask_trim = env_int("FMHA_MASK_TRIM", 1);
+  o.fwd_short = env_int("FMHA_FWD_SHORT", 1);
+  o.fwd_save_split = env_int("FMHA_FWD_SAVE_SPLIT", 1);
+  o.fwd_stream = env_int("FMHA_FWD_STREAM", 1);
+  o.fwd_qb = env_int("FMHA_FWD_QB", 0);
+  o.bwd_pair = env_int("FMHA_BWD_PAIR", -1);
+  o.bwd_short = env_int("FMHA_BWD_SHORT", 1);
+  o.bwd_fused = env_int("FMHA_BWD_FUSED", 0);
+  return o;
+}
+Overrides &overrides() {
+  static Overrides o = read_overrides();
+  return o;
 }
 
 } // namespace
@@ -69,16 +89,18 @@ const char *fmha_strerror(int code) {
   case FMHA_OK: return "ok";
   case FMHA_E_NULL: return "a required pointer is NULL";
   case FMHA_E_DTYPE: return "unknown dtype (0 = fp16, 1 = bf16)";
-  case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64 or 128, and one head's rows must span less than 2^31 elements";
+  case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64, 128 or 256, and one head's rows must span less than 2^31 elements";
   case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned and their strides multiples of 8 elements";
   case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
-  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal and Philox; the backward takes Philox dropout only; k and v rows must be equally far apart)";
+  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart; head dim 256 takes folded tensors only and, in the forward, no valid key counts)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
   default: return "unknown error code";
   }
 }
 
-const char *fmha_version(void) { return "0.1"; }
+const char *fmha_version(void) { return "0.2"; }
+
+void fmha_reload_overrides(void) { overrides() = read_overrides(); }
 
 int fmha_philox_keep_mask(uint64_t seed, uint64_t offset, float p_drop, int32_t bh, int32_t sq,
                           int32_t sk, uint8_t *out, void *hip_stream) {
@@ -188,7 +210,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   a.drop_scale = p->drop_kind == FMHA_DROP_NONE ? 1.f : p->drop_scale;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
-  if (!env_int("FMHA_MASK_TRIM", 1)) a.flags |= kFwdFlagNoTrim;
+  if (!overrides().mask_trim) a.flags |= kFwdFlagNoTrim;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
   a.clock_probe = (unsigned long long *)p->clock_probe;
@@ -213,21 +235,21 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  v.drop != 1 && !p->kv_len && aligned16(a.mask) && (a.mask_sb % 8) == 0 && (a.mask_sq % 8) == 0 &&
                  (!a.drop_mask || aligned16(a.drop_mask)) && (!a.save_softmax || aligned16(a.save_softmax)) &&
                  (!a.save_dropout || aligned16(a.save_dropout)) && (!saving || a.drop_mask) &&
-                 env_int("FMHA_FWD_SHORT", 1) != 0;
+                 overrides().fwd_short != 0;
   // Longer key ranges: where the caller provides an LSE buffer, the save-intermediates operator is the forward
   // launch followed by a streaming kernel that derives both saved outputs from that LSE (instead of a second
   // sweep inside a slower forward).  Same alignment needs as above.
   v.save_split = saving && !v.short_keys && !strided && p->d == 64 && p->lse && (p->sk % 8) == 0 &&
                  v.mask == kMaskFull && !v.causal && a.drop_mask && aligned16(a.mask) && (a.mask_sb % 8) == 0 &&
                  (a.mask_sq % 8) == 0 && aligned16(a.drop_mask) && (!a.save_softmax || aligned16(a.save_softmax)) &&
-                 (!a.save_dropout || aligned16(a.save_dropout)) && env_int("FMHA_FWD_SAVE_SPLIT", 1) != 0;
+                 (!a.save_dropout || aligned16(a.save_dropout)) && overrides().fwd_save_split != 0;
   if (v.save_split) v.saving = false; // the forward launch itself saves nothing
   // Other forwards under an aligned full mask tensor (with or without a dropout tensor) are memory time at
   // head dim 64: the streaming kernel.
   v.stream = !v.short_keys && !v.saving && !strided && p->d == 64 && (p->sk % 8) == 0 && v.mask == kMaskFull &&
              !v.causal && v.drop != 1 && !p->kv_len && aligned16(a.mask) && (a.mask_sb % 8) == 0 &&
              (a.mask_sq % 8) == 0 && (v.drop != 2 || (a.drop_mask && aligned16(a.drop_mask))) &&
-             env_int("FMHA_FWD_STREAM", 1) != 0;
+             overrides().fwd_stream != 0;
   // Two 32-query blocks per wave (on tiles of 32 keys) halve the LDS operand traffic per
   // flop.  That pays (4-6 % measured) for the unmasked variant at head dim 64 on long key
   // ranges when there is enough work for every resident workgroup to get several 256-query
@@ -248,7 +270,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
     const bool little_padding = tiles2 * 256 - p->sq <= p->sq / 8;
     if (cus > 0 && items2 >= 4LL * cus && little_padding && p->sk >= 1024) v.qb = 2;
   }
-  const int force = env_int("FMHA_FWD_QB", 0); // tuning override: 1 or 2
+  const int force = overrides().fwd_qb; // tuning override: 1 or 2
   if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;
   if (strided) v.qb = 1; // the two-block variant is built for the folded layout only
 
@@ -264,6 +286,11 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   else
     rc = p->d == 64 ? fwd_dispatch_bf16_d64(a, v, s) : p->d == 128 ? fwd_dispatch_bf16_d128(a, v, s) : fwd_dispatch_bf16_d256(a, v, s);
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
+}
+
+uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d) {
+  if (bh <= 0 || sq <= 0 || sk <= kBwdFusedMaxKeys / 2 || sk > kBwdFusedMaxKeys || d != 64) return 0;
+  return (uint64_t)bwd_fused_workspace_need(bh, sq);
 }
 
 int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
@@ -319,7 +346,7 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   if (!(a.drop_scale > 0.f)) return FMHA_E_ARG;
   a.drop = make_drop_ctx(p->seed, p->offset, p->drop_kind == FMHA_DROP_PHILOX ? p->p_drop : 0.f, p->sq, p->sk);
   a.flags = p->flags;
-  if (!env_int("FMHA_MASK_TRIM", 1)) a.flags |= kBwdFlagNoTrim;
+  if (!overrides().mask_trim) a.flags |= kBwdFlagNoTrim;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
   int mrc;
@@ -339,12 +366,24 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
   v.causal = p->causal != 0;
   v.drop = p->drop_kind == FMHA_DROP_PHILOX ? 1 : 0;
-  v.pair = env_int("FMHA_BWD_PAIR", -1); // tuning / test override: 0 or 1
+  v.pair = overrides().bwd_pair; // tuning / test override: 0 or 1
   // Heads whose Q, K, V and dO fit in LDS together (up to 256 queries and keys) take one launch instead of two.
-  int short_rows = env_int("FMHA_BWD_SHORT", 1); // 0: never; 1: up to 256 rows; other values: that many rows
+  int short_rows = overrides().bwd_short; // 0: never; 1: up to 256 rows; other values: that many rows
   if (short_rows == 1) short_rows = 256;
   v.short_seq = p->d == 64 && p->sq <= short_rows && p->sk <= short_rows && p->sq <= 256 && p->sk <= 256 &&
                 v.mask != kMaskFull;
+  // The one-pass kernel (one workgroup per head of up to 512 keys, no causal mask, no full mask tensor; beyond 256
+  // keys it needs the caller's workspace) runs only where the caller asks for it: it measures level with the
+  // two-kernel path at best.
+  a.ws = (float *)p->workspace;
+  {
+    const bool asked = (p->flags & FMHA_FLAG_BWD_ONE_PASS) != 0 || overrides().bwd_fused == 1;
+    const bool can = p->d == 64 && !v.short_seq && !v.causal && v.mask != kMaskFull && p->sk <= kBwdFusedMaxKeys &&
+                     (p->sk <= kBwdFusedMaxKeys / 2 ||
+                      (p->workspace && ((uintptr_t)p->workspace & 15u) == 0 &&
+                       p->workspace_bytes >= bwd_fused_workspace_need(p->bh, p->sq)));
+    v.fused = asked && can;
+  }
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;
   if (strided) {

@@ -391,3 +391,72 @@ def test_trailing_hard_masked_keys_are_skipped_exactly(bh, sq, sk, d, dtype, kin
         ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), dout=f32(do), want=("dq", "dk", "dv"), **okw)
         for name, t in zip(("dq", "dk", "dv"), grads):
             assert rel_to_max(f32(t.cpu()), ref[name], floor=1e-3) <= TOL[dtype], name
+
+
+# The one-pass kernel (FMHA_FLAG_BWD_ONE_PASS: one workgroup per head of up to 512 keys forms scores, exponentials
+# and dropout decisions once and produces dQ, dK and dV; beyond 256 keys the second half of the keys adds to fp32
+# partial sums of dQ in the caller's workspace).  Same bar as the two-kernel path.
+ONE_PASS = [
+    # bh, sq, sk, dtype, mask, p_drop
+    (4, 512, 512, "fp16", "pad", 0.1),     # headline train-step shape (few heads): two key chunks
+    (4, 512, 512, "fp16", None, 0.0),
+    (3, 300, 300, "fp16", None, 0.1),      # ragged tiles and a partly filled second chunk
+    (3, 100, 477, "fp16", "pad", 0.1),
+    (2, 700, 260, "fp16", "pad", 0.0),     # four keys in the second chunk
+    (2, 64, 512, "bf16", "pad", 0.1),
+    (2, 333, 257, "bf16", None, 0.0),
+    (5, 1, 300, "fp16", None, 0.0),        # one query
+    (6, 512, 512, "fp16", "tail", 0.1),    # hard-masked tails of every length: chunks and key blocks left out
+    (6, 384, 512, "fp16", "holes", 0.1),
+    (4, 512, 512, "fp16", "kvlen", 0.1),   # valid key counts 100, 256, 257, 512
+    (3, 320, 256, "fp16", "pad", 0.1),     # one chunk: no workspace involved
+]
+
+
+@pytest.mark.parametrize("bh,sq,sk,dtype,mask,p", ONE_PASS)
+def test_one_pass_backward_matches_oracle(bh, sq, sk, dtype, mask, p):
+    q, k, v, do = make_qkv(bh, sq, sk, 64, seed=bh + sk, dtype=dtype, with_dout=True)
+    m = kvl = None
+    if mask == "pad":
+        m = pad_mask(bh // 2 if bh % 2 == 0 else bh, sk, sk // 2, sk)
+    elif mask in ("tail", "holes"):
+        m = tail_mask(mask, bh, sk, 5)
+    elif mask == "kvlen":
+        kvl = torch.tensor([100, 256, 257, 512][:bh], dtype=torch.int32)
+    if m is not None:
+        m = m.to(TDT[dtype])
+    kw, okw = {}, {}
+    if p > 0:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=99, offset=12)
+        okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=99, offset=12)
+    qc, kc, vc, mc = q.cuda(), k.cuda(), v.cuda(), (None if m is None else m.cuda())
+    kvc = None if kvl is None else kvl.cuda()
+    o, lse, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, kv_len=kvc, **kw)
+    dq, dk, dv = capi.bwd(do.cuda(), qc, kc, vc, o, lse, mask=mc, kv_len=kvc, flags=capi.FLAG_BWD_ONE_PASS, **kw)
+    two = capi.bwd(do.cuda(), qc, kc, vc, o, lse, mask=mc, kv_len=kvc, **kw)
+    torch.cuda.synchronize()
+    om = None if m is None else f32(m)
+    if kvl is not None:
+        om = np.zeros((bh, 1, sk), np.float32)
+        for i in range(bh):
+            om[i, 0, int(kvl[i]):] = -np.inf
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=om, dout=f32(do), want=("dq", "dk", "dv"), **okw)
+    for name, t in zip(("dq", "dk", "dv"), (dq, dk, dv)):
+        assert rel_to_max(f32(t.cpu()), ref[name], floor=1e-3) <= TOL[dtype], name
+    # (a different kernel from the default one, not the same launch twice: dQ is summed in another order)
+    if sk > 32 and sq > 1:
+        assert not torch.equal(dq, two[0])
+
+
+def test_one_pass_backward_without_workspace_takes_the_default_path():
+    """Beyond 256 keys the one-pass kernel needs the workspace; without one the flag changes nothing."""
+    q, k, v, do = make_qkv(3, 300, 400, 64, seed=3, with_dout=True)
+    qc, kc, vc, dc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o, lse, _, _ = capi.fwd(qc, kc, vc, want_lse=True)
+    a = capi.bwd(dc, qc, kc, vc, o, lse, flags=capi.FLAG_BWD_ONE_PASS, workspace=None)
+    b = capi.bwd(dc, qc, kc, vc, o, lse)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    assert capi.lib().fmha_bwd_workspace_bytes(3, 300, 400, 64) == 3 * 5 * 16384
+    assert capi.lib().fmha_bwd_workspace_bytes(3, 300, 256, 64) == 0
+    assert capi.lib().fmha_bwd_workspace_bytes(3, 300, 400, 128) == 0
