@@ -68,7 +68,8 @@ enum {
   FMHA_E_ALIGN = -4,       /* q/k/v/o/gradient base pointer not 16-byte aligned */
   FMHA_E_ARG = -5,         /* scale / p_drop / mask description out of range */
   FMHA_E_UNSUPPORTED = -6, /* combination not built (see fmha_strerror) */
-  FMHA_E_LAUNCH = -7       /* the HIP runtime refused the launch */
+  FMHA_E_LAUNCH = -7,      /* the HIP runtime refused the launch */
+  FMHA_E_SCRATCH = -8      /* fmha_bwd_launch_noalloc: the sizes exceed the library's own scratch memory */
 };
 
 /*
@@ -199,6 +200,20 @@ typedef struct fmha_bwd_params {
 } fmha_bwd_params;
 
 int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);
+
+/*
+ * The backward for callers that cannot allocate (no counterpart in the reference): code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same as fmha_bwd_launch, except that
+ * `delta` and `workspace` of the struct are ignored: both come out of an array of
+ * 4 * fmha_bwd_noalloc_max_rows() bytes (8 MiB) that the library holds in the memory of every GPU it
+ * runs on until the process ends.  bh * sq beyond fmha_bwd_noalloc_max_rows() is refused
+ * (FMHA_E_SCRATCH).  The call allocates nothing and synchronises nothing.  All calls on one GPU share
+ * that GPU's array: calls that may overlap there (different streams or threads) race on it; serialise
+ * them or use fmha_bwd_launch with buffers of the caller's own.  Results are bit-identical to
+ * fmha_bwd_launch's.
+ */
+int fmha_bwd_launch_noalloc(const fmha_bwd_params *p, void *hip_stream);
+uint64_t fmha_bwd_noalloc_max_rows(void);
 
 /* Workspace the backward can make use of for these sizes (0: none). */
 uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d);

@@ -17,7 +17,8 @@ FLAG_BWD_ONE_PASS = 2  # bwd(flags=...): the one-pass backward kernel where it a
 DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
-           "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides")
+           "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides",
+           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
 _ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
@@ -104,6 +105,10 @@ def lib():
         L.fmha_fwd_launch.restype = C.c_int
         L.fmha_bwd_launch.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         L.fmha_bwd_launch.restype = C.c_int
+        L.fmha_bwd_launch_noalloc.argtypes = [C.POINTER(BwdParams), C.c_void_p]
+        L.fmha_bwd_launch_noalloc.restype = C.c_int
+        L.fmha_bwd_noalloc_max_rows.argtypes = []
+        L.fmha_bwd_noalloc_max_rows.restype = C.c_uint64
         L.fmha_bwd_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
         L.fmha_bwd_workspace_bytes.restype = C.c_uint64
         L.fmha_philox_keep_mask.argtypes = [C.c_uint64, C.c_uint64, C.c_float, C.c_int32, C.c_int32,
@@ -266,12 +271,13 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
 
 def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False,
         scale=None, drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
-        flags=0, delta=None, grads=None, kv_len=None, workspace=True):
+        flags=0, delta=None, grads=None, kv_len=None, workspace=True, noalloc=False):
     """Launch the backward on the current stream.  Returns (dq, dk, dv).  kv_len and the tensor
     layouts as in fwd(); each gradient comes back in its input's dimension order.
 
     workspace: True allocates the scratch that fmha_bwd_workspace_bytes() asks for (if any), a uint8
-    device tensor is passed on as it is, None / False passes none (the two-kernel path beyond 256 keys)."""
+    device tensor is passed on as it is, None / False passes none (the two-kernel path beyond 256 keys).
+    noalloc: call fmha_bwd_launch_noalloc (delta and workspace out of the library's own scratch memory)."""
     import torch
     bh, sq, d, heads, qs = _rows(q, "q")
     _, sk, _, hk, ks = _rows(k, "k")
@@ -285,7 +291,7 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     for t in (q, k, v, o, dout):
         if not (t.is_cuda and t.dtype == q.dtype):
             raise FmhaError(-5, "q/k/v/o/dout must be device tensors of one dtype")
-    if delta is None:
+    if delta is None and not noalloc:
         delta = torch.empty((bh, sq), dtype=torch.float32, device=q.device)
     if not lse.is_contiguous():
         raise FmhaError(-5, "lse must be contiguous")
@@ -293,7 +299,7 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     _set_rows(P, heads, q=(0, heads, qs), k=(0, hk, ks), v=(0, hv, vs), o=(0, ho, os_), do=(0, hd, ds_),
               dq=(0,) + _rows(dq, "dq")[3:], dk=(0,) + _rows(dk, "dk")[3:], dv=(0,) + _rows(dv, "dv")[3:])
     P.q, P.k, P.v, P.o, P.dout = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), dout.data_ptr()
-    P.lse, P.delta = lse.data_ptr(), delta.data_ptr()
+    P.lse, P.delta = lse.data_ptr(), (None if noalloc else delta.data_ptr())
     P.dq, P.dk, P.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     P.bh, P.sq, P.sk, P.d = bh, sq, sk, d
     P.scale = float(scale) if scale is not None else d ** -0.5
@@ -313,6 +319,10 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     P.seed, P.offset = seed, offset
     P.flags = flags
     _set_kv_len(P, kv_len, bh)
+    if noalloc:
+        _sync_env()
+        check(lib().fmha_bwd_launch_noalloc(C.byref(P), _stream_ptr()))
+        return dq, dk, dv
     if workspace is True:
         need = lib().fmha_bwd_workspace_bytes(bh, sq, sk, d)
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device) if need else None

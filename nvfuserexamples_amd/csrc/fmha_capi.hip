@@ -7,6 +7,7 @@
 #include <cstddef>
 #include <cstring>
 #include <cstdlib>
+#include <mutex>
 
 using namespace fmha;
 
@@ -94,6 +95,7 @@ const char *fmha_strerror(int code) {
   case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
   case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart; head dim 256 takes folded tensors only and, in the forward, no valid key counts)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
+  case FMHA_E_SCRATCH: return "fmha_bwd_launch_noalloc: bh * sq exceeds fmha_bwd_noalloc_max_rows() (the library's own scratch holds one float per query row); use fmha_bwd_launch with caller-provided delta";
   default: return "unknown error code";
   }
 }
@@ -293,12 +295,69 @@ uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d)
   return (uint64_t)bwd_fused_workspace_need(bh, sq);
 }
 
-int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
+} // extern "C"
+
+// The library's own scratch memory, for fmha_bwd_launch_noalloc: delta (bh*sq floats) first, what is left
+// serves as the one-pass kernel's workspace where that fits.  Every GPU holds its own copy of the array; its
+// device address is looked up once per device (the array's name is only a host-side handle).
+namespace {
+constexpr size_t kScratchBytes = 8u << 20;
+constexpr int kMaxDevices = 64;
+} // namespace
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+namespace {
+void *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device, or nullptr.
+void *scratch_on_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_scratch);
+} // namespace
+
+extern "C" {
+
+int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) { return bwd_launch_impl(caller, hip_stream, false); }
+
+int fmha_bwd_launch_noalloc(const fmha_bwd_params *caller, void *hip_stream) { return bwd_launch_impl(caller, hip_stream, true); }
+
+uint64_t fmha_bwd_noalloc_max_rows(void) { return kScratchBytes / sizeof(float); }
+
+} // extern "C"
+
+namespace {
+
+int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_scratch) {
   if (!caller) return FMHA_E_NULL;
   if (caller->struct_bytes < offsetof(fmha_bwd_params, kv_len)) return FMHA_E_ARG;
   fmha_bwd_params local;
   std::memset(&local, 0, sizeof local);
   std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
+  if (own_scratch) {
+    // delta and the workspace come out of the library's array; what the caller put there is not looked at
+    local.delta = nullptr;
+    local.workspace = nullptr;
+    local.workspace_bytes = 0;
+    if (local.bh <= 0 || local.sq <= 0) return FMHA_E_SHAPE;
+    const uint64_t rows = (uint64_t)local.bh * (uint64_t)local.sq;
+    if (rows * sizeof(float) > kScratchBytes) return FMHA_E_SCRATCH;
+    unsigned char *base = (unsigned char *)scratch_on_current_device();
+    if (!base) return FMHA_E_LAUNCH;
+    local.delta = (float *)base;
+    const size_t used = (size_t)((rows * sizeof(float) + 255u) & ~(uint64_t)255u);
+    local.workspace = base + used;
+    local.workspace_bytes = kScratchBytes - used;
+  }
   const fmha_bwd_params *p = &local;
   if (!p->q || !p->k || !p->v || !p->o || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk || !p->dv)
     return FMHA_E_NULL;
@@ -398,4 +457,4 @@ int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) {
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 
-} // extern "C"
+} // namespace
