@@ -61,7 +61,7 @@ def fwd_params(capi, t, train=False):
     P.dtype, P.scale = capi.F16, 0.125
     if train:
         P.lse = t["lse"].data_ptr()
-        P.drop_kind, P.p_drop, P.drop_scale = capi.DROP_PHILOX, 0.1, 1.0 / 0.9
+        P.drop_kind, P.p_drop, P.drop_scale = capi.DROP_PHILOX, 0.1, 0.0  # 0: the mean-preserving factor
         P.seed, P.offset = 0x1234, 0
     return P
 
@@ -74,7 +74,7 @@ def bwd_params(capi, t):
     P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = H, S, 0
     P.bh, P.sq, P.sk, P.d = B * H, S, S, D
     P.dtype, P.scale = capi.F16, 0.125
-    P.drop_kind, P.p_drop, P.drop_scale = capi.DROP_PHILOX, 0.1, 1.0 / 0.9
+    P.drop_kind, P.p_drop, P.drop_scale = capi.DROP_PHILOX, 0.1, 0.0  # 0: the mean-preserving factor
     P.seed, P.offset = 0x1234, 0
     return P
 
@@ -211,7 +211,7 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
             P.dtype, P.scale = capi.F16, 0.125
             P.mask, P.mask_kind = t["mask"].data_ptr(), capi.MASK_ADDITIVE
             P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = bh // bb, s, 0
-            P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, 0.1, 1.0 / 0.9, 0x1234, 0
+            P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, 0.1, 0.0, 0x1234, 0
         Bp.dout, Bp.delta, Bp.dq, Bp.dk, Bp.dv = (t[n].data_ptr() for n in ("dout", "delta", "dq", "dk", "dv"))
         tkeep.append(t)
         tsteps.append((F, Bp))

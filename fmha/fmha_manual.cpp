@@ -277,7 +277,7 @@ void set_mask_and_dropout(P &p, MaskLayout &m, const c10::optional<at::Tensor> &
   if (p_drop > 0.0) {
     p.drop_kind = FMHA_DROP_PHILOX;
     p.p_drop = static_cast<float>(p_drop);
-    p.drop_scale = static_cast<float>(1.0 / (1.0 - p_drop));
+    p.drop_scale = fmha_drop_scale(static_cast<float>(p_drop)); // keeps the mean at the realised keep probability
     p.seed = static_cast<uint64_t>(seed);
     p.offset = static_cast<uint64_t>(offset);
   }

@@ -102,8 +102,10 @@ typedef struct fmha_fwd_params {
 
   int32_t drop_kind;
   const void *drop_mask; /* FMHA_DROP_TENSOR: [bh,sq,sk], element type = dtype */
-  float p_drop;          /* FMHA_DROP_PHILOX: drop probability in [0,1) */
-  float drop_scale;      /* factor on kept probabilities: 2 on the legacy ops, 1/(1-p) otherwise */
+  float p_drop;          /* FMHA_DROP_PHILOX: drop probability in [0,1), realised as round(256 p) / 256;
+                          * below 1/512 nothing is dropped and the call is one without dropout */
+  float drop_scale;      /* factor on kept probabilities: 2 on the legacy ops; with FMHA_DROP_PHILOX, 0 selects
+                          * fmha_drop_scale(p_drop), which keeps the mean */
   uint64_t seed, offset; /* FMHA_DROP_PHILOX */
 
   /* optional [bh,sq,sk] outputs of the save-intermediates op (fmha_manual.cpp:891-897):
@@ -230,6 +232,10 @@ int fmha_philox_keep_mask(uint64_t seed, uint64_t offset, float p_drop, int32_t 
 
 /* 8-bit threshold the keep rule compares against: keep iff random_byte >= threshold. */
 uint32_t fmha_drop_threshold(float p_drop);
+
+/* 256 / (256 - threshold): the reciprocal of the keep probability that the 8-bit threshold realises
+ * (230/256 at p_drop = 0.1, not 0.9), so that E[dropout(x)] = x exactly; 1 when nothing is dropped. */
+float fmha_drop_scale(float p_drop);
 
 /* Static description of a return code. */
 const char *fmha_strerror(int code);

@@ -18,7 +18,7 @@ DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
            "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides",
-           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows")
+           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
 _ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
@@ -116,6 +116,8 @@ def lib():
         L.fmha_philox_keep_mask.restype = C.c_int
         L.fmha_drop_threshold.argtypes = [C.c_float]
         L.fmha_drop_threshold.restype = C.c_uint32
+        L.fmha_drop_scale.argtypes = [C.c_float]
+        L.fmha_drop_scale.restype = C.c_float
         L.fmha_strerror.argtypes = [C.c_int]
         L.fmha_strerror.restype = C.c_char_p
         L.fmha_version.restype = C.c_char_p
@@ -253,8 +255,8 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
             raise FmhaError(-5, "drop_mask must be a contiguous tensor of q's dtype")
         P.drop_mask = drop_mask.data_ptr()
     P.p_drop = p_drop
-    if drop_scale is None:
-        drop_scale = 1.0 / (1.0 - p_drop) if drop_kind == DROP_PHILOX else 1.0
+    if drop_scale is None:   # Philox: the factor that keeps the mean at the realised keep probability
+        drop_scale = lib().fmha_drop_scale(p_drop) if drop_kind == DROP_PHILOX else 1.0
     P.drop_scale = drop_scale
     P.seed, P.offset = seed, offset
     sm = dr = None
@@ -313,8 +315,8 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     if drop_kind == DROP_TENSOR:
         P.drop_mask = drop_mask.data_ptr()
     P.p_drop = p_drop
-    if drop_scale is None:
-        drop_scale = 1.0 / (1.0 - p_drop) if drop_kind == DROP_PHILOX else 1.0
+    if drop_scale is None:   # Philox: the factor that keeps the mean at the realised keep probability
+        drop_scale = lib().fmha_drop_scale(p_drop) if drop_kind == DROP_PHILOX else 1.0
     P.drop_scale = drop_scale
     P.seed, P.offset = seed, offset
     P.flags = flags

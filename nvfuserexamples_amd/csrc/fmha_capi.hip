@@ -85,6 +85,11 @@ uint32_t fmha_drop_threshold(float p_drop) {
   return (uint32_t)t;
 }
 
+float fmha_drop_scale(float p_drop) {
+  const uint32_t thr = fmha_drop_threshold(p_drop);
+  return (float)(256.0 / (256.0 - (double)thr));
+}
+
 const char *fmha_strerror(int code) {
   switch (code) {
   case FMHA_OK: return "ok";
@@ -172,6 +177,11 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_TENSOR && !p->drop_mask) return FMHA_E_NULL;
   if (p->drop_kind != FMHA_DROP_NONE && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
+  if (p->drop_kind == FMHA_DROP_PHILOX) {
+    // a threshold of 0 drops nothing: no dropout at all (and no factor on the probabilities)
+    if (fmha_drop_threshold(p->p_drop) == 0) local.drop_kind = FMHA_DROP_NONE;
+    else if (p->drop_scale == 0.f) local.drop_scale = fmha_drop_scale(p->p_drop);
+  }
   const bool saving = p->save_softmax || p->save_dropout;
   if (saving && (p->drop_kind == FMHA_DROP_PHILOX || p->causal)) return FMHA_E_UNSUPPORTED;
   if (p->drop_kind == FMHA_DROP_TENSOR && p->causal) return FMHA_E_UNSUPPORTED;
@@ -376,6 +386,10 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   }
   if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_PHILOX && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
+  if (p->drop_kind == FMHA_DROP_PHILOX) {
+    if (fmha_drop_threshold(p->p_drop) == 0) local.drop_kind = FMHA_DROP_NONE;
+    else if (p->drop_scale == 0.f) local.drop_scale = fmha_drop_scale(p->p_drop);
+  }
   if (p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED; // backward regenerates Philox decisions only
   if (p->kv_len && (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u))) return FMHA_E_ARG;
 

@@ -40,6 +40,7 @@ class _Params(C.Structure):
         ("round_p", C.c_int32), ("round_o", C.c_int32),
         ("o", C.c_void_p), ("lse", C.c_void_p), ("softmax", C.c_void_p), ("dropout", C.c_void_p),
         ("dout", C.c_void_p), ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+        ("bh_offset", C.c_int64),
     ]
 
 
@@ -58,6 +59,8 @@ def lib():
                                                C.c_int64, C.c_int64, C.c_void_p]
         _lib.fmha_oracle_drop_threshold.argtypes = [C.c_float]
         _lib.fmha_oracle_drop_threshold.restype = C.c_uint32
+        _lib.fmha_oracle_drop_scale.argtypes = [C.c_float]
+        _lib.fmha_oracle_drop_scale.restype = C.c_float
         _lib.fmha_oracle_round.argtypes = [C.c_float, C.c_int]
         _lib.fmha_oracle_round.restype = C.c_float
     return _lib
@@ -87,6 +90,11 @@ def drop_threshold(p):
     return int(lib().fmha_oracle_drop_threshold(float(p)))
 
 
+def drop_scale(p):
+    """Factor on kept values: the reciprocal of the keep probability the 8-bit threshold realises."""
+    return float(lib().fmha_oracle_drop_scale(float(p)))
+
+
 def keep_mask(seed, offset, p, bh, sq, sk):
     """uint8 [bh,sq,sk] array of 0/1: the dropout keep decisions for (seed, offset)."""
     out = np.zeros((bh, sq, sk), dtype=np.uint8)
@@ -110,9 +118,12 @@ def _mask_layout(mask, bh, sq, sk):
 
 
 def attention(q, k, v, mask=None, mask_kind="additive", mask_neg=-10000.0, causal=False,
-              scale=None, drop_mask=None, drop_scale=1.0, p_drop=0.0, seed=0, offset=0,
-              philox=False, round_p=None, round_o=None, dout=None, want=("o",)):
+              scale=None, drop_mask=None, drop_scale=None, p_drop=0.0, seed=0, offset=0,
+              philox=False, round_p=None, round_o=None, dout=None, want=("o",), bh_offset=0):
     """Forward (and, when ``dout`` is given, backward) of the attention path on the CPU.
+
+    ``drop_scale=None``: 1 with a dropout tensor, the mean-preserving factor ``drop_scale(p_drop)`` with Philox.
+    ``bh_offset``: the tensors are heads ``bh_offset ..`` of a larger problem (Philox decisions follow).
 
     Returns a dict with the requested entries of
     ``o, lse, softmax, dropout, dq, dk, dv`` as float32 numpy arrays.
@@ -141,7 +152,12 @@ def attention(q, k, v, mask=None, mask_kind="additive", mask_neg=-10000.0, causa
         P.drop_kind, P.drop_mask = 1, _ptr(dm)
     elif philox:
         P.drop_kind = 2
+        if drop_scale is None:
+            drop_scale = globals()["drop_scale"](p_drop)
+    if drop_scale is None:
+        drop_scale = 1.0
     P.p_drop, P.drop_scale = float(p_drop), float(drop_scale)
+    P.bh_offset = int(bh_offset)
     P.seed, P.offset = int(seed), int(offset)
     P.round_p, P.round_o = ROUND[round_p], ROUND[round_o]
     out = {}

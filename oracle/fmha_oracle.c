@@ -92,12 +92,20 @@ void fmha_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uin
  *   ctr  = (offset_lo, offset_hi, blk_lo, blk_hi),
  *          blk = (bh * ceil(Sq/4) + q/4) * ceil(Sk/4) + k/4
  *   byte = (out[q%4] >> 8*(k%4)) & 0xff ;  keep iff byte >= thr,  thr = round(p*256)
+ * Kept values are scaled by 256 / (256 - thr), the reciprocal of the keep probability that the 8-bit
+ * threshold realises (not of the nominal 1 - p), so that dropout preserves the mean exactly;
+ * thr == 0 keeps everything (scale 1).
  */
 uint32_t fmha_oracle_drop_threshold(float p) {
   double t = floor((double)p * 256.0 + 0.5);
   if (t < 0) t = 0;
   if (t > 255) t = 255;
   return (uint32_t)t;
+}
+
+float fmha_oracle_drop_scale(float p) {
+  uint32_t thr = fmha_oracle_drop_threshold(p);
+  return (float)(256.0 / (256.0 - (double)thr));
 }
 
 int fmha_oracle_keep(uint64_t seed, uint64_t offset, uint32_t thr, int64_t bh, int64_t q,
@@ -150,6 +158,9 @@ typedef struct {
   /* backward */
   const float *dout; /* [bh,sq,d] */
   float *dq, *dk, *dv;
+  /* head b of these tensors is head bh_offset + b of the full problem as far as the Philox block
+   * index is concerned (a sample of the heads of a larger batch keeps its dropout decisions) */
+  int64_t bh_offset;
 } fmha_oracle_params;
 
 static double score_at(const fmha_oracle_params *p, int64_t b, int64_t i, int64_t j) {
@@ -171,7 +182,7 @@ static double drop_factor(const fmha_oracle_params *p, uint32_t thr, int64_t b, 
   if (p->drop_kind == 1)
     return (double)p->drop_mask[(b * p->sq + i) * p->sk + j] * (double)p->drop_scale;
   if (p->drop_kind == 2)
-    return fmha_oracle_keep(p->seed, p->offset, thr, b, i, j, p->sq, p->sk)
+    return fmha_oracle_keep(p->seed, p->offset, thr, p->bh_offset + b, i, j, p->sq, p->sk)
                ? (double)p->drop_scale : 0.0;
   return 1.0;
 }

@@ -20,7 +20,7 @@ def main():
     q, k, v, do = make_qkv(bh, sq, sk, d, seed=42, with_dout=True)
     m = pad_mask(1, sk, sk // 2, sk, seed=42).half()
     seed, offset, p = 0x1234, 7, 0.1
-    kw = dict(mask=m.float().numpy(), philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=seed, offset=offset)
+    kw = dict(mask=m.float().numpy(), philox=True, p_drop=p, seed=seed, offset=offset)
     r = oracle.attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), dout=do.float().numpy(),
                          want=("o", "lse", "dq", "dk", "dv"), **kw)
     np.savez_compressed(os.path.join(HERE, "fwd_small.npz"),

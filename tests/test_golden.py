@@ -12,7 +12,7 @@ def test_forward_backward_fixture_matches_oracle():
     f = np.load(os.path.join(HERE, "fwd_small.npz"))
     p = float(f["p_drop"])
     r = oracle.attention(f["q"].astype(np.float32), f["k"].astype(np.float32), f["v"].astype(np.float32),
-                         mask=f["mask"].astype(np.float32), philox=True, p_drop=p, drop_scale=1 / (1 - p),
+                         mask=f["mask"].astype(np.float32), philox=True, p_drop=p,
                          seed=int(f["seed"]), offset=int(f["offset"]), dout=f["dout"].astype(np.float32),
                          want=("o", "lse", "dq", "dk", "dv"))
     for n, a in r.items():

@@ -31,7 +31,7 @@ def test_autograd_wrapper_matches_eager_autograd(causal, p):
         s_ = s_.masked_fill(~torch.ones(s, s, dtype=torch.bool, device="cuda").tril(), float("-inf"))
     pr = torch.softmax(s_, -1)
     if keep is not None:
-        pr = pr * keep / (1 - p)
+        pr = pr * keep * oracle.drop_scale(p)   # the mean-preserving factor at the realised keep probability
     oe = pr.matmul(ve)
     (oe * do.float()).sum().backward()
     assert (o.float() - oe).abs().max().item() <= 2e-3

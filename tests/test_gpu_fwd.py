@@ -121,7 +121,7 @@ def test_philox_dropout_forward_and_mask_bit_exact(bh, sq, sk, d, causal):
     seed, offset, p = 0xfeedbeefcafe, (1 << 33) + 5, 0.1
     o, lse, _, _ = _run(q, k, v, causal=causal, drop_kind=capi.DROP_PHILOX, p_drop=p, seed=seed, offset=offset,
                         want_lse=True)
-    ref = oracle.attention(f32(q), f32(k), f32(v), causal=causal, philox=True, p_drop=p, drop_scale=1 / (1 - p),
+    ref = oracle.attention(f32(q), f32(k), f32(v), causal=causal, philox=True, p_drop=p,
                            seed=seed, offset=offset, want=("o", "lse"))
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= 2e-3
     assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= 1e-3
@@ -131,7 +131,7 @@ def test_philox_dropout_forward_and_mask_bit_exact(bh, sq, sk, d, causal):
     # and the fused kernel used exactly those decisions: feeding them back as an explicit
     # dropout tensor reproduces its output to rounding
     o2, _, _, _ = _run(q, k, v, drop_kind=capi.DROP_TENSOR, drop_mask=torch.from_numpy(km).to(q.dtype).cuda(),
-                       drop_scale=1 / (1 - p)) if not causal else (o, None, None, None)
+                       drop_scale=capi.lib().fmha_drop_scale(p)) if not causal else (o, None, None, None)
     assert np.abs(f32(o2.cpu()) - f32(o.cpu())).max() <= 1e-3
 
 
@@ -463,3 +463,35 @@ def test_skipped_key_tiles_are_never_read(bh, heads):
     assert not torch.isnan(o).any()
     o_all = _run(q, k, v, mask=m.half().cuda(), flags=capi.FLAG_NO_MASK_TRIM)[0]
     assert torch.isnan(o_all).view(b, -1).any(1).all()
+
+
+def test_dropout_keeps_the_mean():
+    """Kept probabilities are scaled by 256 / (256 - threshold), the reciprocal of the keep probability the
+    8-bit threshold realises, so E[O] is the undropped O.  With q = 0 (uniform attention) and v = 1,
+    O_i = scale * (kept keys of row i) / sk: the mean over 32 x 512 rows of 512 keys is 1 within 3 sigma
+    of 8.4 million keep decisions -- the nominal factor 1 / (1 - p) would sit 15 sigma low at p = 0.1."""
+    bh, s, d, p = 32, 512, 64, 0.1
+    q = torch.zeros(bh, s, d, dtype=torch.float16, device="cuda")
+    k = torch.randn(bh, s, d, device="cuda").half()
+    v = torch.ones(bh, s, d, dtype=torch.float16, device="cuda")
+    o, _, _, _ = _run(q, k, v, drop_kind=capi.DROP_PHILOX, p_drop=p, seed=77, offset=5)
+    thr = capi.lib().fmha_drop_threshold(p)
+    scale = capi.lib().fmha_drop_scale(p)
+    assert thr == 26 and scale == pytest.approx(256 / 230, rel=1e-6)
+    pk = (256 - thr) / 256
+    sigma = scale * np.sqrt(pk * (1 - pk) / (bh * s * s))
+    mean = o.float()[:, :, 0].double().mean().item()
+    assert abs(mean - 1.0) <= 3 * sigma + 2e-5           # (+ the fp16 rounding of O near 1, averaged over the rows)
+    assert abs(mean * (1 / (1 - p)) / scale - 1.0) > 6 * sigma   # what the nominal factor would have given
+
+
+def test_drop_probability_below_one_step_is_no_dropout():
+    """p < 1/512 rounds to a threshold of 0: nothing is dropped and nothing is scaled -- the call is the
+    one without dropout, bit for bit, forward and backward."""
+    q, k, v, do = (t.cuda() for t in make_qkv(4, 200, 300, 64, seed=8, with_dout=True))
+    o0, l0, _, _ = _run(q, k, v, want_lse=True)
+    o1, l1, _, _ = _run(q, k, v, want_lse=True, drop_kind=capi.DROP_PHILOX, p_drop=0.0015, seed=3)
+    assert torch.equal(o0, o1) and torch.equal(l0, l1)
+    g0 = capi.bwd(do, q, k, v, o0, l0)
+    g1 = capi.bwd(do, q, k, v, o0, l0, drop_kind=capi.DROP_PHILOX, p_drop=0.0015, seed=3)
+    assert all(torch.equal(a, b) for a, b in zip(g0, g1))

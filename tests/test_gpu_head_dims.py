@@ -47,7 +47,7 @@ def test_operators_pad_other_head_dims(bh, sq, sk, d, dtype, causal, p, masked):
     assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
     okw = dict(causal=causal)
     if p:
-        okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=9, offset=4)
+        okw.update(philox=True, p_drop=p, seed=9, offset=4)
     ref = oracle.attention(f32(q), f32(k), f32(v), mask=None if m is None else f32(m), dout=f32(do),
                            want=("o", "lse", "dq", "dk", "dv"), **okw)
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= O_TOL[dtype]

@@ -57,7 +57,7 @@ def test_strided_layouts_match_oracle_and_folded_path(b, h, sq, sk, d, dtype, ca
     kw, okw = dict(causal=causal), dict(causal=causal)
     if p:
         kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=11, offset=5)
-        okw.update(philox=True, p_drop=p, drop_scale=1 / (1 - p), seed=11, offset=5)
+        okw.update(philox=True, p_drop=p, seed=11, offset=5)
     m = None
     if masked:
         m = pad_mask(b, sk, sk // 2, sk).to(TDT[dtype])

@@ -1,0 +1,154 @@
+"""Seeded randomized parity sweep: forward and backward through the C ABI against the CPU oracle over
+400 small problems that mix head dims, element types, ragged sizes, mask kinds (padding with -10000 or
+-inf tails, holes, per-key, full tensors), causal masking, Philox dropout, valid key counts and strided
+layouts.  Bars as everywhere else: |O - oracle| <= 2e-3 (fp16) / 2e-2 (bf16) (scaled up where |O|
+exceeds 2), gradients within 1e-2 / 3e-2 of the largest oracle entry, LSE within 5e-3 + 2^-8 |LSE|,
+-inf rows in the same places; where a per-key mask is involved, skipping the hard-masked tail must not
+change a bit.
+
+Gradients that are exactly zero.  When every query of a problem sees exactly one key (sk = 1, a valid
+length of 1, a causal first row alone), softmax is the constant 1 and dQ = dK = 0.  The kernels then
+compute dS_i = P_i (dP_i - delta_i) with dP_i = Z (dO_i . V_k) and delta_i = dO_i . O_i, where O_i is the
+forward's output ROUNDED to the element type: O_i = round(Z V_k).  The two terms differ by
+dO_i . (Z V_k - round(Z V_k)), at most u * A_i with A_i = sum_d |dO_id O_id| and u the unit roundoff of
+the element type (2^-11 fp16, 2^-8 bf16); without dropout Z = 1, round(V_k) = V_k and what is left is the
+2^-2p relative error of the hi + lo split that carries delta and LSE into the matrix pipe, far below
+that.  Hence |dQ_id| <= scale * u * A_i * |K_kd| and, the signs of the row errors being independent,
+|dK_kd| is of the order scale * u * sqrt(sum_i A_i^2) * max|Q|.  Such all-zero gradients are judged on
+ABSOLUTE error against 4 * scale * u * sqrt(sum_i A_i^2) * max(|Q|, |K|) instead of relative to a
+maximum that does not exist."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nvfuserexamples_amd import capi
+from conftest import make_qkv, f32, rel_to_max
+
+pytestmark = pytest.mark.gpu
+
+TDT = {"fp16": torch.float16, "bf16": torch.bfloat16}
+UNIT = {"fp16": 2.0 ** -11, "bf16": 2.0 ** -8}
+
+
+def _case(it, rng, forced=None):
+    c = forced or dict(
+        d=rng.choice([64, 64, 64, 128, 256]), dtype=rng.choice(["fp16", "fp16", "bf16"]),
+        b=rng.choice([1, 2, 3]), h=rng.choice([1, 2, 4]),
+        sq=rng.choice([1, 7, 31, 32, 33, 64, 65, 100, 127, 128, 129, 191, 200, 255, 256, 257, 300, 384, 520]),
+        sk=rng.choice([1, 5, 8, 31, 32, 33, 40, 64, 65, 96, 127, 128, 129, 192, 200, 250, 256, 257, 300, 333, 512, 700]),
+        causal=rng.random() < 0.3, p=rng.choice([0.0, 0.0, 0.1, 0.3]),
+        mask=rng.choice(["none", "pad", "pad", "pad", "full", "keyinf", "padinf", "padholes"]),
+        want_len=rng.random() < 0.3, want_strided=rng.random() < 0.25, one_pass=rng.random() < 0.3)
+    c.setdefault("lens", None)
+    c["use_len"] = c["mask"] == "none" and c.get("want_len", False) and c["d"] != 256
+    c["strided"] = c.get("want_strided", False) and c["mask"] != "full" and c["d"] != 256
+    if c["d"] == 256 and c["sq"] * c["sk"] > 300 * 300:   # keep the CPU oracle's share of the minute small
+        c["sq"], c["sk"] = min(c["sq"], 200), min(c["sk"], 257)
+    return c
+
+
+def _run_case(it, c, rng):
+    d, dtype, b, h, sq, sk, causal, p, maskk = (c[n] for n in ("d", "dtype", "b", "h", "sq", "sk", "causal", "p", "mask"))
+    bh = b * h
+    std = {64: 1.0, 128: 0.5, 256: 0.35}[d]
+    q, k, v, do = make_qkv(bh, sq, sk, d, seed=it, std=std, dtype=dtype, with_dout=True)
+    g = torch.Generator().manual_seed(it)
+    m = mo = None
+    if maskk in ("pad", "padinf", "padholes"):
+        m = torch.zeros(b, 1, 1, sk)
+        lens = c["lens"] or [rng.randint(1, sk) for _ in range(b)]
+        for i in range(b):
+            m[i, 0, 0, lens[i]:] = -10000.0 if maskk != "padinf" else float("-inf")
+        if maskk == "padholes":
+            m[:, :, :, torch.rand(sk, generator=g) < 0.3] = -10000.0
+    elif maskk == "full":
+        m = torch.randn(bh, sq, sk, generator=g) * 2
+    elif maskk == "keyinf":
+        m = torch.randn(bh, 1, sk, generator=g)
+        m[:, :, 1::3] = float("-inf")
+    if m is not None:
+        m = m.to(TDT[dtype])
+        mo = f32(m)
+    kw, okw = dict(causal=causal), dict(causal=causal)
+    if p:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=it * 7 + 1, offset=it)
+        okw.update(philox=True, p_drop=p, seed=it * 7 + 1, offset=it)
+    if c["use_len"]:
+        lens = torch.tensor([rng.randint(1, sk) for _ in range(b)], dtype=torch.int32)
+        kw["kv_len"] = lens.cuda()
+        mo = np.zeros((b, 1, 1, sk), np.float32)
+        for i, n in enumerate(lens.tolist()):
+            mo[i, 0, 0, n:] = -np.inf
+    qc, kc, vc, dc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    if c["strided"]:
+        def f(x):
+            return x.view(b, h, x.shape[1], d).permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        qc, kc, vc, dc = f(qc), f(kc), f(vc), f(dc)
+    mc = None if m is None else m.cuda()
+    bflags = capi.FLAG_BWD_ONE_PASS if c.get("one_pass") else 0
+    o, lse, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, **kw)
+    dq, dk, dv = capi.bwd(dc, qc, kc, vc, o, lse, mask=mc, flags=bflags, **kw)
+    torch.cuda.synchronize()
+    if maskk in ("pad", "padinf", "padholes", "keyinf"):
+        o2, lse2, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, flags=capi.FLAG_NO_MASK_TRIM, **kw)
+        g2 = capi.bwd(dc, qc, kc, vc, o, lse, mask=mc, flags=bflags | capi.FLAG_NO_MASK_TRIM, **kw)
+        assert torch.equal(o, o2) and torch.equal(lse, lse2), "forward: trimmed != untrimmed"
+        if not bflags:
+            assert all(torch.equal(x, y) for x, y in zip((dq, dk, dv), g2)), "backward: trimmed != untrimmed"
+        else:
+            # the one-pass kernel runs full key chunks on a hand-ordered instruction stream and partly
+            # filled ones on a plain loop; the two round the same dS element differently now and then
+            # (a fused multiply-convert against a multiply followed by a convert): one unit in the last place
+            for x, y in zip((dq, dk, dv), g2):
+                assert (x.float() - y.float()).abs().max().item() <= 2e-3 * max(1.0, y.float().abs().max().item())
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=mo, dout=f32(do), want=("o", "lse", "dq", "dk", "dv"), **okw)
+    otol = (2e-3 if dtype == "fp16" else 2e-2) * max(1.0, float(np.abs(ref["o"]).max()) / 2.0)
+    gtol = 1e-2 if dtype == "fp16" else 3e-2
+    got_o = f32(o.reshape(bh, sq, d).cpu())
+    assert np.abs(got_o - ref["o"]).max() <= otol, "o"
+    # the absolute bound for gradients whose true value is zero throughout (module docstring)
+    a_rows = np.abs(f32(do) * got_o).sum(-1)                                   # A_i per (head, query)
+    zero_tol = 4 * d ** -0.5 * UNIT[dtype] * float(np.sqrt((a_rows ** 2).sum(-1)).max()) * \
+        float(max(np.abs(f32(q)).max(), np.abs(f32(k)).max()))
+    for name, t in (("dq", dq), ("dk", dk), ("dv", dv)):
+        a = f32(t.reshape(ref[name].shape).cpu())
+        assert np.isfinite(a).all(), name
+        if name != "dv" and np.abs(ref[name]).max() < 1e-6:
+            assert np.abs(a).max() <= max(zero_tol, 1e-6), f"{name}: zero gradient, |got| {np.abs(a).max():.3e} > {zero_tol:.3e}"
+        else:
+            assert rel_to_max(a, ref[name], floor=1e-3) <= gtol, name
+    fin = np.isfinite(ref["lse"])
+    gl = lse.reshape(bh, sq).cpu().numpy()
+    assert np.array_equal(np.isfinite(gl), fin), "lse: -inf rows differ"
+    if fin.any():
+        assert np.abs(gl[fin] - ref["lse"][fin]).max() <= 5e-3 + 2.0 ** -8 * np.abs(ref["lse"][fin]).max(), "lse"
+
+
+# problems whose gradients with respect to q and k are zero throughout (every query sees one key)
+ZERO_GRADIENT = [
+    dict(d=64, dtype="bf16", b=1, h=2, sq=127, sk=1, causal=False, p=0.1, mask="none"),
+    dict(d=64, dtype="bf16", b=2, h=1, sq=520, sk=1, causal=True, p=0.0, mask="none"),
+    dict(d=128, dtype="fp16", b=1, h=4, sq=257, sk=8, causal=False, p=0.1, mask="padinf", lens=[1], want_strided=True),
+    dict(d=64, dtype="fp16", b=2, h=2, sq=300, sk=1, causal=False, p=0.3, mask="full"),
+    dict(d=64, dtype="fp16", b=1, h=1, sq=1, sk=200, causal=True, p=0.1, mask="none"),
+    dict(d=64, dtype="bf16", b=2, h=2, sq=300, sk=300, causal=False, p=0.1, mask="pad", lens=[1, 1], one_pass=True),
+]
+
+
+@pytest.mark.parametrize("idx", range(len(ZERO_GRADIENT)))
+def test_gradients_that_are_exactly_zero(idx):
+    rng = random.Random(1000 + idx)
+    _run_case(5000 + idx, _case(5000 + idx, rng, dict(ZERO_GRADIENT[idx])), rng)
+
+
+def test_randomized_sweep_against_the_oracle():
+    rng = random.Random(20241125)
+    for it in range(400):
+        c = _case(it, rng)
+        try:
+            _run_case(it, c, rng)
+        except AssertionError as e:
+            raise AssertionError(f"case #{it} {c}: {e}") from e

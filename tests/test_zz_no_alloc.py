@@ -24,7 +24,7 @@ def _params(q, k, v, o, do, lse, mask, dq, dk, dv, delta, flags=0):
     P.scale = d ** -0.5
     P.mask, P.mask_kind = mask.data_ptr(), capi.MASK_ADDITIVE
     P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = bh // mask.shape[0], k.shape[1], 0
-    P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, 0.1, 1 / 0.9, 5, 7
+    P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, 0.1, 0.0, 5, 7  # scale 0: the mean-preserving factor
     P.flags = flags
     return P
 
