@@ -2,7 +2,11 @@
  * C ABI of the gfx950 fused multi-head-attention library (libfmha_hip.so).
  *
  * Plain pointers and sizes only -- no torch / ATen types -- so the library can be
- * bound from C, C++, ctypes or any FFI.  All tensor pointers are DEVICE pointers;
+ * bound from C, C++, ctypes or any FFI.
+ *
+ * Input contract: q, k, v, dout and mask values are finite numbers or, for masks, -inf.  NaN or +inf
+ * inputs are not detected and do not propagate in any defined way (the kernels are compiled without
+ * NaN handling: they use -inf on purpose and never produce a NaN from finite inputs).  All tensor pointers are DEVICE pointers;
  * the library never allocates, frees or synchronises: kernels are enqueued on the
  * HIP stream the caller passes and the call returns immediately.
  *
@@ -98,7 +102,7 @@ typedef struct fmha_fwd_params {
   int32_t mask_kind;
   int32_t causal; /* 1: key j is visible to query i iff j <= i (no tensor involved) */
   int64_t mask_bh_div, mask_stride_b, mask_stride_q;
-  float mask_neg; /* used by FMHA_MASK_KEEP01; -10000 in the reference */
+  float mask_neg; /* used by FMHA_MASK_KEEP01; -10000 in the reference; must be finite and <= 0 */
 
   int32_t drop_kind;
   const void *drop_mask; /* FMHA_DROP_TENSOR: [bh,sq,sk], element type = dtype */
@@ -123,8 +127,7 @@ typedef struct fmha_fwd_params {
   /* Optional valid key counts (the "padded version" the reference leaves as a TODO,
    * fmha_manual.cpp:110,178): head b attends keys [0, kv_len[b / kv_len_bh_div]) only, exactly
    * as if the others carried a -inf mask, and whole key tiles past the count are never touched.
-   * Device pointer to int32, or NULL for all sk keys.  Not with FMHA_DROP_TENSOR / the save outputs, nor at head dim 256
-   * (forward). */
+   * Device pointer to int32, or NULL for all sk keys.  Not with FMHA_DROP_TENSOR / the save outputs. */
   const int32_t *kv_len;
   int32_t kv_len_bh_div;
 

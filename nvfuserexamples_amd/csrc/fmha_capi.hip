@@ -97,8 +97,8 @@ const char *fmha_strerror(int code) {
   case FMHA_E_DTYPE: return "unknown dtype (0 = fp16, 1 = bf16)";
   case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64, 128 or 256, and one head's rows must span less than 2^31 elements";
   case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned and their strides multiples of 8 elements";
-  case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, known mask/drop kind)";
-  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart; head dim 256 takes folded tensors only and, in the forward, no valid key counts)";
+  case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, mask_neg finite and <= 0, known mask/drop kind)";
+  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart; head dim 256 takes folded tensors only)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
   case FMHA_E_SCRATCH: return "fmha_bwd_launch_noalloc: bh * sq exceeds fmha_bwd_noalloc_max_rows() (the library's own scratch holds one float per query row); use fmha_bwd_launch with caller-provided delta";
   default: return "unknown error code";
@@ -174,6 +174,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
     if (!p->mask) return FMHA_E_NULL;
     if (p->mask_bh_div < 1 || p->mask_stride_b < 0 || p->mask_stride_q < 0) return FMHA_E_ARG;
   }
+  if (p->mask_kind == FMHA_MASK_KEEP01 && !(std::isfinite(p->mask_neg) && p->mask_neg <= 0.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_TENSOR && !p->drop_mask) return FMHA_E_NULL;
   if (p->drop_kind != FMHA_DROP_NONE && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
@@ -187,8 +188,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (p->drop_kind == FMHA_DROP_TENSOR && p->causal) return FMHA_E_UNSUPPORTED;
   if (p->kv_len) {
     if (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u)) return FMHA_E_ARG;
-    // (the plain forward loop, which also serves head dim 256, does not read the counts)
-    if (saving || p->drop_kind == FMHA_DROP_TENSOR || p->d == 256) return FMHA_E_UNSUPPORTED;
+    if (saving || p->drop_kind == FMHA_DROP_TENSOR) return FMHA_E_UNSUPPORTED;
   }
   if ((uintptr_t)p->clock_probe & 7u) return FMHA_E_ARG;
 
@@ -384,6 +384,7 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
     if (!p->mask) return FMHA_E_NULL;
     if (p->mask_bh_div < 1 || p->mask_stride_b < 0 || p->mask_stride_q < 0) return FMHA_E_ARG;
   }
+  if (p->mask_kind == FMHA_MASK_KEEP01 && !(std::isfinite(p->mask_neg) && p->mask_neg <= 0.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_PHILOX && !(p->p_drop >= 0.f && p->p_drop < 1.f)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_PHILOX && !std::isfinite(p->drop_scale)) return FMHA_E_ARG;
   if (p->drop_kind == FMHA_DROP_PHILOX) {

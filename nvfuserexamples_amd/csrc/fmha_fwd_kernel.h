@@ -62,7 +62,7 @@ struct FwdArgs {
   float drop_scale;
   DropCtx drop;
   int32_t flags;
-  const int32_t *kv_len; // optional valid key count per group of kv_div heads (pipelined kernel only)
+  const int32_t *kv_len; // optional valid key count per group of kv_div heads (not with tensor dropout / saved outputs)
   int32_t kv_div;
   unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
   RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
@@ -167,8 +167,15 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     }
   }
 
-  // ---- key range
-  int nkt = (a.sk + BK - 1) / BK;
+  // ---- key range: all sk keys, or the head's valid count (keys at or past it get a -inf mask term, whole
+  // tiles past it are not visited; a count of 0 visits one tile that is masked throughout: O = 0, LSE = -inf)
+  int skv = a.sk;
+  if (a.kv_len) {
+    const int n = a.kv_len[bh / a.kv_div];
+    skv = n < 0 ? 0 : (n < a.sk ? n : a.sk);
+  }
+  int nkt = (skv + BK - 1) / BK;
+  if (nkt < 1) nkt = 1;
   if (CAUSAL) {
     int qmax = qt * QT + QT - 1;
     if (qmax > a.sq - 1) qmax = a.sq - 1;
@@ -194,8 +201,8 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     }
     {
       const int kr = k0 + (tid & (BK - 1));
-      mvalid = kr < a.sk;
-      if (MASK == kMaskPerKey) mraw = mkey[mvalid ? kr : a.sk - 1];
+      mvalid = kr < skv;
+      if (MASK == kMaskPerKey) mraw = mkey[kr < a.sk ? kr : a.sk - 1];
     }
   };
   auto lstore = [&](int stage) {

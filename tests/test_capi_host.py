@@ -32,10 +32,14 @@ def test_library_exports_every_declared_symbol():
 def test_strerror_and_threshold():
     L = capi.lib()
     assert L.fmha_strerror(0) == b"ok"
-    msgs = {L.fmha_strerror(c) for c in range(-7, 1)}
-    assert len(msgs) == 8 and all(msgs)
-    for p in (0.0, 0.05, 0.1, 0.25, 0.5, 0.9, 0.999):
+    msgs = {L.fmha_strerror(c) for c in range(-8, 1)}
+    assert len(msgs) == 9 and all(msgs)
+    assert b"256" in L.fmha_strerror(-3) and b"unknown" in L.fmha_strerror(-99)
+    for p in (0.0, 0.001, 0.05, 0.1, 0.25, 0.5, 0.9, 0.999):
         assert L.fmha_drop_threshold(p) == oracle.drop_threshold(p)
+        assert L.fmha_drop_scale(p) == pytest.approx(oracle.drop_scale(p), rel=1e-7)
+        assert L.fmha_drop_scale(p) * (256 - L.fmha_drop_threshold(p)) / 256 == pytest.approx(1.0, abs=1e-6)
+    assert L.fmha_bwd_noalloc_max_rows() * 4 == 8 << 20
 
 
 def _valid_params():
@@ -58,6 +62,10 @@ def _valid_params():
     (lambda P: setattr(P, "scale", float("nan")), -5),
     (lambda P: setattr(P, "mask_kind", 9), -5),
     (lambda P: setattr(P, "mask_kind", 1), -1),                       # mask kind without a pointer
+    (lambda P: (setattr(P, "mask", 0x1000), setattr(P, "mask_kind", 2), setattr(P, "mask_bh_div", 1),
+                setattr(P, "mask_neg", float("-inf"))), -5),         # 0/1 masks: mask_neg must be finite ...
+    (lambda P: (setattr(P, "mask", 0x1000), setattr(P, "mask_kind", 2), setattr(P, "mask_bh_div", 1),
+                setattr(P, "mask_neg", 5.0)), -5),                    # ... and not positive
     (lambda P: (setattr(P, "drop_kind", 1), setattr(P, "p_drop", 1.0)), -5),
     (lambda P: setattr(P, "drop_kind", 2), -1),                       # tensor dropout without a tensor
     (lambda P: (setattr(P, "save_softmax", 0x1000), setattr(P, "causal", 1)), -6),

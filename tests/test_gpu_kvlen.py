@@ -42,12 +42,14 @@ CASES = [
     (6, 6, 320, 320, 64, "fp16", True, 0.0),      # causal
     (4, 2, 256, 256, 128, "bf16", False, 0.0),
     (600, 300, 128, 192, 64, "fp16", False, 0.0),  # more items than resident workgroups: per-item counts
+    (4, 2, 200, 333, 256, "fp16", False, 0.1),     # head dim 256: the plain forward loop reads the counts too
+    (4, 4, 192, 192, 256, "bf16", True, 0.0),
 ]
 
 
 @pytest.mark.parametrize("bh,b,sq,sk,d,dtype,causal,p", CASES)
 def test_kv_len_matches_oracle_with_inf_mask(bh, b, sq, sk, d, dtype, causal, p):
-    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
+    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std={64: 1.0, 128: 0.5, 256: 0.35}[d], dtype=dtype, with_dout=True)
     lens = _lens(b, sk, seed=sk)
     kw, okw = dict(causal=causal), dict(causal=causal)
     if p:
@@ -87,8 +89,9 @@ def test_kv_len_equals_additive_padding_mask_bit_for_bit(bh, b, s, d):
         assert torch.equal(a, c)
 
 
-def test_zero_count_gives_zero_output():
-    q, k, v = make_qkv(4, 64, 96, 64, seed=1)
+@pytest.mark.parametrize("d", [64, 256])
+def test_zero_count_gives_zero_output(d):
+    q, k, v = make_qkv(4, 64, 96, d, seed=1, std=0.5)
     lens = torch.tensor([0, 40], dtype=torch.int32)
     o, lse, _, _ = capi.fwd(q.cuda(), k.cuda(), v.cuda(), kv_len=lens.cuda(), want_lse=True)
     torch.cuda.synchronize()
