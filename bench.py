@@ -12,7 +12,21 @@ through the C ABI (``libfmha_hip.so``) on torch's current HIP stream:
 Inputs are resident in HBM before the timed region; several input sets are rotated
 so that consecutive steps do not find their operands in the 256 MB last-level cache.
 Prints ONE JSON line.  ``value`` is forward TFLOP/s (4*BH*S*S*D flops per step); the
-train-step figure (14*BH*S*S*D) rides along under ``fwd_bwd`` when that path is built.
+train-step figure (14*BH*S*S*D) rides along under ``fwd_bwd``, and the long-sequence and
+wide-head train-step configurations under ``configs``.
+
+Timing protocol (every leg): W warm-up steps, then at least 0.3 s of the same steps so that the
+board's clocks and power state settle (the kernels are power-limited: the first millisecond of a
+cold run is not representative), then 25 blocks of exactly K steps each, every block bracketed by
+HIP events on the launch stream and a device synchronisation; the MEDIAN block is reported
+(``ms_per_step``), with the spread beside it.  ``roofline.launch_us`` is the same statistic over
+blocks in which every launch has an event pair of its own (the figure comparable with rocprofv3's
+per-kernel average); the step time exceeds it by the gap between back-to-back launches.
+
+Work that is counted is work that is executed: the headline forward and train step run with
+FMHA_FLAG_NO_MASK_TRIM, i.e. they visit every key tile of the dense shape the flop count is defined
+on.  The library's default -- leaving out key tiles that the padding mask leaves without a live key,
+with bit-identical results -- is timed beside them (``fwd_mask_trim``, ``fwd_bwd.mask_trim_*``).
 """
 import argparse
 import ctypes as C
@@ -52,8 +66,9 @@ def make_inputs(torch, capi, nsets, seed=0, train=False):
     return sets
 
 
-def fwd_params(capi, t, train=False):
+def fwd_params(capi, t, train=False, flags=0):
     P = capi.FwdParams()
+    P.flags = flags
     P.q, P.k, P.v, P.o = (t[n].data_ptr() for n in ("q", "k", "v", "o"))
     P.mask, P.mask_kind = t["mask"].data_ptr(), capi.MASK_ADDITIVE
     P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = H, S, 0
@@ -66,8 +81,9 @@ def fwd_params(capi, t, train=False):
     return P
 
 
-def bwd_params(capi, t):
+def bwd_params(capi, t, flags=0):
     P = capi.BwdParams()
+    P.flags = flags
     for n in ("q", "k", "v", "o", "dout", "lse", "delta", "dq", "dk", "dv"):
         setattr(P, n, t[n].data_ptr())
     P.mask, P.mask_kind = t["mask"].data_ptr(), capi.MASK_ADDITIVE
@@ -79,36 +95,66 @@ def bwd_params(capi, t):
     return P
 
 
-def time_steps(torch, step, steps, warmup):
-    """HIP events on the stream the kernels are launched on (torch's current stream)."""
+BLOCKS = 25     # timed blocks per leg; the median block is reported
+BURN_S = 0.3    # seconds of the same steps before timing, for clocks and power state to settle
+
+
+def _median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
+def settle(torch, step, warmup):
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        step(i)
-    e1.record()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) * 1e3
-    return e0.elapsed_time(e1) / steps, wall / steps
+    t0, i = time.perf_counter(), warmup
+    while time.perf_counter() - t0 < BURN_S:
+        for _ in range(20):
+            step(i)
+            i += 1
+        torch.cuda.synchronize()
+    return i
 
 
-def time_launches(torch, step, steps, warmup):
-    """Average duration of ONE launch: a HIP event pair around every launch of the timed region
-    (same stream as the kernels).  Excludes the idle gap between back-to-back launches, so it is
-    the figure comparable with rocprofv3's per-kernel average."""
-    for i in range(warmup):
-        step(i)
-    torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for i, (a, b) in enumerate(ev):
-        a.record()
-        step(i)
-        b.record()
-    torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in ev) / steps
+def time_steps(torch, step, steps, warmup, blocks=BLOCKS, stats=None):
+    """Median over `blocks` blocks of exactly `steps` steps each; HIP events on the stream the kernels are
+    launched on (torch's current stream), a synchronisation either side of every block.  Returns
+    (ms per step, host wall ms per step of the median block); `stats` receives the spread."""
+    i0 = settle(torch, step, warmup)
+    per, walls = [], []
+    for b in range(blocks):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            step(i0 + i)
+        e1.record()
+        torch.cuda.synchronize()
+        walls.append((time.perf_counter() - t0) * 1e3 / steps)
+        per.append(e0.elapsed_time(e1) / steps)
+    if stats is not None:
+        stats.update(blocks=blocks, steps_per_block=steps, block_ms_min=round(min(per), 5), block_ms_max=round(max(per), 5))
+    return _median(per), _median(walls)
+
+
+def time_launches(torch, step, steps, warmup, blocks=BLOCKS):
+    """Duration of ONE launch: a HIP event pair around every launch (same stream as the kernels), averaged
+    over a block of `steps` launches; the median block.  Excludes the idle gap between back-to-back
+    launches, so it is the figure comparable with rocprofv3's per-kernel average."""
+    i0 = settle(torch, step, warmup)
+    per = []
+    for b in range(blocks):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i, (a, c) in enumerate(ev):
+            a.record()
+            step(i0 + i)
+            c.record()
+        torch.cuda.synchronize()
+        per.append(sum(a.elapsed_time(c) for a, c in ev) / steps)
+    return _median(per)
 
 
 def short_sequence_legs(torch, capi, L, stream, steps, warmup):
@@ -309,6 +355,67 @@ def head_dim_256_leg(torch, capi):
             "bwd_us": round(b_ms * 1e3, 1), "bwd_tflops": round(2.5 * flops / (b_ms * 1e-3) / 1e12, 1)}
 
 
+def config_leg(torch, capi, L, stream, steps, warmup, b, h, s, d, dtype, causal, p_drop, std, nsets):
+    """Forward, backward and train step of one benchmark configuration (no padding mask), through the C ABI.
+    Flops: 4 / 10 / 14 * BH*S*S*D, times (S+1)/(2S) under the causal mask (the tiles above the diagonal are
+    neither counted nor visited).  Bytes: forward 4*BH*S*D*e + BH*S*4 (LSE), backward 8*BH*S*D*e + 2*BH*S*4."""
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    bh = b * h
+    g = torch.Generator().manual_seed(11)
+    sets = []
+    for _ in range(nsets):
+        t = {n: (torch.randn(bh, s, d, generator=g) * std).to(tdt).cuda() for n in ("q", "k", "v", "dout")}
+        for n in ("o", "dq", "dk", "dv"):
+            t[n] = torch.empty_like(t["q"])
+        t["lse"], t["delta"] = (torch.empty(bh, s, dtype=torch.float32, device="cuda") for _ in range(2))
+        F, Bp = capi.FwdParams(), capi.BwdParams()
+        for P in (F, Bp):
+            P.q, P.k, P.v, P.o, P.lse = (t[n].data_ptr() for n in ("q", "k", "v", "o", "lse"))
+            P.bh, P.sq, P.sk, P.d = bh, s, s, d
+            P.dtype, P.scale, P.causal = (capi.F16 if dtype == "f16" else capi.BF16), d ** -0.5, int(causal)
+            if p_drop:
+                P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, p_drop, 0.0, 0x1234, 0
+        Bp.dout, Bp.delta, Bp.dq, Bp.dk, Bp.dv = (t[n].data_ptr() for n in ("dout", "delta", "dq", "dk", "dv"))
+        sets.append((t, F, Bp))
+    capi.check(L.fmha_fwd_launch(C.byref(sets[0][1]), stream))
+    capi.check(L.fmha_bwd_launch(C.byref(sets[0][2]), stream))
+
+    def fwd(i):
+        L.fmha_fwd_launch(C.byref(sets[i % nsets][1]), stream)
+
+    def bwd(i):
+        L.fmha_bwd_launch(C.byref(sets[i % nsets][2]), stream)
+
+    def both(i):
+        fwd(i)
+        bwd(i)
+    for _, F, _ in sets:   # every set's O and LSE must exist before its backward is timed alone
+        L.fmha_fwd_launch(C.byref(F), stream)
+    n = max(5, steps // 4) if s * s * bh > 2 ** 27 else steps
+    blocks = 9 if s * s * bh * d > 2 ** 34 else BLOCKS
+    ms_f, _ = time_steps(torch, fwd, n, warmup, blocks)
+    ms_b, _ = time_steps(torch, bwd, n, warmup, blocks)
+    ms_t, _ = time_steps(torch, both, n, warmup, blocks)
+    dense = float(bh) * s * s * d
+    cf = (s + 1) / (2.0 * s) if causal else 1.0
+    e = 2
+    by_f = 4.0 * bh * s * d * e + bh * s * 4
+    by_b = 8.0 * bh * s * d * e + 2 * bh * s * 4
+
+    def part(ms, fl, by):
+        tf = fl * cf / (ms * 1e-3) / 1e12
+        return {"us": round(ms * 1e3, 1), "tflops": round(tf, 1), "mfma_frac": round(tf / PEAK_MFMA_TFLOPS, 4),
+                "hbm_GBps": round(by / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)}
+    out = {"workload": f"B{b} H{h} S{s} D{d} {dtype}, {'causal mask' if causal else 'no mask'}, "
+                       f"{'Philox dropout p=%g' % p_drop if p_drop else 'no dropout'}; {nsets} input set(s) rotated",
+           "flops_counted": "causal count: dense x (S+1)/(2S)" if causal else "dense",
+           "fwd": part(ms_f, 4 * dense, by_f), "bwd": part(ms_b, 10 * dense, by_b),
+           "fwd_bwd": part(ms_t, 14 * dense, by_f + by_b), "steps_per_block": n, "blocks": blocks}
+    if causal:
+        out["fwd_bwd"]["tflops_full_count"] = round(14 * dense / (ms_t * 1e-3) / 1e12, 1)
+    return out
+
+
 def torch_sdpa_context(torch, steps, warmup):
     """For scale only: PyTorch's own fused attention (torch.nn.functional.scaled_dot_product_attention,
     whichever backend it selects) on the same GPU at the headline shape, [B,H,S,D] fp16 tensors -- the
@@ -469,24 +576,33 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---- forward (headline)
+    # ---- forward (headline): every key tile of the dense shape is visited (FMHA_FLAG_NO_MASK_TRIM), so the
+    # flops that are counted are flops that are executed; the library's default (tiles under the hard-masked
+    # tail left out, same bits) is `fps` and is timed beside it
     sets = make_inputs(torch, capi, args.sets)
     fps = [fwd_params(capi, t) for t in sets]
-    rc = L.fmha_fwd_launch(C.byref(fps[0]), stream)
-    capi.check(rc)
+    fps_dense = [fwd_params(capi, t, flags=capi.FLAG_NO_MASK_TRIM) for t in sets]
+    capi.check(L.fmha_fwd_launch(C.byref(fps[0]), stream))
+    capi.check(L.fmha_fwd_launch(C.byref(fps_dense[0]), stream))
 
     def fwd_step(i):
         L.fmha_fwd_launch(C.byref(fps[i % len(fps)]), stream)
 
-    ms, wall_ms = time_steps(torch, fwd_step, args.steps, args.warmup)
+    def fwd_dense(i):
+        L.fmha_fwd_launch(C.byref(fps_dense[i % len(fps_dense)]), stream)
+
+    spread = {}
+    ms, wall_ms = time_steps(torch, fwd_dense, args.steps, args.warmup, stats=spread)
+    ms_launch = time_launches(torch, fwd_dense, args.steps, args.warmup)
+    ms_trim, _ = time_steps(torch, fwd_step, args.steps, args.warmup)
+    ms_trim_launch = time_launches(torch, fwd_step, args.steps, args.warmup)
     flops = 4.0 * B * H * S * S * D
     bytes_ = 4.0 * B * H * S * D * 2 + B * S * 2
     tflops = flops / (ms * 1e-3) / 1e12
     # warm-cache figure for reference: one input set only
     def fwd_warm(i):
-        L.fmha_fwd_launch(C.byref(fps[0]), stream)
+        L.fmha_fwd_launch(C.byref(fps_dense[0]), stream)
     ms_warm, _ = time_steps(torch, fwd_warm, args.steps, args.warmup)
-    ms_launch = time_launches(torch, fwd_step, args.steps, args.warmup)
     # the same steps dealt to two streams in turn (default priority): the first workgroups of a launch start
     # on the compute units that the previous launch has already left, which hides the drain-and-dispatch
     # gap between back-to-back launches on one stream.  Reported beside the headline, never as `value`.
@@ -496,12 +612,15 @@ def main():
         for i in range(n):
             L.fmha_fwd_launch(C.byref(fps[i % len(fps)]), s2p[i & 1])
     torch.cuda.synchronize()
-    two_stream_steps(args.warmup)
+    two_stream_steps(max(args.warmup, 2000))
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    two_stream_steps(args.steps)
-    torch.cuda.synchronize()
-    ms_two = (time.perf_counter() - t0) * 1e3 / args.steps  # host clock around the whole region, synchronised both ends
+    regions = []
+    for _ in range(BLOCKS):
+        t0 = time.perf_counter()
+        two_stream_steps(max(args.steps, 100))
+        torch.cuda.synchronize()
+        regions.append((time.perf_counter() - t0) * 1e3 / max(args.steps, 100))  # host clock, synchronised both ends
+    ms_two = _median(regions)
     tflops_launch = flops / (ms_launch * 1e-3) / 1e12
     # the same batches with the valid lengths handed over as counts (kv_len) instead of an additive
     # mask: same outputs bit for bit, key tiles past a sequence's length are skipped.  Reported
@@ -560,7 +679,7 @@ def main():
     # share of the (query tile, 128-key tile pair) products the kernel really visits: it leaves out the tile
     # pairs that hold only hard-masked keys (their weights are exactly zero)
     visited = float(sum(((n.float() / 128).ceil() * 128 / S).mean().item() for n in lens) / len(lens))
-    del sets, fps, lps, lens
+    del sets, fps, fps_dense, lps, lens
 
     out = {
         "metric": "MHA fwd TFLOP/s (B32,H16,S512,D64 fp16)", "value": round(tflops, 2), "unit": "TFLOP/s",
@@ -568,34 +687,44 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "BERT-large attention forward: B32 H16 S512 D64 fp16, additive [B,1,1,S] "
-                               "padding mask (valid length U{256..512}), scale 1/8, no dropout",
+                               "padding mask (valid length U{256..512}), scale 1/8, no dropout; every key tile "
+                               "visited (FMHA_FLAG_NO_MASK_TRIM)",
                    "layout": "[B*H,S,D] contiguous", "input_sets_rotated": args.sets},
-        # achieved = algorithmic flops of one launch / mean launch duration (event pair per launch);
+        "timing": dict(spread, protocol=f"{args.warmup} warm-up steps + {BURN_S} s of the same steps, then the median of "
+                                        f"{BLOCKS} blocks of {args.steps} steps, each between HIP events and a synchronisation"),
+        "value_frac_of_mfma_peak": round(tflops / PEAK_MFMA_TFLOPS, 4),
+        # achieved = algorithmic flops of one launch / launch duration (event pair per launch, median block);
         # traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
         # counter reads for a 256 MiB copy (profiles/fmha_fwd_pipe_kernel_B32H16S512D64_f16.md)
         "roofline": {"bound": "mfma", "achieved": round(tflops_launch, 2), "peak": PEAK_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tflops_launch / PEAK_MFMA_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "fmha_fwd_pipe_kernel<f16,D64,per-key mask>", "flops_per_launch": flops,
-                     # flops_per_launch is the dense count of the shape (what the metric is defined on); the
-                     # kernel skips key tiles that the padding mask leaves without a live key
-                     "visited_tile_share": round(visited, 4),
-                     "executed_tflops": round(tflops_launch * visited, 2),
+                     "executed_frac": round(tflops_launch / PEAK_MFMA_TFLOPS, 4),   # every counted tile is visited
+                     "visited_tile_share": 1.0,
                      "algorithmic_bytes_per_launch": bytes_,
                      "hbm_achieved_GBps": round(bytes_ / (ms * 1e-3) / 1e9, 1),
                      "hbm_frac": round(bytes_ / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                      "hbm_achieved_GBps_launch": round(bytes_ / (ms_launch * 1e-3) / 1e9, 1),
-                     "launch_us": round(ms_launch * 1e3, 2)},
+                     "launch_us": round(ms_launch * 1e3, 2),
+                     "launch_gap_us": round((ms - ms_launch) * 1e3, 2)},
+        # the library's default on the same batches: key tiles that hold only hard-masked keys are left out
+        # (bit-identical outputs); flops still counted for the dense shape, and the share really executed
+        "fwd_mask_trim": {"ms_per_step": round(ms_trim, 5), "launch_us": round(ms_trim_launch * 1e3, 2),
+                          "tflops_dense_count": round(flops / (ms_trim * 1e-3) / 1e12, 2),
+                          "visited_tile_share": round(visited, 4),
+                          "tflops_executed": round(flops * visited / (ms_trim * 1e-3) / 1e12, 2),
+                          "speedup_vs_every_tile": round(ms / ms_trim, 3)},
         "fwd_warm_cache": {"ms_per_step": round(ms_warm, 5),
                            "tflops": round(flops / (ms_warm * 1e-3) / 1e12, 2)},
         "host_wall_ms_per_step": round(wall_ms, 5),
-        "fwd_two_streams": {"workload": "the same steps issued to two streams in turn (independent batches in flight "
+        "fwd_two_streams": {"workload": "the default steps issued to two streams in turn (independent batches in flight "
                                         "together); host clock over the whole region",
-                            "ms_per_step": round(ms_two, 5), "tflops": round(flops / (ms_two * 1e-3) / 1e12, 2)},
+                            "ms_per_step": round(ms_two, 5), "speedup_vs_one_stream": round(ms_trim / ms_two, 3)},
         "fwd_kv_len": {"workload": "same batches, valid lengths passed as counts instead of the mask tensor",
-                       "ms_per_step": round(ms_len, 5), "speedup_vs_mask": round(ms / ms_len, 3)},
+                       "ms_per_step": round(ms_len, 5), "speedup_vs_default_mask_path": round(ms_trim / ms_len, 3)},
         "fwd_packed_qkv": {"workload": "same batches as a packed [B,S,3,H,D] tensor read in place, O written as "
-                                       "[B,S,H,D]",
+                                       "[B,S,H,D] (default mask path)",
                            "ms_per_step": round(ms_packed, 5),
                            "permute_copies_spared_ms": round(ms_perm, 5)},
     }
@@ -607,42 +736,84 @@ def main():
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
-    # ---- train step (forward with LSE + Philox dropout, then backward)
+    # ---- train step (forward with LSE + Philox dropout, then backward): every key tile visited, as the
+    # headline; the default (trimming) run and the valid-length run beside it
     if not args.no_bwd:
         tsets = make_inputs(torch, capi, args.sets, seed=1, train=True)
-        tf = [fwd_params(capi, t, train=True) for t in tsets]
-        tb = [bwd_params(capi, t) for t in tsets]
+        NT = capi.FLAG_NO_MASK_TRIM
+        tf = [fwd_params(capi, t, train=True, flags=NT) for t in tsets]
+        tb = [bwd_params(capi, t, flags=NT) for t in tsets]
         rc_f = L.fmha_fwd_launch(C.byref(tf[0]), stream)
         rc_b = L.fmha_bwd_launch(C.byref(tb[0]), stream)
         if rc_f == 0 and rc_b == 0:
+            for F in tf:
+                L.fmha_fwd_launch(C.byref(F), stream)   # O and LSE of every set, for the backward timed alone
+
             def train_step(i):
                 L.fmha_fwd_launch(C.byref(tf[i % len(tf)]), stream)
                 L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream)
-            steps = max(10, args.steps // 2)
-            ms_t, _ = time_steps(torch, train_step, steps, max(5, args.warmup // 2))
+
             def bwd_step(i):
                 L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream)
-            ms_b, _ = time_steps(torch, bwd_step, steps, max(5, args.warmup // 2))
+
+            def fwd_t(i):
+                L.fmha_fwd_launch(C.byref(tf[i % len(tf)]), stream)
+            tsp = {}
+            ms_t, _ = time_steps(torch, train_step, args.steps, args.warmup, stats=tsp)
+            ms_b, _ = time_steps(torch, bwd_step, args.steps, args.warmup)
+            ms_f, _ = time_steps(torch, fwd_t, args.steps, args.warmup)
             fl_t = 14.0 * B * H * S * S * D
+            by_t = 12.0 * B * H * S * D * 2 + 3 * B * H * S * 4 + 2 * B * S * 2
             out["fwd_bwd"] = {
-                "workload": "same shape, train step: fwd (+LSE) + bwd, Philox dropout p=0.1, padding mask",
+                "workload": "same shape, train step: fwd (+LSE) + bwd, Philox dropout p=0.1, padding mask, every key "
+                            "tile visited (FMHA_FLAG_NO_MASK_TRIM)",
                 "ms_per_step": round(ms_t, 5), "tflops": round(fl_t / (ms_t * 1e-3) / 1e12, 2),
                 "frac_of_mfma_peak": round(fl_t / (ms_t * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS, 4),
-                "bwd_only_ms": round(ms_b, 5),
-                "bwd_only_tflops": round(10.0 * B * H * S * S * D / (ms_b * 1e-3) / 1e12, 2), "steps": steps}
+                "hbm_frac": round(by_t / (ms_t * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                "fwd_only_ms": round(ms_f, 5), "bwd_only_ms": round(ms_b, 5),
+                "bwd_only_tflops": round(10.0 * B * H * S * S * D / (ms_b * 1e-3) / 1e12, 2),
+                "timing": tsp}
+            for P in tf + tb:
+                P.flags = 0
+            ms_tt, _ = time_steps(torch, train_step, args.steps, args.warmup)
+            ms_bt, _ = time_steps(torch, bwd_step, args.steps, args.warmup)
+            tlens = [(t["mask"][:, 0, 0, :] == 0).sum(dim=1).to(torch.int32).contiguous() for t in tsets]
+            vis_t = float(sum(((n.float() / 128).ceil() * 128 / S).mean().item() for n in tlens) / len(tlens))
+            out["fwd_bwd"].update(mask_trim_ms_per_step=round(ms_tt, 5), mask_trim_bwd_only_ms=round(ms_bt, 5),
+                                  mask_trim_tflops_dense_count=round(fl_t / (ms_tt * 1e-3) / 1e12, 2),
+                                  mask_trim_visited_tile_share=round(vis_t, 4),
+                                  mask_trim_tflops_executed=round(fl_t * vis_t / (ms_tt * 1e-3) / 1e12, 2))
+            # the one-pass backward (opt-in) on the same batches
+            need = int(L.fmha_bwd_workspace_bytes(B * H, S, S, D))
+            ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+            for P in tb:
+                P.flags, P.workspace, P.workspace_bytes = capi.FLAG_BWD_ONE_PASS, ws.data_ptr(), need
+            if L.fmha_bwd_launch(C.byref(tb[0]), stream) == 0:
+                ms_b1, _ = time_steps(torch, bwd_step, args.steps, args.warmup)
+                out["fwd_bwd"]["one_pass_bwd_only_ms"] = round(ms_b1, 5)
+            for P in tb:
+                P.flags, P.workspace, P.workspace_bytes = 0, None, 0
             # the same train step with the valid lengths handed over as counts (kv_len) instead of the mask
             # tensor: same results, key tiles past a sequence's length skipped in all three kernels
-            tlens = [(t["mask"][:, 0, 0, :] == 0).sum(dim=1).to(torch.int32).contiguous() for t in tsets]
             for P, n in zip(tf + tb, tlens + tlens):
                 P.mask, P.mask_kind = None, capi.MASK_NONE
                 P.kv_len, P.kv_len_bh_div = n.data_ptr(), H
             if L.fmha_fwd_launch(C.byref(tf[0]), stream) == 0 and L.fmha_bwd_launch(C.byref(tb[0]), stream) == 0:
-                ms_tl, _ = time_steps(torch, train_step, steps, max(5, args.warmup // 2))
+                ms_tl, _ = time_steps(torch, train_step, args.steps, args.warmup)
                 out["fwd_bwd"]["kv_len_ms_per_step"] = round(ms_tl, 5)
-                out["fwd_bwd"]["kv_len_speedup_vs_mask"] = round(ms_t / ms_tl, 3)
+                out["fwd_bwd"]["kv_len_speedup_vs_default_mask_path"] = round(ms_tt / ms_tl, 3)
+            del ws
         else:
             out["fwd_bwd"] = {"error": f"fwd rc={rc_f} bwd rc={rc_b}: " + L.fmha_strerror(rc_b or rc_f).decode()}
         del tsets
+        torch.cuda.empty_cache()
+        # ---- the other train-step configurations (no padding): long sequences, and wide heads in bf16 under the causal mask
+        out["configs"] = {
+            "C4_long_sequence": config_leg(torch, capi, L, stream, args.steps, args.warmup, 4, 16, 2048, 64, "f16",
+                                           False, 0.1, 1.0, 2),
+            "C5_wide_head_bf16_causal": config_leg(torch, capi, L, stream, args.steps, args.warmup, 16, 32, 1024, 128,
+                                                   "bf16", True, 0.0, 0.5, 1),
+        }
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch)
