@@ -416,6 +416,39 @@ def config_leg(torch, capi, L, stream, steps, warmup, b, h, s, d, dtype, causal,
     return out
 
 
+def fp8_leg(torch, capi, L, stream, steps, warmup):
+    """The e4m3 forward (a separate operator, first untuned kernel) at the headline shape with the same padding
+    masks: time and TFLOP/s against the dense fp8 MFMA peak.  Never part of `value`."""
+    g = torch.Generator().manual_seed(21)
+    sets = []
+    for _ in range(4):
+        q8, k8, v8 = (torch.randn(B * H, S, D, generator=g).to(torch.float8_e4m3fn).cuda() for _ in range(3))
+        lens = torch.randint(S // 2, S + 1, (B,), generator=g)
+        mask = torch.zeros(B, 1, 1, S)
+        for b in range(B):
+            mask[b, 0, 0, lens[b]:] = -10000.0
+        mask = mask.half().cuda()
+        o = torch.empty(B * H, S, D, dtype=torch.float16, device="cuda")
+        P = capi.FwdFp8Params()
+        P.q, P.k, P.v, P.o = q8.data_ptr(), k8.data_ptr(), v8.data_ptr(), o.data_ptr()
+        P.mask, P.mask_bh_div, P.mask_stride_b = mask.data_ptr(), H, S
+        P.bh, P.sq, P.sk, P.d = B * H, S, S, D
+        P.out_dtype, P.scale = capi.F16, 0.125
+        P.descale_q = P.descale_k = P.descale_v = 1.0
+        sets.append((P, q8, k8, v8, mask, o))
+    capi.check(L.fmha_fwd_fp8_launch(C.byref(sets[0][0]), stream))
+
+    def step(i):
+        L.fmha_fwd_fp8_launch(C.byref(sets[i % len(sets)][0]), stream)
+    ms, _ = time_steps(torch, step, steps, warmup)
+    fl = 4.0 * B * H * S * S * D
+    by = 3.0 * B * H * S * D + B * H * S * D * 2 + B * S * 2
+    return {"workload": "B32 H16 S512 D64, q/k/v e4m3, O fp16, [B,1,1,S] padding mask; 4 input sets rotated",
+            "us": round(ms * 1e3, 2), "tflops": round(fl / (ms * 1e-3) / 1e12, 1),
+            "frac_of_fp8_mfma_peak": round(fl / (ms * 1e-3) / 1e12 / 5000.0, 4),
+            "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)}
+
+
 def torch_sdpa_context(torch, steps, warmup):
     """For scale only: PyTorch's own fused attention (torch.nn.functional.scaled_dot_product_attention,
     whichever backend it selects) on the same GPU at the headline shape, [B,H,S,D] fp16 tensors -- the
@@ -733,6 +766,7 @@ def main():
     out["operators_BH512_S128_D64"] = operator_legs(torch, args.steps, args.warmup)
     out["torch_sdpa_same_gpu"] = torch_sdpa_context(torch, args.steps, args.warmup)
     out["head_dim_256"] = head_dim_256_leg(torch, capi)
+    out["fp8_e4m3_forward"] = fp8_leg(torch, capi, L, stream, args.steps, args.warmup)
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 

@@ -426,6 +426,52 @@ fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, co
   return std::make_tuple(dq, dk, dv);
 }
 
+// Forward on e4m3 inputs (torch.float8_e4m3fn, [B*H,S,D] contiguous, D = 64 or 128) with one dequantisation
+// factor per tensor; O comes back as float16, or bfloat16 when out_bf16 (the dtype an optional per-key additive
+// mask [B*H|B,1,Sk] / [B,1,1,Sk] must have).  Returns (O, LSE fp32).  Not in the reference (fp16 only).
+std::tuple<at::Tensor, at::Tensor> fmha_fwd_fp8(const at::Tensor &q8, const at::Tensor &k8, const at::Tensor &v8,
+                                                double descale_q, double descale_k, double descale_v,
+                                                const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
+                                                bool out_bf16) {
+  for (const at::Tensor *t : {&q8, &k8, &v8})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat8_e4m3fn && t->dim() == 3 && t->is_contiguous(),
+                "mha_manual: q, k, v must be contiguous [B*H,S,D] float8_e4m3fn GPU tensors");
+  TORCH_CHECK(k8.size(0) == q8.size(0) && v8.sizes() == k8.sizes() && k8.size(2) == q8.size(2),
+              "mha_manual: shapes must be q [BH,Sq,D], k [BH,Sk,D], v [BH,Sk,D]");
+  at::DeviceGuard guard(q8.device());
+  const auto odt = out_bf16 ? at::kBFloat16 : at::kHalf;
+  at::Tensor o = at::empty(q8.sizes(), q8.options().dtype(odt));
+  at::Tensor lse = at::empty({q8.size(0), q8.size(1)}, q8.options().dtype(at::kFloat));
+  fmha_fwd_fp8_params p = {};
+  p.struct_bytes = sizeof p;
+  p.q = q8.data_ptr();
+  p.k = k8.data_ptr();
+  p.v = v8.data_ptr();
+  p.o = o.data_ptr();
+  p.lse = lse.data_ptr<float>();
+  p.bh = static_cast<int32_t>(q8.size(0));
+  p.sq = static_cast<int32_t>(q8.size(1));
+  p.sk = static_cast<int32_t>(k8.size(1));
+  p.d = static_cast<int32_t>(q8.size(2));
+  p.out_dtype = out_bf16 ? FMHA_DTYPE_BF16 : FMHA_DTYPE_F16;
+  p.scale = static_cast<float>(scale > 0 ? scale : 1.0 / std::sqrt(static_cast<double>(q8.size(2))));
+  p.descale_q = static_cast<float>(descale_q);
+  p.descale_k = static_cast<float>(descale_k);
+  p.descale_v = static_cast<float>(descale_v);
+  p.causal = is_causal ? 1 : 0;
+  MaskLayout m;
+  if (mask.has_value() && mask->defined()) {
+    m = mask_layout(*mask, o, q8.size(0), q8.size(1), k8.size(1), "mask");
+    TORCH_CHECK(m.stride_q == 0, "mha_manual: the e4m3 forward takes per-key masks ([..,1,Sk]) only");
+    p.mask = m.t.data_ptr();
+    p.mask_bh_div = m.bh_div;
+    p.mask_stride_b = m.stride_b;
+  }
+  const int rc = fmha_fwd_fp8_launch(&p, current_stream(q8));
+  TORCH_CHECK(rc == FMHA_OK, "mha_manual e4m3 forward: ", fmha_strerror(rc));
+  return std::make_tuple(o, lse);
+}
+
 // uint8 [bh,sq,sk] keep decisions (1 keep / 0 drop) for (seed, offset, p_drop) on `like`'s device.
 at::Tensor philox_keep_mask_op(const at::Tensor &like, int64_t bh, int64_t sq, int64_t sk, double p_drop,
                                  int64_t seed, int64_t offset) {
@@ -450,6 +496,8 @@ TORCH_LIBRARY(mha_manual, m) {
   m.def("fmha_bwd(Tensor dout, Tensor q, Tensor k, Tensor v, Tensor o, Tensor lse, Tensor? mask, float scale, bool "
         "is_causal, float p_drop, int seed, int offset, Tensor? kv_len=None) -> (Tensor, Tensor, Tensor)");
   m.def("fmha_philox_keep_mask(Tensor like, int bh, int sq, int sk, float p_drop, int seed, int offset) -> Tensor");
+  m.def("fmha_fwd_fp8(Tensor q8, Tensor k8, Tensor v8, float descale_q, float descale_k, float descale_v, Tensor? mask, "
+        "float scale, bool is_causal, bool out_bf16=False) -> (Tensor, Tensor)");
 }
 
 // On ROCm builds of PyTorch the CUDA dispatch key is the HIP device's key.
@@ -460,6 +508,7 @@ TORCH_LIBRARY_IMPL(mha_manual, CUDA, m) {
   m.impl("fmha_fwd", fmha_fwd);
   m.impl("fmha_bwd", fmha_bwd);
   m.impl("fmha_philox_keep_mask", philox_keep_mask_op);
+  m.impl("fmha_fwd_fp8", fmha_fwd_fp8);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) { m.doc() = "gfx950 fused multi-head attention (operators live in torch.ops.mha_manual)"; }

@@ -156,6 +156,33 @@ typedef struct fmha_fwd_params {
 int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream);
 
 /*
+ * Forward on 8-bit floating point inputs (no counterpart in the reference, which is fp16 only:
+ * fmha/fmha_manual.cpp:120).  q, k, v hold OCP e4m3 bytes (torch.float8_e4m3fn), [bh, s, d] contiguous,
+ * with one dequantisation factor per tensor (x = descale_x * x8); both products run on the fp8 matrix
+ * instructions with fp32 accumulation, the softmax is fp32, the probabilities -- unnormalised, relative to
+ * the running row maximum -- are rounded to e4m3 before the second product and the row sums are taken
+ * before that rounding:
+ *   O = descale_v * (round_e4m3(P) v8) / rowsum(P),   P = exp(scale * descale_q * descale_k * q8 k8^T + mask - rowmax)
+ * o (and the optional per-key additive mask, mask[(b / mask_bh_div) * mask_stride_b + j]) are fp16 or
+ * bf16 (out_dtype); lse is optional.  Head dim 64 or 128.  A first, untuned kernel: e4m3 carries three
+ * mantissa bits, so outputs agree with the 16-bit path to a few per cent of their magnitude, not to 2e-3.
+ */
+typedef struct fmha_fwd_fp8_params {
+  uint64_t struct_bytes; /* sizeof(fmha_fwd_fp8_params); see fmha_fwd_params */
+  const void *q, *k, *v;
+  void *o;
+  float *lse;
+  const void *mask;
+  int64_t mask_bh_div, mask_stride_b;
+  int32_t bh, sq, sk, d;
+  int32_t out_dtype; /* FMHA_DTYPE_F16 / FMHA_DTYPE_BF16 */
+  float scale, descale_q, descale_k, descale_v;
+  int32_t causal;
+} fmha_fwd_fp8_params;
+
+int fmha_fwd_fp8_launch(const fmha_fwd_fp8_params *p, void *hip_stream);
+
+/*
  * Backward (no counterpart in the reference, which has no backward kernel:
  * README.md:1).  Inputs are those of the forward plus the upstream gradient
  * `dout`, the forward output `o` and the saved `lse`; the dropout decisions are

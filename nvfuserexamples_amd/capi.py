@@ -18,7 +18,7 @@ DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
            "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides",
-           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale")
+           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale", "fmha_fwd_fp8_launch")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
 _ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
@@ -83,6 +83,18 @@ class BwdParams(_Params):
     ]
 
 
+class FwdFp8Params(_Params):
+    _fields_ = [
+        ("struct_bytes", C.c_uint64),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p), ("lse", C.c_void_p),
+        ("mask", C.c_void_p), ("mask_bh_div", C.c_int64), ("mask_stride_b", C.c_int64),
+        ("bh", C.c_int32), ("sq", C.c_int32), ("sk", C.c_int32), ("d", C.c_int32),
+        ("out_dtype", C.c_int32),
+        ("scale", C.c_float), ("descale_q", C.c_float), ("descale_k", C.c_float), ("descale_v", C.c_float),
+        ("causal", C.c_int32),
+    ]
+
+
 class FmhaError(RuntimeError):
     def __init__(self, code, msg):
         super().__init__(f"fmha error {code}: {msg}")
@@ -105,6 +117,8 @@ def lib():
         L.fmha_fwd_launch.restype = C.c_int
         L.fmha_bwd_launch.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         L.fmha_bwd_launch.restype = C.c_int
+        L.fmha_fwd_fp8_launch.argtypes = [C.POINTER(FwdFp8Params), C.c_void_p]
+        L.fmha_fwd_fp8_launch.restype = C.c_int
         L.fmha_bwd_launch_noalloc.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         L.fmha_bwd_launch_noalloc.restype = C.c_int
         L.fmha_bwd_noalloc_max_rows.argtypes = []
@@ -333,6 +347,39 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     _sync_env()
     check(lib().fmha_bwd_launch(C.byref(P), _stream_ptr()))
     return dq, dk, dv
+
+
+def fwd_fp8(q8, k8, v8, descale_q=1.0, descale_k=1.0, descale_v=1.0, mask=None, causal=False, scale=None,
+            out_dtype=None, want_lse=False):
+    """Forward on e4m3 inputs (torch.float8_e4m3fn, contiguous [bh, s, d]) on the current stream.
+    Returns (o, lse|None); o is float16 unless out_dtype says bfloat16.  mask: additive [bh|B, 1, sk] /
+    [B,1,1,sk] in o's dtype."""
+    import torch
+    out_dtype = out_dtype or torch.float16
+    for t in (q8, k8, v8):
+        if not (t.is_cuda and t.dtype == torch.float8_e4m3fn and t.dim() == 3 and t.is_contiguous()):
+            raise FmhaError(-5, "q, k, v must be contiguous [bh, s, d] float8_e4m3fn device tensors")
+    bh, sq, d = q8.shape
+    sk = k8.shape[1]
+    if k8.shape != (bh, sk, d) or v8.shape != (bh, sk, d):
+        raise FmhaError(-3, "q/k/v shapes do not agree")
+    P = FwdFp8Params()
+    o = torch.empty((bh, sq, d), dtype=out_dtype, device=q8.device)
+    lse = torch.empty((bh, sq), dtype=torch.float32, device=q8.device) if want_lse else None
+    P.q, P.k, P.v, P.o = q8.data_ptr(), k8.data_ptr(), v8.data_ptr(), o.data_ptr()
+    P.lse = lse.data_ptr() if lse is not None else None
+    P.bh, P.sq, P.sk, P.d = bh, sq, sk, d
+    P.out_dtype = F16 if out_dtype == torch.float16 else BF16
+    P.scale = float(scale) if scale is not None else d ** -0.5
+    P.descale_q, P.descale_k, P.descale_v = descale_q, descale_k, descale_v
+    P.causal = int(bool(causal))
+    if mask is not None:
+        mask, div, sb, sqs = mask_layout(mask, bh, sq, sk)
+        if mask.dtype != out_dtype or sqs != 0:
+            raise FmhaError(-5, "the e4m3 forward takes a per-key mask ([.., 1, sk]) of o's dtype")
+        P.mask, P.mask_bh_div, P.mask_stride_b = mask.data_ptr(), div, sb
+    check(lib().fmha_fwd_fp8_launch(C.byref(P), _stream_ptr()))
+    return o, lse
 
 
 def philox_keep_mask(seed, offset, p_drop, bh, sq, sk, device="cuda"):

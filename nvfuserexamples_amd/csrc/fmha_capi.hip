@@ -2,6 +2,7 @@
 // launch.  Declared in include/fmha_capi.h.  No allocation, no synchronisation.
 #include "../../include/fmha_capi.h"
 #include "fmha_launch.h"
+#include "fmha_fwd_fp8.h"
 
 #include <cmath>
 #include <cstddef>
@@ -336,6 +337,34 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
 } // namespace
 
 extern "C" {
+
+int fmha_fwd_fp8_launch(const fmha_fwd_fp8_params *caller, void *hip_stream) {
+  if (!caller) return FMHA_E_NULL;
+  if (caller->struct_bytes < offsetof(fmha_fwd_fp8_params, causal) + sizeof(int32_t)) return FMHA_E_ARG;
+  fmha_fwd_fp8_params local;
+  std::memset(&local, 0, sizeof local);
+  std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
+  const fmha_fwd_fp8_params *p = &local;
+  if (!p->q || !p->k || !p->v || !p->o) return FMHA_E_NULL;
+  if (p->out_dtype != FMHA_DTYPE_F16 && p->out_dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
+  if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;
+  if (p->d != 64 && p->d != 128) return FMHA_E_SHAPE;
+  if ((int64_t)p->sq * p->d >= (1ll << 31) || (int64_t)p->sk * p->d >= (1ll << 31)) return FMHA_E_SHAPE;
+  if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->o)) return FMHA_E_ALIGN;
+  if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return FMHA_E_ARG;
+  for (float f : {p->descale_q, p->descale_k, p->descale_v})
+    if (!(f > 0.f) || !std::isfinite(f)) return FMHA_E_ARG;
+  if (p->mask && (p->mask_bh_div < 1 || p->mask_stride_b < 0)) return FMHA_E_ARG;
+  Fp8Args a;
+  a.q = (const uint8_t *)p->q; a.k = (const uint8_t *)p->k; a.v = (const uint8_t *)p->v;
+  a.o = p->o; a.lse = p->lse;
+  a.mask = p->mask; a.mask_sb = p->mask_stride_b; a.mask_div = p->mask ? (int32_t)p->mask_bh_div : 1;
+  a.bh = p->bh; a.sq = p->sq; a.sk = p->sk;
+  a.score_scale_l2 = p->scale * p->descale_q * p->descale_k * FMHA_LOG2E;
+  a.out_scale = p->descale_v;
+  const int rc = fwd_fp8_dispatch(a, p->d, p->out_dtype == FMHA_DTYPE_BF16, p->causal != 0, (hipStream_t)hip_stream);
+  return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
+}
 
 int fmha_bwd_launch(const fmha_bwd_params *caller, void *hip_stream) { return bwd_launch_impl(caller, hip_stream, false); }
 

@@ -60,4 +60,8 @@ int bwd_dispatch_f16_d128_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s
 int bwd_dispatch_bf16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d128_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 
+// e4m3 forward (fmha_fwd_fp8.hip): 0 ok, 1 not built, 2 launch failed
+struct Fp8Args;
+int fwd_fp8_dispatch(const Fp8Args &a, int d, bool out_bf16, bool causal, hipStream_t s);
+
 } // namespace fmha

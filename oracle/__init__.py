@@ -66,7 +66,7 @@ def lib():
     return _lib
 
 
-ROUND = {None: 0, "none": 0, "fp32": 0, "fp16": 1, "half": 1, "bf16": 2}
+ROUND = {None: 0, "none": 0, "fp32": 0, "fp16": 1, "half": 1, "bf16": 2, "e4m3": 3}
 
 
 def _f32(a):
@@ -84,6 +84,13 @@ def philox4x32_10(ctr, key):
     out = np.zeros(4, dtype=np.uint32)
     lib().fmha_oracle_philox4x32_10(_ptr(c), _ptr(k), _ptr(out))
     return out
+
+
+def round_to(x, kind):
+    """Element-wise rounding of a float array to fp16 / bf16 / e4m3 (returned as float32)."""
+    x = _f32(x)
+    f = lib().fmha_oracle_round
+    return np.array([f(float(v), ROUND[kind]) for v in x.ravel()], dtype=np.float32).reshape(x.shape)
 
 
 def drop_threshold(p):

@@ -56,9 +56,25 @@ static float round_bf16(float x) {
   return r;
 }
 
+static float round_e4m3(float x) {
+  /* round-to-nearest-even to OCP e4m3 (4 exponent bits, bias 7, 3 mantissa bits, no infinities),
+   * saturating at the largest finite value 448; subnormal spacing 2^-9 below 2^-6 */
+  if (isnan(x)) return x;
+  float ax = fabsf(x);
+  if (ax >= 448.0f) return copysignf(448.0f, x);
+  if (ax < 0.015625f) return copysignf(nearbyintf(ax * 512.0f) / 512.0f, x);
+  int e;
+  frexpf(ax, &e);
+  float ulp = ldexpf(1.0f, e - 4); /* 4 significant bits */
+  float r = nearbyintf(ax / ulp) * ulp;
+  if (r > 448.0f) r = 448.0f;
+  return copysignf(r, x);
+}
+
 static float round_to(float x, int kind) {
   if (kind == 1) return round_f16(x);
   if (kind == 2) return round_bf16(x);
+  if (kind == 3) return round_e4m3(x);
   return x;
 }
 
@@ -148,7 +164,9 @@ typedef struct {
   float p_drop;      /* Philox threshold source */
   float drop_scale;  /* multiplies kept probabilities (2.0 legacy, 1/(1-p) seeded) */
   uint64_t seed, offset;
-  int32_t round_p;   /* 0: none, 1: fp16, 2: bf16 -- rounding of P before P.V (fmha_manual.cpp:87) */
+  int32_t round_p;   /* 0: none, 1: fp16, 2: bf16 -- rounding of P before P.V (fmha_manual.cpp:87);
+                      * 3: e4m3, applied to the UNNORMALISED exp(s - rowmax) with the row sum taken before
+                      * the rounding (the rounding model of the 8-bit forward, which the reference lacks) */
   int32_t round_o;   /* rounding of outputs (fmha_manual.cpp:95) */
   /* outputs (any may be NULL) */
   float *o;          /* [bh,sq,d] */
@@ -187,13 +205,19 @@ static double drop_factor(const fmha_oracle_params *p, uint32_t thr, int64_t b, 
   return 1.0;
 }
 
-/* One softmax row: fills prob[0..sk) and returns log-sum-exp. */
+/* One softmax row: fills prob[0..sk) and returns log-sum-exp; *sum_out (if given) receives
+ * sum_j exp(s_j - max), the factor between prob and the unnormalised exponentials. */
+static double softmax_row_sum(const fmha_oracle_params *p, int64_t b, int64_t i, double *prob, double *sum_out);
 static double softmax_row(const fmha_oracle_params *p, int64_t b, int64_t i, double *prob) {
+  return softmax_row_sum(p, b, i, prob, NULL);
+}
+static double softmax_row_sum(const fmha_oracle_params *p, int64_t b, int64_t i, double *prob, double *sum_out) {
   double mx = -INFINITY;
   for (int64_t j = 0; j < p->sk; ++j) {
     prob[j] = score_at(p, b, i, j);
     if (prob[j] > mx) mx = prob[j];
   }
+  if (sum_out) *sum_out = 1.0;
   if (mx == -INFINITY) { /* fully masked row: defined as all-zero probabilities */
     for (int64_t j = 0; j < p->sk; ++j) prob[j] = 0.0;
     return -INFINITY;
@@ -204,6 +228,7 @@ static double softmax_row(const fmha_oracle_params *p, int64_t b, int64_t i, dou
     sum += prob[j];
   }
   for (int64_t j = 0; j < p->sk; ++j) prob[j] /= sum;
+  if (sum_out) *sum_out = sum;
   return mx + log(sum);
 }
 
@@ -214,7 +239,8 @@ int fmha_oracle_fwd(const fmha_oracle_params *p) {
   uint32_t thr = fmha_oracle_drop_threshold(p->p_drop);
   for (int64_t b = 0; b < p->bh; ++b) {
     for (int64_t i = 0; i < p->sq; ++i) {
-      double lse = softmax_row(p, b, i, prob);
+      double rowsum = 1.0;
+      double lse = softmax_row_sum(p, b, i, prob, &rowsum);
       if (p->lse) p->lse[b * p->sq + i] = (float)lse;
       for (int64_t c = 0; c < p->d; ++c) acc[c] = 0.0;
       for (int64_t j = 0; j < p->sk; ++j) {
@@ -222,7 +248,8 @@ int fmha_oracle_fwd(const fmha_oracle_params *p) {
         double pd = pj * drop_factor(p, thr, b, i, j);
         if (p->softmax) p->softmax[(b * p->sq + i) * p->sk + j] = round_to((float)pj, p->round_o);
         if (p->dropout) p->dropout[(b * p->sq + i) * p->sk + j] = round_to((float)pd, p->round_o);
-        double w = (double)round_to((float)pd, p->round_p);
+        double w = p->round_p == 3 ? (double)round_to((float)(pd * rowsum), 3) / rowsum
+                                   : (double)round_to((float)pd, p->round_p);
         const float *vj = p->v + (b * p->sk + j) * p->d;
         for (int64_t c = 0; c < p->d; ++c) acc[c] += w * (double)vj[c];
       }

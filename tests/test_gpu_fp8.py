@@ -1,0 +1,115 @@
+"""Forward on e4m3 inputs (fmha_fwd_fp8_launch) against the CPU oracle run with the same rounding model:
+inputs are the e4m3 values themselves (exact in fp32), the unnormalised probabilities exp(s - rowmax) are
+rounded to e4m3 before the second product and the row sum is taken before that rounding.
+
+Tolerances.  e4m3 keeps three mantissa bits: every probability carries a rounding error of up to 2^-4
+relative, and WHICH way it rounds depends on the scale it is rounded at.  The kernel rounds relative to the
+running row maximum of the tile it is in, the oracle relative to the final one, so the two sets of rounding
+errors are of the same size but not the same errors; what the model predicts is the LEVEL of the error:
+   rms(O - exact) <= 1.5 * rms(model - exact) + 2^-11 max|O|     (the kernel is as accurate as the format allows)
+   max|O - exact| <= 2^-4 * max|v|   (the bound if every probability of a row rounded the same way: O is a
+                                      weighted mean of v rows whose weights are each off by at most 2^-4 relative)
+   LSE (no rounding involved) within 2e-3
+where `exact` is the oracle on the same e4m3 inputs without any rounding of the probabilities.  Where nothing
+rounds (all probabilities 1, or one key per row) the kernel must agree with the oracle to the rounding of O."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from nvfuserexamples_amd import capi
+from conftest import pad_mask, f32
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # bh, sq, sk, d, out dtype, mask, causal
+    (4, 128, 128, 64, torch.float16, None, False),
+    (4, 512, 512, 64, torch.float16, "pad", False),     # headline shape, few heads
+    (3, 100, 77, 64, torch.float16, None, False),        # ragged tiles
+    (2, 320, 320, 64, torch.float16, None, True),        # causal
+    (2, 200, 333, 128, torch.bfloat16, "pad", False),
+    (2, 257, 257, 128, torch.float16, "pad", True),
+    (2, 1, 1000, 64, torch.float16, None, False),        # decode step
+]
+
+
+def _quantise(x, amax=448.0):
+    """Per-tensor scaling into the e4m3 range; returns (e4m3 tensor, dequantisation factor)."""
+    s = float(x.abs().max()) / amax
+    return (x / s).to(torch.float8_e4m3fn), s
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,odt,mask,causal", CASES)
+def test_fp8_forward_matches_the_oracle_with_the_same_rounding(bh, sq, sk, d, odt, mask, causal):
+    g = torch.Generator().manual_seed(bh + sk)
+    std = 1.0 if d == 64 else 0.5
+    q, k, v = (torch.randn(bh, s, d, generator=g) * std for s in (sq, sk, sk))
+    q8, dq = _quantise(q)
+    k8, dk = _quantise(k)
+    v8, dv = _quantise(v)
+    m = None
+    if mask == "pad":
+        m = pad_mask(bh // 2 if bh % 2 == 0 else bh, sk, sk // 2, sk).to(odt)
+    o, lse = capi.fwd_fp8(q8.cuda(), k8.cuda(), v8.cuda(), dq, dk, dv, mask=None if m is None else m.cuda(),
+                          causal=causal, out_dtype=odt, want_lse=True)
+    torch.cuda.synchronize()
+    qf, kf, vf = (f32(t.float()) for t in (q8, k8, v8))   # the e4m3 values, exactly
+    kw = dict(mask=None if m is None else f32(m), causal=causal, scale=d ** -0.5 * dq * dk, want=("o", "lse"))
+    ref = oracle.attention(qf, kf, vf * np.float32(dv), round_p="e4m3", **kw)
+    exact = oracle.attention(qf, kf, vf * np.float32(dv), **kw)
+    got = f32(o.cpu())
+    top = np.abs(exact["o"]).max()
+    out_round = 2.0 ** -11 if odt == torch.float16 else 2.0 ** -8
+    rms = lambda x: float(np.sqrt(np.mean(np.square(x, dtype=np.float64))))
+    assert rms(got - exact["o"]) <= 1.5 * rms(ref["o"] - exact["o"]) + out_round * top
+    assert np.abs(got - exact["o"]).max() <= 2.0 ** -4 * float(np.abs(vf).max()) * dv + out_round * top
+    assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= 2e-3
+    # and the 8-bit path is a different computation from a cast of the 16-bit one: the model's rounding shows
+    assert np.abs(ref["o"] - exact["o"]).max() > 1e-4 * top
+
+
+@pytest.mark.parametrize("d,odt", [(64, torch.float16), (128, torch.bfloat16)])
+def test_fp8_forward_is_exact_where_nothing_rounds(d, odt):
+    """q = 0: every probability is 1 (an e4m3 value), O is the mean of the e4m3 values of v.  One-hot q and k
+    with a score gap of 100: one probability is 1, the others underflow to 0, O_i = v[i mod d] -- which also
+    pins the key <-> register permutation of the first product and the transposed V tile, element by element."""
+    g = torch.Generator().manual_seed(d)
+    bh, sq, sk = 3, 200, 333
+    v = torch.randn(bh, sk, d, generator=g)
+    v8 = v.to(torch.float8_e4m3fn)
+    q8 = torch.zeros(bh, sq, d).to(torch.float8_e4m3fn)
+    k8 = torch.randn(bh, sk, d, generator=g).to(torch.float8_e4m3fn)
+    o, lse = capi.fwd_fp8(q8.cuda(), k8.cuda(), v8.cuda(), descale_v=0.5, out_dtype=odt, want_lse=True)
+    want = 0.5 * v8.float().mean(1, keepdim=True).expand(bh, sq, d)
+    tol = (2.0 ** -10 if odt == torch.float16 else 2.0 ** -7) * float(want.abs().max()) + 1e-6
+    assert (o.float().cpu() - want).abs().max().item() <= tol
+    assert (lse.cpu() - np.log(sk)).abs().max().item() <= 1e-5
+    sq = sk = d                                   # one key per query matches
+    eye = torch.eye(d).expand(bh, d, d) * 16.0    # 16 * 16 * (100 / 256) = 100
+    e8 = eye.contiguous().to(torch.float8_e4m3fn)
+    vv = torch.randn(bh, sk, d, generator=g).to(torch.float8_e4m3fn)
+    o, _ = capi.fwd_fp8(e8.cuda(), e8.cuda(), vv.cuda(), scale=100.0 / 256.0, out_dtype=odt)
+    assert torch.equal(o.float().cpu(), vv.float().to(odt).float())
+
+
+def test_fp8_forward_refuses_what_it_does_not_serve():
+    x = torch.zeros(2, 64, 96, device="cuda").to(torch.float8_e4m3fn)
+    with pytest.raises(capi.FmhaError):
+        capi.fwd_fp8(x, x, x)                                   # head dim 96
+    y = torch.zeros(2, 64, 64, device="cuda").to(torch.float8_e4m3fn)
+    with pytest.raises(capi.FmhaError):
+        capi.fwd_fp8(y, y, y, descale_q=0.0)                    # a factor must be positive
+    with pytest.raises(capi.FmhaError):
+        capi.fwd_fp8(y, y, y, mask=torch.zeros(2, 64, 64, dtype=torch.float16, device="cuda"))  # per-key masks only
+
+
+def test_fp8_operator_equals_the_c_abi_call():
+    from nvfuserexamples_amd import load_ops
+    ops = load_ops()
+    g = torch.Generator().manual_seed(1)
+    q8, k8, v8 = (torch.randn(4, 160, 64, generator=g).to(torch.float8_e4m3fn).cuda() for _ in range(3))
+    m = pad_mask(2, 160, 80, 160).half().cuda()
+    o, lse = ops.fmha_fwd_fp8(q8, k8, v8, 0.5, 2.0, 1.5, m, 0.0, False)
+    o2, lse2 = capi.fwd_fp8(q8, k8, v8, 0.5, 2.0, 1.5, mask=m, want_lse=True)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)

@@ -264,3 +264,27 @@ def test_dropout_factor_keeps_the_mean(p):
     # the nominal factor 1 / (1 - p) is biased wherever 256 p is not an integer: by -0.17 % at p = 0.1 (8 sigma here)
     if p == 0.1:
         assert abs(km.mean() / (1 - p) - 1.0) > 4 * sigma
+
+
+def test_e4m3_rounding_matches_the_library_cast():
+    """The oracle's e4m3 rounding (the model of the 8-bit forward) against torch's float8_e4m3fn cast:
+    a dense sweep of the finite range, the subnormal region and the ties, bit for bit."""
+    x = torch.cat([torch.linspace(-448, 448, 60001), torch.randn(20000) * 0.01, torch.randn(20000),
+                   torch.tensor([0.0, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -9, 448.0, 447.0, 0.0155, 0.0157,
+                                 0.9375, 0.96875, 1.0625, 1.1875])])
+    want = x.to(torch.float8_e4m3fn).float().numpy()
+    got = oracle.round_to(x.numpy(), "e4m3")
+    assert np.array_equal(got, want)
+
+
+def test_e4m3_probability_model_reduces_to_the_exact_forward_when_nothing_rounds():
+    """With one key per row the unnormalised probability is exactly 1, which e4m3 holds: the 8-bit model
+    equals the unrounded forward; with more keys it differs by at most 2^-4 relative per probability."""
+    q, k, v = make_qkv(2, 9, 1, 64, seed=5)
+    a = oracle.attention(f32(q), f32(k), f32(v), round_p="e4m3")["o"]
+    b = oracle.attention(f32(q), f32(k), f32(v))["o"]
+    assert np.array_equal(a, b)
+    q, k, v = make_qkv(2, 16, 40, 64, seed=6)
+    a = oracle.attention(f32(q), f32(k), f32(v), round_p="e4m3")["o"]
+    b = oracle.attention(f32(q), f32(k), f32(v))["o"]
+    assert 0 < np.abs(a - b).max() <= 2.0 ** -4 * np.abs(f32(v)).max()
