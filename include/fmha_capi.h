@@ -68,7 +68,7 @@ enum {
   FMHA_OK = 0,
   FMHA_E_NULL = -1,        /* a required pointer is NULL */
   FMHA_E_DTYPE = -2,       /* unknown dtype */
-  FMHA_E_SHAPE = -3,       /* non-positive size or unsupported head dim (64, 128 and, folded layout only, 256 are built) */
+  FMHA_E_SHAPE = -3,       /* non-positive size or unsupported head dim (64, 128 and 256 are built) */
   FMHA_E_ALIGN = -4,       /* q/k/v/o/gradient base pointer not 16-byte aligned */
   FMHA_E_ARG = -5,         /* scale / p_drop / mask description out of range */
   FMHA_E_UNSUPPORTED = -6, /* combination not built (see fmha_strerror) */

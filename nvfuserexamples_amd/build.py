@@ -39,17 +39,12 @@ def _tus():
     """(source, object name, extra defines) for every translation unit of the library."""
     tus = [("fmha_capi.hip", "fmha_capi.o", []), ("fmha_fwd_fp8.hip", "fmha_fwd_fp8.o", [])]
     for bf in (0, 1):
-        for d in (64, 128):
+        for d in (64, 128, 256):
             for strided in (0, 1):  # folded contiguous tensors / row layouts given at run time
                 tag = f"{'bf16' if bf else 'f16'}_d{d}" + ("_strided" if strided else "")
                 defs = [f"-DFMHA_TU_BF16={bf}", f"-DFMHA_TU_D={d}", f"-DFMHA_TU_STRIDED={strided}"]
                 tus.append(("fmha_fwd.hip", f"fmha_fwd_{tag}.o", defs))
                 tus.append(("fmha_bwd.hip", f"fmha_bwd_{tag}.o", defs))
-        # head dim 256: folded layout only
-        tag = f"{'bf16' if bf else 'f16'}_d256"
-        defs = [f"-DFMHA_TU_BF16={bf}", "-DFMHA_TU_D=256", "-DFMHA_TU_STRIDED=0"]
-        tus.append(("fmha_fwd.hip", f"fmha_fwd_{tag}.o", defs))
-        tus.append(("fmha_bwd.hip", f"fmha_bwd_{tag}.o", defs))
     return tus
 
 

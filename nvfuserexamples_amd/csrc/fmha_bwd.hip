@@ -11,6 +11,12 @@
 #else
 #define FMHA_TU_SHORT 0
 #endif
+#if FMHA_TU_D == 256
+#define FMHA_TU_WIDE 1
+#include "fmha_bwd_wide.h"
+#else
+#define FMHA_TU_WIDE 0
+#endif
 
 #if FMHA_TU_BF16
 #define FMHA_TU_T __bf16
@@ -41,14 +47,24 @@ template <typename K> int set_lds(K kern, int bytes) {
 
 template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipStream_t s) {
   constexpr int kLdsQ = BwdCfg<FMHA_TU_D, bwd_dq_tile_rows<FMHA_TU_D>()>::LDS_BYTES;
+  auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP, kStrided>;
+#if FMHA_TU_WIDE
+  // head dim 256: the dK / dV work of a key block is split between two waves (fmha_bwd_wide.h; at head
+  // dims 128 and 64 the same kernel measured level with and a third slower than the one-wave kernel)
+  using CfgK = BwdWideCfg<FMHA_TU_D, MASK>;
+  constexpr int kLdsK = CfgK::LDS_BYTES;
+  constexpr int kNWK = CfgK::NW, KT = CfgK::KT;
+  auto kk = fmha_bwd_dkdv_wide_kernel<FMHA_TU_T, FMHA_TU_D, MASK, CAUSAL, DROP, kStrided>;
+#else
   using CfgK = BwdCfg<FMHA_TU_D, bwd_dkdv_tile_rows<FMHA_TU_D, CAUSAL, DROP>()>;
   constexpr int kLdsK = CfgK::LDS_BYTES + (MASK == kMaskFull ? CfgK::MASK_BYTES : 0);
-  static_assert(kLdsQ <= 160 * 1024 && kLdsK <= 160 * 1024, "tiles do not fit the LDS of a compute unit");
-  auto kq = fmha_bwd_dq_kernel<FMHA_TU_T, FMHA_TU_D, kQB, kNW, MASK, CAUSAL, DROP, kStrided>;
+  constexpr int kNWK = kNW, KT = kNW * kKB * 32;
   auto kk = fmha_bwd_dkdv_kernel<FMHA_TU_T, FMHA_TU_D, kKB, kNW, MASK, CAUSAL, DROP, kStrided>;
+#endif
+  static_assert(kLdsQ <= 160 * 1024 && kLdsK <= 160 * 1024, "tiles do not fit the LDS of a compute unit");
   static const int attr = set_lds(kq, kLdsQ) | set_lds(kk, kLdsK);
   if (attr) return 2;
-  constexpr int QT = kNW * kQB * 32, KT = kNW * kKB * 32;
+  constexpr int QT = kNW * kQB * 32;
   // dQ first: it also writes delta, which the dK/dV kernel reads (same stream => ordered)
   // causal: workgroups take pairs of tiles (see the kernels) when that leaves at least two
   // rounds of workgroups for the device
@@ -72,7 +88,7 @@ template <int MASK, bool CAUSAL, int DROP> int launch(BwdArgs &a, int pair, hipS
   a.pair = want_pair(a.ntile);
   nblk = (long long)a.bh * (a.pair ? (a.ntile + 1) / 2 : a.ntile);
   if (nblk > 0x7fffffffLL) return 2;
-  hipLaunchKernelGGL(kk, dim3((unsigned)nblk), dim3(kNW * 64), kLdsK, s, a);
+  hipLaunchKernelGGL(kk, dim3((unsigned)nblk), dim3(kNWK * 64), kLdsK, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 

@@ -63,9 +63,8 @@ struct BwdArgs {
 // mask the shorter tiles lose more to the uneven tile counts, and the dropout variant spills
 // too much, so those keep 64-row tiles at one wave per SIMD.
 template <int D> constexpr int bwd_dq_tile_rows() { return 64; }
-// (Head dim 256 -- built for coverage, not tuned -- takes the short tiles throughout: four 64-row tiles
-// of 512 bytes per row plus a mask tile would not fit the LDS.)
-template <int D, bool CAUSAL, int DROP> constexpr bool bwd_dkdv_small_tiles() { return D == 256 || (D == 128 && !CAUSAL && DROP == 0); }
+// (Head dim 256 has a dK/dV kernel of its own, fmha_bwd_wide.h.)
+template <int D, bool CAUSAL, int DROP> constexpr bool bwd_dkdv_small_tiles() { return D == 128 && !CAUSAL && DROP == 0; }
 template <int D, bool CAUSAL, int DROP> constexpr int bwd_dkdv_tile_rows() {
   return bwd_dkdv_small_tiles<D, CAUSAL, DROP>() ? 32 : 64;
 }

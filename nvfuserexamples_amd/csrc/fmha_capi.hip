@@ -99,7 +99,7 @@ const char *fmha_strerror(int code) {
   case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64, 128 or 256, and one head's rows must span less than 2^31 elements";
   case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned and their strides multiples of 8 elements";
   case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, mask_neg finite and <= 0, known mask/drop kind)";
-  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart; head dim 256 takes folded tensors only)";
+  case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart)";
   case FMHA_E_LAUNCH: return "HIP launch failed";
   case FMHA_E_SCRATCH: return "fmha_bwd_launch_noalloc: bh * sq exceeds fmha_bwd_noalloc_max_rows() (the library's own scratch holds one float per query row); use fmha_bwd_launch with caller-provided delta";
   default: return "unknown error code";
@@ -235,7 +235,6 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if ((mrc = make_row_map(a.mo, p->heads, p->o_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
   if (strided && (saving || p->drop_kind == FMHA_DROP_TENSOR)) return FMHA_E_UNSUPPORTED;
-  if (p->d == 256 && strided) return FMHA_E_UNSUPPORTED; // head dim 256: folded layout only
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
@@ -291,9 +290,9 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   int rc;
   if (strided) {
     if (p->dtype == FMHA_DTYPE_F16)
-      rc = p->d == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : fwd_dispatch_f16_d128_strided(a, v, s);
+      rc = p->d == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : p->d == 128 ? fwd_dispatch_f16_d128_strided(a, v, s) : fwd_dispatch_f16_d256_strided(a, v, s);
     else
-      rc = p->d == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : fwd_dispatch_bf16_d128_strided(a, v, s);
+      rc = p->d == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : p->d == 128 ? fwd_dispatch_bf16_d128_strided(a, v, s) : fwd_dispatch_bf16_d256_strided(a, v, s);
   } else if (p->dtype == FMHA_DTYPE_F16)
     rc = p->d == 64 ? fwd_dispatch_f16_d64(a, v, s) : p->d == 128 ? fwd_dispatch_f16_d128(a, v, s) : fwd_dispatch_f16_d256(a, v, s);
   else
@@ -462,7 +461,6 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   if ((mrc = make_row_map(a.mdq, p->heads, p->dq_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mdk, p->heads, p->dk_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mdv, p->heads, p->dv_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
-  if (p->d == 256 && strided) return FMHA_E_UNSUPPORTED; // head dim 256: folded layout only
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
 
   BwdVariant v;
@@ -491,9 +489,9 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   int rc;
   if (strided) {
     if (p->dtype == FMHA_DTYPE_F16)
-      rc = p->d == 64 ? bwd_dispatch_f16_d64_strided(a, v, s) : bwd_dispatch_f16_d128_strided(a, v, s);
+      rc = p->d == 64 ? bwd_dispatch_f16_d64_strided(a, v, s) : p->d == 128 ? bwd_dispatch_f16_d128_strided(a, v, s) : bwd_dispatch_f16_d256_strided(a, v, s);
     else
-      rc = p->d == 64 ? bwd_dispatch_bf16_d64_strided(a, v, s) : bwd_dispatch_bf16_d128_strided(a, v, s);
+      rc = p->d == 64 ? bwd_dispatch_bf16_d64_strided(a, v, s) : p->d == 128 ? bwd_dispatch_bf16_d128_strided(a, v, s) : bwd_dispatch_bf16_d256_strided(a, v, s);
   } else if (p->dtype == FMHA_DTYPE_F16)
     rc = p->d == 64 ? bwd_dispatch_f16_d64(a, v, s) : p->d == 128 ? bwd_dispatch_f16_d128(a, v, s) : bwd_dispatch_f16_d256(a, v, s);
   else

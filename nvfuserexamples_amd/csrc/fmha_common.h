@@ -65,6 +65,8 @@ union Pack8 {
 template <typename T> FMHA_DEV typename Elem<T>::v8 as_v8(u32x4 u);
 template <> FMHA_DEV f16x8 as_v8<_Float16>(u32x4 u) { Pack16 p; p.u = u; return p.h; }
 template <> FMHA_DEV bf16x8 as_v8<__bf16>(u32x4 u) { Pack16 p; p.u = u; return p.b; }
+FMHA_DEV u32x4 as_u32x4(f16x8 v) { Pack16 p; p.h = v; return p.u; }
+FMHA_DEV u32x4 as_u32x4(bf16x8 v) { Pack16 p; p.b = v; return p.u; }
 
 template <typename T> FMHA_DEV typename Elem<T>::v4 as_v4(u32x2 u);
 template <> FMHA_DEV f16x4 as_v4<_Float16>(u32x2 u) { Pack8 p; p.u = u; return p.h; }

@@ -42,7 +42,7 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
   // the save pass (and tensor dropout at head dim 128) runs on the plain loop; everything else is
   // software-pipelined
   auto kern = [] {
-    if constexpr (!kPipe) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP>;
+    if constexpr (!kPipe) return fmha_fwd_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP, kStrided && FMHA_TU_D == 256>;
     else return fmha_fwd_pipe_kernel<FMHA_TU_T, FMHA_TU_D, QB, kNW, MASK, CAUSAL, DROP, kStrided>;
   }();
   // once per kernel: allow the dynamic LDS size, and for the persistent kernel find how many
@@ -170,7 +170,7 @@ template <int MASK, bool CAUSAL> int plain_by_drop(FwdArgs &a, int drop, hipStre
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
-  if (v.qb == 2 || v.short_keys || v.save_split || v.stream || kStrided) return 1;
+  if (v.qb == 2 || v.short_keys || v.save_split || v.stream || (kStrided && v.drop == 2)) return 1;
   if (v.mask == kMaskPerKey)
     return v.causal ? plain_by_drop<kMaskPerKey, true>(a, v.drop, s) : plain_by_drop<kMaskPerKey, false>(a, v.drop, s);
   if (v.mask == kMaskFull)

@@ -108,9 +108,9 @@ template <> FMHA_DEV float dot2_ones<__bf16>(bf16x8 v, int pair, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(x, one, acc, false);
 }
 
-template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP>
+template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED = false>
 __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
-  using RW = Rows<false, D>; // this kernel serves the reference's operators: folded contiguous tensors only
+  using RW = Rows<STRIDED, D>; // (run-time row layouts are built at head dim 256 only, where this is the only forward)
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;

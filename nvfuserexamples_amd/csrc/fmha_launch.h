@@ -26,8 +26,10 @@ int fwd_dispatch_f16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d64(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d128(FwdArgs &a, const FwdVariant &v, hipStream_t s);
-int fwd_dispatch_f16_d256(FwdArgs &a, const FwdVariant &v, hipStream_t s);  // folded layout only
+int fwd_dispatch_f16_d256(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d256(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_f16_d256_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
+int fwd_dispatch_bf16_d256_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d64_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_f16_d128_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
 int fwd_dispatch_bf16_d64_strided(FwdArgs &a, const FwdVariant &v, hipStream_t s);
@@ -53,8 +55,10 @@ int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);
-int bwd_dispatch_f16_d256(BwdArgs &a, const BwdVariant &v, hipStream_t s);  // folded layout only
+int bwd_dispatch_f16_d256(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d256(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_f16_d256_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
+int bwd_dispatch_bf16_d256_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d128_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_bf16_d64_strided(BwdArgs &a, const BwdVariant &v, hipStream_t s);

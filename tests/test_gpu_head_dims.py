@@ -77,12 +77,12 @@ def test_autograd_and_strided_views_at_head_dim_96():
 
 
 def test_head_dims_beyond_the_built_ones_are_refused():
-    """Beyond 256, and head dim 256 in anything but the folded layout: an error, never a wrong answer."""
+    """Beyond 256: an error, never a wrong answer."""
     from nvfuserexamples_amd import load_ops
     ops = load_ops()
     x = torch.zeros(2, 64, 264, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError):
         ops.fmha_fwd(x, x, x, None, 0.0, False, 0.0, 0, 0)
-    w = torch.zeros(2, 64, 2, 256, dtype=torch.float16, device="cuda").transpose(1, 2)  # [B,H,S,D] view of [B,S,H,D]
+    w = torch.zeros(2, 64, 2, 264, dtype=torch.float16, device="cuda").transpose(1, 2)  # [B,H,S,D] view of [B,S,H,D]
     with pytest.raises(capi.FmhaError):
         capi.fwd(w, w, w)

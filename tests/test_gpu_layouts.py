@@ -47,13 +47,16 @@ CASES = [
     # short heads: the one-launch backward reads and writes the same layouts
     (3, 4, 197, 197, 64, "fp16", False, 0.1, False, True),    # ViT-B/16 length, packed projection
     (2, 3, 100, 128, 64, "bf16", True, 0.0, True, False),
+    # head dim 256: plain forward loop, dQ kernel and the wave-pair dK/dV kernel on run-time row layouts
+    (2, 2, 200, 264, 256, "fp16", False, 0.1, True, False),
+    (2, 2, 192, 192, 256, "bf16", True, 0.0, False, True),
 ]
 
 
 @pytest.mark.parametrize("b,h,sq,sk,d,dtype,causal,p,masked,packed", CASES)
 def test_strided_layouts_match_oracle_and_folded_path(b, h, sq, sk, d, dtype, causal, p, masked, packed):
     bh = b * h
-    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std=0.5 if d == 128 else 1.0, dtype=dtype, with_dout=True)
+    q, k, v, do = make_qkv(bh, sq, sk, d, seed=bh + sk, std={64: 1.0, 128: 0.5, 256: 0.35}[d], dtype=dtype, with_dout=True)
     kw, okw = dict(causal=causal), dict(causal=causal)
     if p:
         kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=11, offset=5)
