@@ -284,13 +284,14 @@ void set_mask_and_dropout(P &p, MaskLayout &m, const c10::optional<at::Tensor> &
 }
 
 
-// Head dims the kernels are not built for (anything but 64, 128 and 256) run zero-padded to
-// the next built size: zero columns add nothing to Q.K^T, the padded columns of V give zero columns
-// of O (and zero columns of dO leave the other gradients untouched), so results are those of the
-// original head dim.  Costs a copy of every operand and the arithmetic on the padding.
+// The C ABI takes any head dim that is a multiple of 8 up to 256 as it is (rows of whole 16-byte pieces:
+// the kernels run at the next built size, 64 / 128 / 256, and neither read nor write the missing columns).
+// Only head dims that are not multiples of 8 are zero-padded here, to the next multiple: zero columns add
+// nothing to Q.K^T, the padded columns of V give zero columns of O (and zero columns of dO leave the other
+// gradients untouched), so results are those of the original head dim, at the cost of a copy of every operand.
 int64_t padded_head_dim(int64_t d) {
   TORCH_CHECK(d >= 1 && d <= 256, "mha_manual: head dim must be in [1, 256], got ", d);
-  return d <= 64 ? 64 : d <= 128 ? 128 : 256;
+  return (d + 7) / 8 * 8;
 }
 at::Tensor pad_head_dim(const at::Tensor &x, int64_t to) {
   return at::constant_pad_nd(x, {0, to - x.size(-1)}, 0);
@@ -298,7 +299,7 @@ at::Tensor pad_head_dim(const at::Tensor &x, int64_t to) {
 
 // q, k, v: [B*H,S,D] contiguous (the reference's layout) or [B,H,S,D] views of any batch / head /
 // row strides (e.g. x.view(B,S,H,D).transpose(1,2), or a slice of a packed QKV projection), read
-// in place (D = 64 or 128, folded tensors also 256; other head dims are padded, see above).  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
+// in place (any D up to 256; see above).  scale <= 0 selects 1/sqrt(D).  Dropout decisions come from Philox4x32-10 keyed by
 // (seed, offset); p_drop == 0 disables dropout.  Returns (O, LSE fp32): O in q's shape and
 // dimension order, LSE [B*H,Sq] or [B,H,Sq].
 std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tensor &k_, const at::Tensor &v_,

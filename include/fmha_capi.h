@@ -68,7 +68,7 @@ enum {
   FMHA_OK = 0,
   FMHA_E_NULL = -1,        /* a required pointer is NULL */
   FMHA_E_DTYPE = -2,       /* unknown dtype */
-  FMHA_E_SHAPE = -3,       /* non-positive size or unsupported head dim (64, 128 and 256 are built) */
+  FMHA_E_SHAPE = -3,       /* non-positive size or unsupported head dim (multiples of 8 up to 256) */
   FMHA_E_ALIGN = -4,       /* q/k/v/o/gradient base pointer not 16-byte aligned */
   FMHA_E_ARG = -5,         /* scale / p_drop / mask description out of range */
   FMHA_E_UNSUPPORTED = -6, /* combination not built (see fmha_strerror) */
@@ -84,6 +84,10 @@ enum {
  *   mask[(b / mask_bh_div) * mask_stride_b + i * mask_stride_q + j]
  * so [bh,sq,sk] is (div 1, stride_b sq*sk, stride_q sk), a [B,1,1,sk] padding mask
  * over bh = B*H is (div H, stride_b sk, stride_q 0).
+ * Head dim d: 64 in the reference (fmha_manual.cpp:24-29); here any multiple of 8 up to 256.  The kernels
+ * are built for 64, 128 and 256; other head dims run at the next of those and neither read nor write
+ * the columns a row does not have (no padded copies), on the run-time-layout code path.  Tensor dropout
+ * and the saved outputs exist at d = 64, 128 and 256 only.
  * Computes  O = (dropout(softmax(scale * q k^T + mask_term [+ causal]))) v
  * with fp32 accumulation and fp32 softmax, the probabilities rounded to the
  * element type before the second product (fmha_manual.cpp:87) and O rounded on

@@ -54,6 +54,7 @@ struct BwdArgs {
   int32_t kv_div;
   RowMap mq, mk, mv, mo, mdo, mdq, mdk, mdv; // row layouts (mk.ss == mv.ss)
   float *ws; // one-pass kernel only: fp32 partial dQ sums between key chunks
+  int32_t dcols; // elements per row that exist (<= the kernel's head dim; run-time layouts only)
 };
 
 // BT: rows per LDS tile (keys in the dQ kernel, queries in the dK/dV kernel).  The dK/dV kernel
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(NW * 64)
     u32x4 tq[KS], td[KS], to[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const size_t col = ks * 16 + h * 8;
+      const size_t col = ks * 16 + h * 8 < RW::cols(a) ? ks * 16 + h * 8 : 0; // padding chunks are zeroed below
       tq[ks] = *(const u32x4 *)(Qb + (size_t)qc * RW::ss(a.mq) + col);
       td[ks] = *(const u32x4 *)(dOb + (size_t)qc * RW::ss(a.mdo) + col);
       to[ks] = *(const u32x4 *)(Ob + (size_t)qc * RW::ss(a.mo) + col);
@@ -222,8 +223,9 @@ __global__ __launch_bounds__(NW * 64)
     float dsum = 0.f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const v8 qraw = as_v8<T>(tq[ks]);
-      const v8 doraw = as_v8<T>(td[ks]);
+      const bool live = ks * 16 + h * 8 < RW::cols(a);
+      const v8 qraw = as_v8<T>(chunk_or_zero(tq[ks], live));
+      const v8 doraw = as_v8<T>(chunk_or_zero(td[ks], live));
       const v8 ov = as_v8<T>(to[ks]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -289,8 +291,8 @@ __global__ __launch_bounds__(NW * 64)
   tcopy.init(tid, RW::ss(a.mk)); // K and V rows are equally far apart
   auto dma_kv = [&](int kt) {
     const uint32_t dst = lds_base + (uint32_t)(kt & 1) * 2 * TILEB;
-    tcopy.issue(Kb, kt * BK, kclamp, dst, tid);
-    tcopy.issue(Vb, kt * BK, kclamp, dst + TILEB, tid);
+    tcopy.issue(Kb, kt * BK, kclamp, dst, tid, RW::cols(a));
+    tcopy.issue(Vb, kt * BK, kclamp, dst + TILEB, tid, RW::cols(a));
   };
   T mraw = (T)0.f;
   bool mvalid = false;
@@ -474,7 +476,7 @@ __global__ __launch_bounds__(NW * 64)
     const int q = q0w + qb * 32 + ql;
     if (q < a.sq) {
 #pragma unroll
-      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQb + (size_t)q * RW::ss(a.mdq) + db * 32, dq[qb][db], a.scale, h);
+      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dQb + (size_t)q * RW::ss(a.mdq) + db * 32, dq[qb][db], a.scale, h, RW::cols(a) - db * 32);
     }
   }
   __syncthreads(); // the next pass refills the tiles
@@ -543,7 +545,7 @@ __global__ __launch_bounds__(NW * 64)
     u32x4 tk[KS], tv[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const size_t col = ks * 16 + h * 8;
+      const size_t col = ks * 16 + h * 8 < RW::cols(a) ? ks * 16 + h * 8 : 0; // padding chunks are zeroed below
       tk[ks] = *(const u32x4 *)(Kb + (size_t)kc * RW::ss(a.mk) + col);
       tv[ks] = *(const u32x4 *)(Vb + (size_t)kc * RW::ss(a.mv) + col);
     }
@@ -551,8 +553,9 @@ __global__ __launch_bounds__(NW * 64)
     if (MASK == kMaskPerKey) mraw_key = ((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + kc];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const v8 kraw = as_v8<T>(tk[ks]);
-      const v8 vraw = as_v8<T>(tv[ks]);
+      const bool live = ks * 16 + h * 8 < RW::cols(a);
+      const v8 kraw = as_v8<T>(chunk_or_zero(tk[ks], live));
+      const v8 vraw = as_v8<T>(chunk_or_zero(tv[ks], live));
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         kreg[kb][ks][j] = (T)((float)kraw[j] * a.scale_l2);
@@ -612,8 +615,8 @@ __global__ __launch_bounds__(NW * 64)
   tcopy_do.init(tid, RW::ss(a.mdo));
   auto dma_qdo = [&](int qt) {
     const uint32_t dst = lds_base + (uint32_t)(qt & 1) * 2 * TILEB;
-    tcopy.issue(Qb, qt * BQ, a.sq, dst, tid);
-    tcopy_do.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid);
+    tcopy.issue(Qb, qt * BQ, a.sq, dst, tid, RW::cols(a));
+    tcopy_do.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid, RW::cols(a));
   };
   float lraw = 0.f, draw = 0.f;
   bool qvalid = false;
@@ -834,8 +837,8 @@ __global__ __launch_bounds__(NW * 64)
     if (key < a.sk) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        store_acc_block_row<T>(dKb + (size_t)key * RW::ss(a.mdk) + db * 32, dk[kb][db], a.scale, h);
-        store_acc_block_row<T>(dVb + (size_t)key * RW::ss(a.mdv) + db * 32, dv[kb][db], 1.f, h);
+        store_acc_block_row<T>(dKb + (size_t)key * RW::ss(a.mdk) + db * 32, dk[kb][db], a.scale, h, RW::cols(a) - db * 32);
+        store_acc_block_row<T>(dVb + (size_t)key * RW::ss(a.mdv) + db * 32, dv[kb][db], 1.f, h, RW::cols(a) - db * 32);
       }
     }
   }

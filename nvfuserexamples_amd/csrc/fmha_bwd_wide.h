@@ -92,12 +92,13 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
       const int kc = key < a.sk ? key : a.sk - 1; // keys past the end re-read the last row; their mask term is "-inf"
       u32x4 raw[KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) raw[ks] = *(const u32x4 *)(src + (size_t)kc * ss + ks * 16 + h * 8);
+      for (int ks = 0; ks < KS; ++ks) // (padding chunks of a narrower head: chunk 0 instead, zeroed below)
+        raw[ks] = *(const u32x4 *)(src + (size_t)kc * ss + (ks * 16 + h * 8 < RW::cols(a) ? ks * 16 + h * 8 : 0));
       T mraw_key = (T)0.f;
       if (MASK == kMaskPerKey) mraw_key = ((const T *)a.mask)[(size_t)(bh / a.mask_div) * a.mask_sb + kc];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const v8 r = as_v8<T>(raw[ks]);
+        const v8 r = as_v8<T>(chunk_or_zero(raw[ks], ks * 16 + h * 8 < RW::cols(a)));
 #pragma unroll
         for (int j = 0; j < 8; ++j) oreg[ks][j] = (T)((float)r[j] * f);
       }
@@ -141,8 +142,8 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
     tcopy_do.init(tid, RW::ss(a.mdo));
     auto dma_qdo = [&](int qt) {
       const uint32_t dst = lds_base + (uint32_t)(qt & 1) * 2 * TILEB;
-      tcopy.issue(Qb, qt * BQ, a.sq, dst, tid);
-      tcopy_do.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid);
+      tcopy.issue(Qb, qt * BQ, a.sq, dst, tid, RW::cols(a));
+      tcopy_do.issue(dOb, qt * BQ, a.sq, dst + TILEB, tid, RW::cols(a));
     };
     float lraw = 0.f, draw = 0.f;
     bool qvalid = false;
@@ -348,7 +349,7 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
                      : (T *)a.dv + RW::head(a.mdv, bh, a.sk) + (size_t)key * RW::ss(a.mdv);
       const float f = roleG ? a.scale : 1.f;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dst + db * 32, acc[db], f, h);
+      for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dst + db * 32, acc[db], f, h, RW::cols(a) - db * 32);
     }
     __syncthreads(); // the next pass refills the tiles
   }

@@ -96,7 +96,7 @@ const char *fmha_strerror(int code) {
   case FMHA_OK: return "ok";
   case FMHA_E_NULL: return "a required pointer is NULL";
   case FMHA_E_DTYPE: return "unknown dtype (0 = fp16, 1 = bf16)";
-  case FMHA_E_SHAPE: return "bad shape: sizes must be positive, head dim 64, 128 or 256, and one head's rows must span less than 2^31 elements";
+  case FMHA_E_SHAPE: return "bad shape: sizes must be positive, the head dim a multiple of 8 up to 256, and one head's rows must span less than 2^31 elements";
   case FMHA_E_ALIGN: return "q/k/v/o/gradient pointers must be 16-byte aligned and their strides multiples of 8 elements";
   case FMHA_E_ARG: return "argument out of range (struct_bytes must be set to the size of the parameter struct, scale must be > 0, p_drop in [0,1), mask_bh_div >= 1, mask_neg finite and <= 0, known mask/drop kind)";
   case FMHA_E_UNSUPPORTED: return "combination not built (tensor dropout / saved intermediates exclude causal, Philox, valid key counts and strided layouts; the backward takes Philox dropout only; k and v rows must be equally far apart)";
@@ -126,6 +126,10 @@ int fmha_philox_keep_mask(uint64_t seed, uint64_t offset, float p_drop, int32_t 
 }
 
 } // extern "C"
+
+// Head dims the kernels are built for: 64, 128 and 256.  Anything else (a multiple of 8) runs on the next
+// built size through the run-time-layout kernels, which never read or write the missing columns.
+static int built_head_dim(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 
 // Row layout of one tensor from the caller's (heads, strides); see fmha_capi.h.  `strided` is
 // set when the layout is not the folded contiguous one (it is never cleared).
@@ -166,7 +170,8 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (!p->q || !p->k || !p->v || !p->o) return FMHA_E_NULL;
   if (p->dtype != FMHA_DTYPE_F16 && p->dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
   if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;
-  if (p->d != 64 && p->d != 128 && p->d != 256) return FMHA_E_SHAPE;
+  if (p->d < 8 || p->d > 256 || (p->d & 7) != 0) return FMHA_E_SHAPE;
+  const int D = built_head_dim(p->d); // the kernels' head dim; rows of fewer elements count as zero-padded
   if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->o)) return FMHA_E_ALIGN;
   if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return FMHA_E_ARG;
   if (p->mask_kind < FMHA_MASK_NONE || p->mask_kind > FMHA_MASK_KEEP01) return FMHA_E_ARG;
@@ -233,6 +238,8 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if ((mrc = make_row_map(a.mk, p->heads, p->k_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mv, p->heads, p->v_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mo, p->heads, p->o_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+  if (p->d != D) strided = true;
+  a.dcols = p->d;
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
   if (strided && (saving || p->drop_kind == FMHA_DROP_TENSOR)) return FMHA_E_UNSUPPORTED;
 
@@ -290,13 +297,13 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   int rc;
   if (strided) {
     if (p->dtype == FMHA_DTYPE_F16)
-      rc = p->d == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : p->d == 128 ? fwd_dispatch_f16_d128_strided(a, v, s) : fwd_dispatch_f16_d256_strided(a, v, s);
+      rc = D == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_f16_d128_strided(a, v, s) : fwd_dispatch_f16_d256_strided(a, v, s);
     else
-      rc = p->d == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : p->d == 128 ? fwd_dispatch_bf16_d128_strided(a, v, s) : fwd_dispatch_bf16_d256_strided(a, v, s);
+      rc = D == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_bf16_d128_strided(a, v, s) : fwd_dispatch_bf16_d256_strided(a, v, s);
   } else if (p->dtype == FMHA_DTYPE_F16)
-    rc = p->d == 64 ? fwd_dispatch_f16_d64(a, v, s) : p->d == 128 ? fwd_dispatch_f16_d128(a, v, s) : fwd_dispatch_f16_d256(a, v, s);
+    rc = D == 64 ? fwd_dispatch_f16_d64(a, v, s) : D == 128 ? fwd_dispatch_f16_d128(a, v, s) : fwd_dispatch_f16_d256(a, v, s);
   else
-    rc = p->d == 64 ? fwd_dispatch_bf16_d64(a, v, s) : p->d == 128 ? fwd_dispatch_bf16_d128(a, v, s) : fwd_dispatch_bf16_d256(a, v, s);
+    rc = D == 64 ? fwd_dispatch_bf16_d64(a, v, s) : D == 128 ? fwd_dispatch_bf16_d128(a, v, s) : fwd_dispatch_bf16_d256(a, v, s);
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 
@@ -401,7 +408,8 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
     return FMHA_E_NULL;
   if (p->dtype != FMHA_DTYPE_F16 && p->dtype != FMHA_DTYPE_BF16) return FMHA_E_DTYPE;
   if (p->bh <= 0 || p->sq <= 0 || p->sk <= 0) return FMHA_E_SHAPE;
-  if (p->d != 64 && p->d != 128 && p->d != 256) return FMHA_E_SHAPE;
+  if (p->d < 8 || p->d > 256 || (p->d & 7) != 0) return FMHA_E_SHAPE;
+  const int D = built_head_dim(p->d); // the kernels' head dim; rows of fewer elements count as zero-padded
   if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->o) || !aligned16(p->dout) ||
       !aligned16(p->dq) || !aligned16(p->dk) || !aligned16(p->dv))
     return FMHA_E_ALIGN;
@@ -461,6 +469,8 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   if ((mrc = make_row_map(a.mdq, p->heads, p->dq_stride, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mdk, p->heads, p->dk_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
   if ((mrc = make_row_map(a.mdv, p->heads, p->dv_stride, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+  if (p->d != D) strided = true;
+  a.dcols = p->d;
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
 
   BwdVariant v;
@@ -489,13 +499,13 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   int rc;
   if (strided) {
     if (p->dtype == FMHA_DTYPE_F16)
-      rc = p->d == 64 ? bwd_dispatch_f16_d64_strided(a, v, s) : p->d == 128 ? bwd_dispatch_f16_d128_strided(a, v, s) : bwd_dispatch_f16_d256_strided(a, v, s);
+      rc = D == 64 ? bwd_dispatch_f16_d64_strided(a, v, s) : D == 128 ? bwd_dispatch_f16_d128_strided(a, v, s) : bwd_dispatch_f16_d256_strided(a, v, s);
     else
-      rc = p->d == 64 ? bwd_dispatch_bf16_d64_strided(a, v, s) : p->d == 128 ? bwd_dispatch_bf16_d128_strided(a, v, s) : bwd_dispatch_bf16_d256_strided(a, v, s);
+      rc = D == 64 ? bwd_dispatch_bf16_d64_strided(a, v, s) : D == 128 ? bwd_dispatch_bf16_d128_strided(a, v, s) : bwd_dispatch_bf16_d256_strided(a, v, s);
   } else if (p->dtype == FMHA_DTYPE_F16)
-    rc = p->d == 64 ? bwd_dispatch_f16_d64(a, v, s) : p->d == 128 ? bwd_dispatch_f16_d128(a, v, s) : bwd_dispatch_f16_d256(a, v, s);
+    rc = D == 64 ? bwd_dispatch_f16_d64(a, v, s) : D == 128 ? bwd_dispatch_f16_d128(a, v, s) : bwd_dispatch_f16_d256(a, v, s);
   else
-    rc = p->d == 64 ? bwd_dispatch_bf16_d64(a, v, s) : p->d == 128 ? bwd_dispatch_bf16_d128(a, v, s) : bwd_dispatch_bf16_d256(a, v, s);
+    rc = D == 64 ? bwd_dispatch_bf16_d64(a, v, s) : D == 128 ? bwd_dispatch_bf16_d128(a, v, s) : bwd_dispatch_bf16_d256(a, v, s);
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 

@@ -164,7 +164,22 @@ struct RowMap {
 // Kernels are built twice: for the folded contiguous layout, whose strides are compile-time
 // constants (the row map is not read at all), and for row maps given at run time, which cost a
 // few per cent in scalar address arithmetic and registers.
+// Head dims between the built ones: a tensor's rows hold `dcols` < D elements (a multiple of 8: whole 16-byte
+// chunks) and the kernels behave as if the rows were padded with zeros up to D -- chunks past dcols are
+// never read (register loads fetch chunk 0 instead and are zeroed afterwards; direct copies to LDS take
+// their 16 bytes from g_zero_chunk) and never written.  Zero columns change neither Q.K^T nor the kept
+// columns of O and of the gradients.  Only the run-time-layout kernels know about it (rows dv elements
+// apart are a run-time row stride anyway); in the others cols() is the constant D and all of it folds away.
+static __device__ __attribute__((aligned(64))) uint32_t g_zero_chunk[16];
+FMHA_DEV u32x4 chunk_or_zero(u32x4 v, bool live) {
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  return live ? v : z;
+}
 template <bool STRIDED, int D> struct Rows {
+  template <typename A> static FMHA_DEV int cols(const A &a) {
+    if constexpr (STRIDED) return a.dcols;
+    else return D;
+  }
   static FMHA_DEV size_t head(const RowMap &m, int bh, int rows) {
     if constexpr (STRIDED) return m.head(bh);
     else return (size_t)bh * (size_t)rows * D;
@@ -200,8 +215,21 @@ template <typename T, int D, int BT, int NT> struct TileCopy {
   }
   // base: row 0 of the head; lds_tile: LDS byte address of the destination tile; tid: the caller's
   // index among the NT threads
-  FMHA_DEV void issue(const T *base, int row0, int rend, uint32_t lds_tile, int tid) const {
+  // dv: elements a row really has (chunks past them come from g_zero_chunk)
+  FMHA_DEV void issue(const T *base, int row0, int rend, uint32_t lds_tile, int tid, int dv = D) const {
     const uint32_t wave_dst = lds_tile + (uint32_t)(tid >> 6) * 1024u;
+    if (dv < D) { // wave-uniform
+#pragma unroll
+      for (int i = 0; i < CPT; ++i) {
+        int row, col;
+        slot(tid + i * NT, row, col);
+        int r = row0 + row;
+        r = r < rend ? r : rend - 1;
+        const T *src = col * 8 < dv ? base + ((uint32_t)r * ss + (uint32_t)(col * 8)) : (const T *)g_zero_chunk;
+        dma_global_to_lds_b128(src, wave_dst + (uint32_t)(i * NT * 16));
+      }
+      return;
+    }
     if (row0 + BT <= rend) { // wave-uniform: a full tile needs no per-lane address arithmetic
       const T *tb = base + (uint32_t)row0 * ss;
 #pragma unroll
@@ -273,7 +301,8 @@ FMHA_DEV float xhalf_sum(float x) {
 // pieces between the two half-waves (v_permlane32_swap) gives each lane 16 contiguous bytes --
 // lane h = 0 the first half of a 32-byte group, lane h = 1 the second -- so the same data leaves
 // in half as many, twice as large, writes.  dst: the lane's row; the block starts at column 0.
-template <typename T> FMHA_DEV void store_acc_block_row(T *dst_row, const f32x16 &acc, float scale, int h) {
+// ncol: columns of this block that exist in the destination row (a multiple of 8).
+template <typename T> FMHA_DEV void store_acc_block_row(T *dst_row, const f32x16 &acc, float scale, int h, int ncol = 32) {
 #pragma unroll
   for (int gp = 0; gp < 2; ++gp) {
     typename Elem<T>::v4 x, y; // pieces g = 2gp and g = 2gp + 1
@@ -294,7 +323,7 @@ template <typename T> FMHA_DEV void store_acc_block_row(T *dst_row, const f32x16
     auto r0 = __builtin_amdgcn_permlane32_swap((int)px.u.x, (int)py.u.x, false, false);
     auto r1 = __builtin_amdgcn_permlane32_swap((int)px.u.y, (int)py.u.y, false, false);
     const u32x4 both = {(uint32_t)r0[0], (uint32_t)r1[0], (uint32_t)r0[1], (uint32_t)r1[1]};
-    *(u32x4 *)(dst_row + 16 * gp + 8 * h) = both;
+    if (16 * gp + 8 * h < ncol) *(u32x4 *)(dst_row + 16 * gp + 8 * h) = both;
   }
 }
 

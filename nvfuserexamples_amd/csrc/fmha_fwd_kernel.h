@@ -66,6 +66,7 @@ struct FwdArgs {
   int32_t kv_div;
   unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
   RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
+  int32_t dcols;         // elements per row that exist (<= the kernel's head dim; run-time layouts only)
   // Balanced dealing of a per-key mask's rows over the persistent workgroups (pipelined kernel; set
   // by its launch code, 0 rows = off).  It applies when every workgroup has the same number of items
   // (2 to 4), one per round, and a round's items of one mask row (bal_ipr = heads per row x query
@@ -160,8 +161,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     for (int ks = 0; ks < KS; ++ks) {
       // rows past the end re-read the last row (never stored); unconditional loads do not stall on each other
       const int qc = q < a.sq ? q : a.sq - 1;
-      const u32x4 t = *(const u32x4 *)(Qb + (size_t)qc * RW::ss(a.mq) + ks * 16 + h * 8);
-      const v8 raw = as_v8<T>(t);
+      const bool live = ks * 16 + h * 8 < RW::cols(a);
+      const u32x4 t = *(const u32x4 *)(Qb + (size_t)qc * RW::ss(a.mq) + (live ? ks * 16 + h * 8 : 0));
+      const v8 raw = as_v8<T>(chunk_or_zero(t, live));
 #pragma unroll
       for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
     }
@@ -196,8 +198,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       // meets finite values of V (unconditional loads do not stall on each other)
       int kr = k0 + row;
       kr = kr < a.sk ? kr : a.sk - 1;
-      kst[i] = *(const u32x4 *)(Kb + (size_t)kr * RW::ss(a.mk) + col * 8);
-      vst[i] = *(const u32x4 *)(Vb + (size_t)kr * RW::ss(a.mv) + col * 8);
+      const int cc = col * 8 < RW::cols(a) ? col * 8 : 0; // padding chunks: zeroed when they are written to LDS
+      kst[i] = *(const u32x4 *)(Kb + (size_t)kr * RW::ss(a.mk) + cc);
+      vst[i] = *(const u32x4 *)(Vb + (size_t)kr * RW::ss(a.mv) + cc);
     }
     {
       const int kr = k0 + (tid & (BK - 1));
@@ -212,8 +215,9 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     for (int i = 0; i < CPT; ++i) {
       const int c = tid + i * NT;
       const int row = c / CPR, col = c % CPR;
-      *(u32x4 *)(kd + row * ROWB + col * 16) = kst[i];
-      *(u32x4 *)(vd + row * ROWB + col * 16) = vst[i];
+      const bool live = col * 8 < RW::cols(a);
+      *(u32x4 *)(kd + row * ROWB + col * 16) = chunk_or_zero(kst[i], live);
+      *(u32x4 *)(vd + row * ROWB + col * 16) = chunk_or_zero(vst[i], live);
     }
     if (tid < BK) {
       // extra contraction step, A side: (1, mask_hi, mask_lo, 1, 0 ...); keys past the end get
@@ -535,7 +539,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
           v4 t;
 #pragma unroll
           for (int i = 0; i < 4; ++i) t[i] = (T)(o[qb][db][4 * g + i] * inv);
-          *(v4 *)(Ob + (size_t)q * RW::ss(a.mo) + db * 32 + 8 * g + 4 * h) = t;
+          if (db * 32 + 8 * g + 4 * h < RW::cols(a)) *(v4 *)(Ob + (size_t)q * RW::ss(a.mo) + db * 32 + 8 * g + 4 * h) = t;
         }
       // the constant part of a full mask's term entered the product rounded to T; the
       // difference cancels in O but belongs in the log-sum-exp

@@ -295,7 +295,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   TileCopy<T, D, BK, NT> tcopy;
   tcopy.init(tid, RW::ss(a.mk)); // K and V rows are equally far apart
   auto dma_tile = [&](const T *base, int kend, int tile, uint32_t area_off) {
-    tcopy.issue(base, tile * BK, kend > 0 ? kend : 1, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid);
+    tcopy.issue(base, tile * BK, kend > 0 ? kend : 1, lds_base + area_off + (uint32_t)(tile & 1) * TILEB, tid, RW::cols(a));
   };
   // K tile u of the stream that runs from the current item on into the next one (u may reach
   // past the current item's last tile; nkt2 is even, so the stage parity carries over)
@@ -319,8 +319,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     for (int qb = 0; qb < QB; ++qb) {
       const T *row = q_row(it, qb);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        dma_global_to_lds_b128(row + ks * 16, lds_base + C::LDS_BYTES + (uint32_t)((qb * KS + ks) * NT * 16) + wave_dst);
+      for (int ks = 0; ks < KS; ++ks) // (chunks past a narrower head's end come from the zero chunk)
+        dma_global_to_lds_b128(ks * 16 + h * 8 < RW::cols(a) ? row + ks * 16 : (const T *)g_zero_chunk,
+                               lds_base + C::LDS_BYTES + (uint32_t)((qb * KS + ks) * NT * 16) + wave_dst);
     }
   };
 
@@ -943,7 +944,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
         const T *row = q_row(cur, qb);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const v8 raw = as_v8<T>(*(const u32x4 *)(row + ks * 16));
+          const bool live = ks * 16 + h * 8 < RW::cols(a);
+          const v8 raw = as_v8<T>(chunk_or_zero(*(const u32x4 *)(live ? row + ks * 16 : row), live));
 #pragma unroll
           for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
         }
@@ -1007,7 +1009,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
       if (q < a.sq) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * RW::ss(a.mo) + db * 32, o[qb][db], inv, h);
+        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * RW::ss(a.mo) + db * 32, o[qb][db], inv, h, RW::cols(a) - db * 32);
         const float cfix = (MASK == kMaskFull) ? a.mask_b - (float)(T)a.mask_b : 0.f;
         if (a.lse && h == 0)
           a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + cfix + fast_log2(lt)) * FMHA_LN2 : NEG_INF;

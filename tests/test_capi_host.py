@@ -55,7 +55,8 @@ def _valid_params():
     (lambda P: setattr(P, "struct_bytes", 0), -5),                    # the struct must carry its size
     (lambda P: setattr(P, "struct_bytes", 64), -5),                   # ... at least up to the first release's fields
     (lambda P: setattr(P, "dtype", 7), -2),
-    (lambda P: setattr(P, "d", 80), -3),
+    (lambda P: setattr(P, "d", 84), -3),                              # head dims: multiples of 8 ...
+    (lambda P: setattr(P, "d", 264), -3),                             # ... up to 256
     (lambda P: setattr(P, "sq", 0), -3),
     (lambda P: setattr(P, "k", 0x1008), -4),
     (lambda P: setattr(P, "scale", 0.0), -5),

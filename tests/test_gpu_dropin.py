@@ -51,6 +51,17 @@ def test_train_ops_like_reference_test(ops):
     assert (saved[2].float() - dr_ref).abs().max().item() <= 2e-3
 
 
+def test_inference_op_at_a_narrower_head(ops):
+    """The reference's operator exists at head dim 64 only (fmha/fmha_manual.cpp:24-29); here narrower rows of
+    whole 16-byte pieces run as they are, scaled by 1/sqrt(d): the reference's 1/8 (fmha/fmha_manual.cpp:68) at d = 64."""
+    q, k, v, amask, _ = _inputs(5)
+    q, k, v = (t[:, :, :48].contiguous() for t in (q, k, v))
+    fused = ops.fmha_nvfuser(q, k, v, amask)
+    ctx = eager.infer_mha(q, k, v, amask)
+    assert fused.shape == q.shape
+    assert (ctx.float() - fused.float()).abs().max().item() <= 2e-3
+
+
 def test_general_ops_roundtrip(ops):
     q, k, v, _, _ = _inputs(2)
     o, lse = ops.fmha_fwd(q, k, v, None, 0.0, False, 0.0, 0, 0)
@@ -63,8 +74,8 @@ def test_general_ops_roundtrip(ops):
 
 def test_errors_surface_as_runtime_errors(ops):
     q, k, v, m, _ = _inputs(3)
-    with pytest.raises(RuntimeError):
-        ops.fmha_nvfuser(q[:, :, :48].contiguous(), k[:, :, :48].contiguous(), v[:, :, :48].contiguous(), m)
+    with pytest.raises(RuntimeError):   # rows must be whole 16-byte pieces
+        ops.fmha_nvfuser(q[:, :, :44].contiguous(), k[:, :, :44].contiguous(), v[:, :, :44].contiguous(), m)
     with pytest.raises(RuntimeError):
         ops.fmha_nvfuser(q, k, v, m[:, :, :64])
     with pytest.raises(RuntimeError):
