@@ -16,6 +16,7 @@
 // at run time, so the ops are stateless and re-entrant.
 #include <ATen/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <torch/csrc/autograd/custom_function.h>
 #include <torch/extension.h>
 
 #include <algorithm>
@@ -487,6 +488,56 @@ at::Tensor philox_keep_mask_op(const at::Tensor &like, int64_t bh, int64_t sq, i
   return out;
 }
 
+// Autograd formula of fmha_fwd (the reference registers none: fmha/fmha_manual.cpp:1240-1250, its perf runs
+// are under no_grad): O is differentiable in q, k and v; the row log-sum-exp, the mask and the key counts
+// are not.  Nothing of size S x S is kept for the backward: it recomputes P from the saved LSE and
+// regenerates the dropout decisions from the same (seed, offset).
+class FmhaFunction : public torch::autograd::Function<FmhaFunction> {
+ public:
+  static torch::autograd::variable_list forward(torch::autograd::AutogradContext *ctx, const at::Tensor &q,
+                                                const at::Tensor &k, const at::Tensor &v,
+                                                const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
+                                                double p_drop, int64_t seed, int64_t offset,
+                                                const c10::optional<at::Tensor> &kv_len) {
+    at::AutoDispatchBelowADInplaceOrView below;
+    auto [o, lse] = fmha_fwd(q, k, v, mask, scale, is_causal, p_drop, seed, offset, kv_len);
+    const bool has_mask = mask.has_value() && mask->defined(), has_len = kv_len.has_value() && kv_len->defined();
+    ctx->save_for_backward({q, k, v, o, lse, has_mask ? *mask : at::empty({0}, q.options()),
+                            has_len ? *kv_len : at::empty({0}, q.options().dtype(at::kInt))});
+    ctx->saved_data["has_mask"] = has_mask;
+    ctx->saved_data["has_len"] = has_len;
+    ctx->saved_data["scale"] = scale;
+    ctx->saved_data["is_causal"] = is_causal;
+    ctx->saved_data["p_drop"] = p_drop;
+    ctx->saved_data["seed"] = seed;
+    ctx->saved_data["offset"] = offset;
+    ctx->mark_non_differentiable({lse});
+    return {o, lse};
+  }
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext *ctx,
+                                                 torch::autograd::variable_list grads) {
+    const auto saved = ctx->get_saved_variables();
+    const at::Tensor &q = saved[0], &k = saved[1], &v = saved[2], &o = saved[3], &lse = saved[4];
+    const at::Tensor dout = grads[0].defined() ? grads[0] : at::zeros_like(o);
+    c10::optional<at::Tensor> mask, kv_len;
+    if (ctx->saved_data["has_mask"].toBool()) mask = saved[5];
+    if (ctx->saved_data["has_len"].toBool()) kv_len = saved[6];
+    auto [dq, dk, dv] = fmha_bwd(dout, q, k, v, o, lse, mask, ctx->saved_data["scale"].toDouble(),
+                                 ctx->saved_data["is_causal"].toBool(), ctx->saved_data["p_drop"].toDouble(),
+                                 ctx->saved_data["seed"].toInt(), ctx->saved_data["offset"].toInt(), kv_len);
+    at::Tensor none;
+    return {dq, dk, dv, none, none, none, none, none, none, none};
+  }
+};
+
+std::tuple<at::Tensor, at::Tensor> fmha_fwd_autograd(const at::Tensor &q, const at::Tensor &k, const at::Tensor &v,
+                                                     const c10::optional<at::Tensor> &mask, double scale,
+                                                     bool is_causal, double p_drop, int64_t seed, int64_t offset,
+                                                     const c10::optional<at::Tensor> &kv_len) {
+  auto r = FmhaFunction::apply(q, k, v, mask, scale, is_causal, p_drop, seed, offset, kv_len);
+  return std::make_tuple(r[0], r[1]);
+}
+
 TORCH_LIBRARY(mha_manual, m) {
   m.def("fmha_nvfuser(Tensor input, Tensor qk, Tensor v, Tensor amask) -> Tensor");
   m.def("fmha_train_nvfuser(Tensor input, Tensor qk, Tensor v, Tensor pad_mask, Tensor dropout_mask) -> Tensor");
@@ -511,5 +562,8 @@ TORCH_LIBRARY_IMPL(mha_manual, CUDA, m) {
   m.impl("fmha_philox_keep_mask", philox_keep_mask_op);
   m.impl("fmha_fwd_fp8", fmha_fwd_fp8);
 }
+
+// fmha_fwd is differentiable by itself; the other operators stay without a formula, like the reference's.
+TORCH_LIBRARY_IMPL(mha_manual, Autograd, m) { m.impl("fmha_fwd", fmha_fwd_autograd); }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) { m.doc() = "gfx950 fused multi-head attention (operators live in torch.ops.mha_manual)"; }

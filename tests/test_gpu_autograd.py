@@ -37,3 +37,23 @@ def test_autograd_wrapper_matches_eager_autograd(causal, p):
     assert (o.float() - oe).abs().max().item() <= 2e-3
     for a, b in ((qa.grad, qe.grad), (ka.grad, ke.grad), (va.grad, ve.grad)):
         assert (a.float() - b).abs().max().item() <= 1e-2 * b.abs().max().item()
+
+
+def test_the_operator_itself_is_differentiable():
+    """torch.ops.mha_manual.fmha_fwd carries its autograd formula in C++ (Autograd dispatch key): no Python
+    wrapper is needed, the row log-sum-exp is marked non-differentiable, and under no_grad nothing is recorded."""
+    from nvfuserexamples_amd import load_ops
+    from nvfuserexamples_amd import capi
+    ops = load_ops()
+    bh, s, d = 4, 160, 64
+    q, k, v, do = (t.cuda() for t in make_qkv(bh, s, s, d, seed=9, with_dout=True))
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o, lse = ops.fmha_fwd(qa, ka, va, None, 0.0, True, 0.1, 3, 1)
+    assert o.requires_grad and not lse.requires_grad
+    o.backward(do)
+    dq, dk, dv = capi.bwd(do, q, k, v, o.detach(), lse, causal=True, drop_kind=capi.DROP_PHILOX, p_drop=0.1, seed=3, offset=1)
+    torch.cuda.synchronize()
+    assert torch.equal(qa.grad, dq) and torch.equal(ka.grad, dk) and torch.equal(va.grad, dv)
+    with torch.no_grad():
+        o2, _ = ops.fmha_fwd(qa, ka, va, None, 0.0, True, 0.1, 3, 1)
+    assert not o2.requires_grad and torch.equal(o2, o.detach())
