@@ -40,8 +40,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
-# rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) of the headline forward kernel, bytes per launch
-MEASURED_TRAFFIC_BYTES = int((82105 + 32768) * 1024)
+# HBM bytes per launch of the headline forward kernel with every key tile visited, as counted by rocprofv3
+# (FETCH_SIZE 49 329.3 x 2.000 + WRITE_SIZE 32 768.0 x 1.000 KiB, the factors from 256 MiB copies in the same
+# runs: profiles/fmha_fwd_pipe_kernel_B32H16S512D64_f16.md).  A counter reading of the build as profiled,
+# not something this script can measure; the algorithmic figure is computed beside it.
+MEASURED_TRAFFIC_BYTES = int((98658.6 + 32768.0) * 1024)
 
 B, H, S, D = 32, 16, 512, 64
 
@@ -449,6 +452,63 @@ def fp8_leg(torch, capi, L, stream, steps, warmup):
             "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)}
 
 
+def profile_leg(torch, capi, L, stream, args):
+    """`--profile LEG`: nothing but LEG's launches, `--steps` times after `--warmup`, for a run under
+    `rocprofv3` (kernel trace or counters) in which every dispatch of a kernel belongs to one workload.
+    Prints a one-line note instead of the benchmark line."""
+    leg = args.profile
+    steps = []
+    keep = []
+    if leg in ("fwd", "fwd_trim", "train", "train_one_pass"):
+        train = leg.startswith("train")
+        sets = make_inputs(torch, capi, args.sets, seed=1 if train else 0, train=train)
+        flags = 0 if leg == "fwd_trim" else capi.FLAG_NO_MASK_TRIM
+        F = [fwd_params(capi, t, train=train, flags=flags) for t in sets]
+        steps.append(lambda i: L.fmha_fwd_launch(C.byref(F[i % len(F)]), stream))
+        keep += [sets, F]
+        if train:
+            Bp = [bwd_params(capi, t, flags=flags) for t in sets]
+            if leg == "train_one_pass":
+                need = int(L.fmha_bwd_workspace_bytes(B * H, S, S, D))
+                ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+                for P in Bp:
+                    P.flags, P.workspace, P.workspace_bytes = flags | capi.FLAG_BWD_ONE_PASS, ws.data_ptr(), need
+                keep.append(ws)
+            steps.append(lambda i: L.fmha_bwd_launch(C.byref(Bp[i % len(Bp)]), stream))
+            keep.append(Bp)
+    elif leg in ("c4", "c5", "d256"):
+        b, h, s, d, dt, causal, p, std = {"c4": (4, 16, 2048, 64, torch.float16, False, 0.1, 1.0),
+                                          "c5": (16, 32, 1024, 128, torch.bfloat16, True, 0.0, 0.5),
+                                          "d256": (8, 16, 2048, 256, torch.float16, False, 0.0, 0.35)}[leg]
+        g = torch.Generator().manual_seed(11)
+        q, k, v, do = ((torch.randn(b * h, s, d, generator=g) * std).to(dt).cuda() for _ in range(4))
+        kw = dict(causal=causal)
+        if p:
+            kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=0x1234, offset=0)
+        o, lse = capi.fwd(q, k, v, want_lse=True, **kw)[:2]
+        grads = tuple(torch.empty_like(q) for _ in range(3))
+        delta = torch.empty_like(lse)
+        steps.append(lambda i: capi.fwd(q, k, v, want_lse=True, out=o, **kw))
+        steps.append(lambda i: capi.bwd(do, q, k, v, o, lse, grads=grads, delta=delta, **kw))
+    elif leg == "fp8":
+        g = torch.Generator().manual_seed(21)
+        q8, k8, v8 = (torch.randn(B * H, S, D, generator=g).to(torch.float8_e4m3fn).cuda() for _ in range(3))
+        mask = torch.zeros(B, 1, 1, S)
+        for b_, n_ in enumerate(torch.randint(S // 2, S + 1, (B,), generator=g).tolist()):
+            mask[b_, 0, 0, n_:] = -10000.0
+        mask = mask.half().cuda()
+        steps.append(lambda i: capi.fwd_fp8(q8, k8, v8, mask=mask, scale=0.125))
+    else:
+        print(f"bench.py: unknown --profile leg {leg!r}", file=sys.stderr)
+        return 2
+    for i in range(args.warmup + args.steps):
+        for st in steps:
+            st(i)
+    torch.cuda.synchronize()
+    print(json.dumps({"profile_leg": leg, "steps": args.steps, "warmup": args.warmup}))
+    return 0
+
+
 def torch_sdpa_context(torch, steps, warmup):
     """For scale only: PyTorch's own fused attention (torch.nn.functional.scaled_dot_product_attention,
     whichever backend it selects) on the same GPU at the headline shape, [B,H,S,D] fp16 tensors -- the
@@ -586,6 +646,9 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: under `rocprofv3 --pmc FETCH_SIZE` "
                          "(or WRITE_SIZE) its known traffic calibrates the counter for the attention kernels")
+    ap.add_argument("--profile", metavar="LEG", default=None,
+                    help="run only LEG's launches (fwd, fwd_trim, train, train_one_pass, c4, c5, d256, fp8) and no "
+                         "timing: for rocprofv3 runs in which every dispatch of a kernel is the same workload")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; attention shards over batch*heads without "
@@ -608,6 +671,8 @@ def main():
             dst.copy_(src)   # reads 256 MiB, writes 256 MiB per launch
         torch.cuda.synchronize()
         del src, dst
+    if args.profile:
+        return profile_leg(torch, capi, L, stream, args)
 
     # ---- forward (headline): every key tile of the dense shape is visited (FMHA_FLAG_NO_MASK_TRIM), so the
     # flops that are counted are flops that are executed; the library's default (tiles under the hard-masked
