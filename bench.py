@@ -420,8 +420,8 @@ def config_leg(torch, capi, L, stream, steps, warmup, b, h, s, d, dtype, causal,
 
 
 def fp8_leg(torch, capi, L, stream, steps, warmup):
-    """The e4m3 forward (a separate operator, first untuned kernel) at the headline shape with the same padding
-    masks: time and TFLOP/s against the dense fp8 MFMA peak.  Never part of `value`."""
+    """The e4m3 forward (a separate operator) at the headline shape with the same padding masks: time and
+    TFLOP/s against the dense fp8 MFMA peak.  Never part of `value`."""
     g = torch.Generator().manual_seed(21)
     sets = []
     for _ in range(4):

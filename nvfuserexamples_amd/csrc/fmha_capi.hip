@@ -367,6 +367,7 @@ int fmha_fwd_fp8_launch(const fmha_fwd_fp8_params *caller, void *hip_stream) {
   a.mask = p->mask; a.mask_sb = p->mask_stride_b; a.mask_div = p->mask ? (int32_t)p->mask_bh_div : 1;
   a.bh = p->bh; a.sq = p->sq; a.sk = p->sk;
   a.score_scale_l2 = p->scale * p->descale_q * p->descale_k * FMHA_LOG2E;
+  a.inv_score_scale_l2 = 1.f / a.score_scale_l2;
   a.out_scale = p->descale_v;
   const int rc = fwd_fp8_dispatch(a, p->d, p->out_dtype == FMHA_DTYPE_BF16, p->causal != 0, (hipStream_t)hip_stream);
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);

@@ -165,8 +165,11 @@ typedef struct {
   float drop_scale;  /* multiplies kept probabilities (2.0 legacy, 1/(1-p) seeded) */
   uint64_t seed, offset;
   int32_t round_p;   /* 0: none, 1: fp16, 2: bf16 -- rounding of P before P.V (fmha_manual.cpp:87);
-                      * 3: e4m3, applied to the UNNORMALISED exp(s - rowmax) with the row sum taken before
-                      * the rounding (the rounding model of the 8-bit forward, which the reference lacks) */
+                      * 3: e4m3, the rounding model of the 8-bit forward (which the reference lacks): applied to
+                      * the UNNORMALISED 2^(y - M), y the score in log2 units and M = ceil(max_j y_j), an integer,
+                      * so that any other integer reference gives the same rounded values up to a power of two;
+                      * the weights are the rounded values over THEIR sum (a convex combination: a row with one
+                      * dominant key reproduces that key's value exactly); the LSE stays unrounded */
   int32_t round_o;   /* rounding of outputs (fmha_manual.cpp:95) */
   /* outputs (any may be NULL) */
   float *o;          /* [bh,sq,d] */
@@ -243,12 +246,20 @@ int fmha_oracle_fwd(const fmha_oracle_params *p) {
       double lse = softmax_row_sum(p, b, i, prob, &rowsum);
       if (p->lse) p->lse[b * p->sq + i] = (float)lse;
       for (int64_t c = 0; c < p->d; ++c) acc[c] = 0.0;
+      double e4_factor = 1.0, e4_den = 1.0;
+      if (p->round_p == 3 && lse > -INFINITY) {
+        const double yl2 = (lse - log(rowsum)) * 1.4426950408889634; /* row maximum in log2 units */
+        e4_factor = rowsum * exp2(yl2 - ceil(yl2));
+        e4_den = 0.0;
+        for (int64_t j = 0; j < p->sk; ++j) e4_den += (double)round_to((float)(prob[j] * e4_factor), 3);
+        if (e4_den == 0.0) e4_den = 1.0;
+      }
       for (int64_t j = 0; j < p->sk; ++j) {
         double pj = prob[j];
         double pd = pj * drop_factor(p, thr, b, i, j);
         if (p->softmax) p->softmax[(b * p->sq + i) * p->sk + j] = round_to((float)pj, p->round_o);
         if (p->dropout) p->dropout[(b * p->sq + i) * p->sk + j] = round_to((float)pd, p->round_o);
-        double w = p->round_p == 3 ? (double)round_to((float)(pd * rowsum), 3) / rowsum
+        double w = p->round_p == 3 ? (double)round_to((float)(pd * e4_factor), 3) / e4_den
                                    : (double)round_to((float)pd, p->round_p);
         const float *vj = p->v + (b * p->sk + j) * p->d;
         for (int64_t c = 0; c < p->d; ++c) acc[c] += w * (double)vj[c];

@@ -1,17 +1,22 @@
 """Forward on e4m3 inputs (fmha_fwd_fp8_launch) against the CPU oracle run with the same rounding model:
-inputs are the e4m3 values themselves (exact in fp32), the unnormalised probabilities exp(s - rowmax) are
-rounded to e4m3 before the second product and the row sum is taken before that rounding.
+inputs are the e4m3 values themselves (exact in fp32); the unnormalised probabilities 2^(y - M), y the score in
+log2 units and M an INTEGER reference exponent near the row maximum, are rounded to e4m3 before the second
+product, and O is that product over the sum of the ROUNDED probabilities.
 
-Tolerances.  e4m3 keeps three mantissa bits: every probability carries a rounding error of up to 2^-4
-relative, and WHICH way it rounds depends on the scale it is rounded at.  The kernel rounds relative to the
-running row maximum of the tile it is in, the oracle relative to the final one, so the two sets of rounding
-errors are of the same size but not the same errors; what the model predicts is the LEVEL of the error:
-   rms(O - exact) <= 1.5 * rms(model - exact) + 2^-11 max|O|     (the kernel is as accurate as the format allows)
-   max|O - exact| <= 2^-4 * max|v|   (the bound if every probability of a row rounded the same way: O is a
-                                      weighted mean of v rows whose weights are each off by at most 2^-4 relative)
-   LSE (no rounding involved) within 2e-3
+Tolerances.  e4m3 keeps three mantissa bits: every probability carries a rounding error of up to 2^-4 relative.
+Because the reference exponent is an integer, the kernel (whose reference is set by the first tile of a row and
+raised lazily) and the oracle (ceil of the row maximum) round the same values up to an exact power of two, so
+they round them the same way -- except where a score sits within fp32 rounding of a tie between two e4m3
+values, or deep in the subnormal range, which moves single weights by one e4m3 step:
+   99.9 % of |O - model| <= 2e-3 * max|v| + rounding of O, all of it <= 2^-4 * max|v|
+                                    (kernel and model compute the same thing; a flipped tie in a row of few keys
+                                     moves that row by one e4m3 step of one weight)
+   rms(O - exact) <= 1.5 * rms(model - exact) + 2^-11 max|O|   (and that thing is as accurate as the format allows)
+   max|O - exact| <= 2^-3 * max|v|   (the bound if every probability of a row rounded one way and their sum the other)
+   LSE (accumulated from the unrounded probabilities) within 2e-3
 where `exact` is the oracle on the same e4m3 inputs without any rounding of the probabilities.  Where nothing
-rounds (all probabilities 1, or one key per row) the kernel must agree with the oracle to the rounding of O."""
+rounds (all probabilities equal, one key per row, one dominant key) the kernel must agree with the oracle to the
+rounding of O."""
 import numpy as np
 import pytest
 import torch
@@ -62,8 +67,12 @@ def test_fp8_forward_matches_the_oracle_with_the_same_rounding(bh, sq, sk, d, od
     top = np.abs(exact["o"]).max()
     out_round = 2.0 ** -11 if odt == torch.float16 else 2.0 ** -8
     rms = lambda x: float(np.sqrt(np.mean(np.square(x, dtype=np.float64))))
+    dev = np.abs(got - ref["o"])
+    vmax = float(np.abs(vf).max()) * dv
+    assert np.quantile(dev, 0.999) <= 2e-3 * vmax + out_round * top
+    assert dev.max() <= 2.0 ** -4 * vmax + out_round * top
     assert rms(got - exact["o"]) <= 1.5 * rms(ref["o"] - exact["o"]) + out_round * top
-    assert np.abs(got - exact["o"]).max() <= 2.0 ** -4 * float(np.abs(vf).max()) * dv + out_round * top
+    assert np.abs(got - exact["o"]).max() <= 2.0 ** -3 * float(np.abs(vf).max()) * dv + out_round * top
     assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= 2e-3
     # and the 8-bit path is a different computation from a cast of the 16-bit one: the model's rounding shows
     assert np.abs(ref["o"] - exact["o"]).max() > 1e-4 * top

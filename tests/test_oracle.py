@@ -278,13 +278,34 @@ def test_e4m3_rounding_matches_the_library_cast():
 
 
 def test_e4m3_probability_model_reduces_to_the_exact_forward_when_nothing_rounds():
-    """With one key per row the unnormalised probability is exactly 1, which e4m3 holds: the 8-bit model
-    equals the unrounded forward; with more keys it differs by at most 2^-4 relative per probability."""
+    """With one key per row the weight is P~ / P~ = 1 whatever the rounding did: the 8-bit model equals the
+    unrounded forward.  The same holds for a row with one dominant key (the others underflow e4m3).  With more
+    keys it differs, by at most 2^-4 relative per probability and as much again for their sum."""
     q, k, v = make_qkv(2, 9, 1, 64, seed=5)
     a = oracle.attention(f32(q), f32(k), f32(v), round_p="e4m3")["o"]
     b = oracle.attention(f32(q), f32(k), f32(v))["o"]
     assert np.array_equal(a, b)
+    eye = np.eye(16, dtype=np.float32)[None] * 10.0           # q_i . k_j = 100 [i == j]: gaps of 100 / 4 nats
+    vv = f32(make_qkv(1, 16, 16, 16, seed=7)[2])
+    a = oracle.attention(eye, eye, vv, round_p="e4m3", scale=0.25)["o"]
+    assert np.array_equal(a, vv)
     q, k, v = make_qkv(2, 16, 40, 64, seed=6)
     a = oracle.attention(f32(q), f32(k), f32(v), round_p="e4m3")["o"]
     b = oracle.attention(f32(q), f32(k), f32(v))["o"]
-    assert 0 < np.abs(a - b).max() <= 2.0 ** -4 * np.abs(f32(v)).max()
+    assert 0 < np.abs(a - b).max() <= 2.0 ** -3 * np.abs(f32(v)).max()
+
+
+def test_e4m3_probability_model_against_a_restatement_on_the_library_cast():
+    """The model, restated with torch's own float8_e4m3fn cast as the rounding: P~ = e4m3(2^(y - ceil(max y))) with
+    y the scores in log2 units, O = P~ v / sum P~.  Any integer reference gives the same weights except in the
+    subnormal range (below 2^-6, where e4m3 rounds on a fixed grid of 2^-9): with the reference 3 lower, values are
+    8 times larger (still far below 448) and only probabilities below 2^-6 of the row maximum may round differently,
+    each by at most 2^-10 of it."""
+    q, k, v = (f32(t) for t in make_qkv(3, 20, 50, 32, seed=8))
+    got = oracle.attention(q, k, v, round_p="e4m3")["o"]
+    y = torch.from_numpy(q).double() @ torch.from_numpy(k).double().transpose(1, 2) * float(np.float32(32 ** -0.5)) * np.log2(np.e)
+    for shift, tol in ((0.0, 1e-6), (3.0, 50 * 2.0 ** -10)):
+        m = torch.ceil(y.amax(-1, keepdim=True)) - shift
+        pt = torch.exp2(y - m).float().to(torch.float8_e4m3fn).double()
+        want = (pt @ torch.from_numpy(v).double()) / pt.sum(-1, keepdim=True)
+        assert np.abs(got - want.numpy()).max() <= tol * np.abs(v).max()
