@@ -164,12 +164,15 @@ int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream);
  * fmha/fmha_manual.cpp:120).  q, k, v hold OCP e4m3 bytes (torch.float8_e4m3fn), [bh, s, d] contiguous,
  * with one dequantisation factor per tensor (x = descale_x * x8); both products run on the fp8 matrix
  * instructions with fp32 accumulation, the softmax is fp32, the probabilities -- unnormalised, relative to
- * the running row maximum -- are rounded to e4m3 before the second product and the row sums are taken
- * before that rounding:
- *   O = descale_v * (round_e4m3(P) v8) / rowsum(P),   P = exp(scale * descale_q * descale_k * q8 k8^T + mask - rowmax)
+ * an INTEGER reference exponent M (in log2 units) near the row maximum, so that the rounding does not depend
+ * on the order in which the keys are visited -- are rounded to e4m3 before the second product, and O is that
+ * product over the sum of the ROUNDED probabilities (a convex combination of the value rows):
+ *   P~ = round_e4m3(2^(y - M)),  y = log2(e) * (scale * descale_q * descale_k * q8 k8^T + mask),  M = ceil(rowmax y)
+ *   O  = descale_v * (P~ v8) / rowsum(P~)
  * o (and the optional per-key additive mask, mask[(b / mask_bh_div) * mask_stride_b + j]) are fp16 or
- * bf16 (out_dtype); lse is optional.  Head dim 64 or 128.  A first, untuned kernel: e4m3 carries three
- * mantissa bits, so outputs agree with the 16-bit path to a few per cent of their magnitude, not to 2e-3.
+ * bf16 (out_dtype); lse (optional) is the exact row log-sum-exp, from the unrounded probabilities.  Head dim 64
+ * or 128.  e4m3 carries three mantissa bits, so outputs agree with the 16-bit path to a few per cent of their
+ * magnitude, not to 2e-3.
  */
 typedef struct fmha_fwd_fp8_params {
   uint64_t struct_bytes; /* sizeof(fmha_fwd_fp8_params); see fmha_fwd_params */
