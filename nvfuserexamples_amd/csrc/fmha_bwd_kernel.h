@@ -793,7 +793,10 @@ __global__ __launch_bounds__(NW * 64)
             if (DROP == 1) {
               const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
               gv = keep ? gv : -Dl[t];
-              pzv = keep ? p * a.drop_scale : 0.f;
+              pzv = keep ? p : 0.f; // (drop_scale multiplies dV once, on store)
+              // keep the selection in fp32: left alone the compiler converts first and selects halves, which costs
+              // a conversion per element and a pack per pair instead of one packed conversion per pair
+              asm volatile("" : "+v"(pzv));
             }
             pz[4 * gq + t] = pzv;
             ds[4 * gq + t] = p * gv;
@@ -838,7 +841,7 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         store_acc_block_row<T>(dKb + (size_t)key * RW::ss(a.mdk) + db * 32, dk[kb][db], a.scale, h, RW::cols(a) - db * 32);
-        store_acc_block_row<T>(dVb + (size_t)key * RW::ss(a.mdv) + db * 32, dv[kb][db], 1.f, h, RW::cols(a) - db * 32);
+        store_acc_block_row<T>(dVb + (size_t)key * RW::ss(a.mdv) + db * 32, dv[kb][db], DROP == 1 ? a.drop_scale : 1.f, h, RW::cols(a) - db * 32);
       }
     }
   }

@@ -230,7 +230,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
             if (DROP == 1) {
               const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
               gv = keep ? fmaf(g[4 * gq + t], a.drop_scale, -Dl[t]) : -Dl[t];
-              pz = keep ? p * a.drop_scale : 0.f;
+              pz = keep ? p : 0.f; // (drop_scale multiplies dV once, on store)
             }
             pfrag[gq >> 1][4 * (gq & 1) + t] = (T)pz;
             dsfrag[gq >> 1][4 * (gq & 1) + t] = (T)(p * gv);
@@ -251,7 +251,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         store_acc_block_row<T>(dKr + db * 32, dk[db], a.scale, h);
-        store_acc_block_row<T>(dVr + db * 32, dv[db], 1.f, h);
+        store_acc_block_row<T>(dVr + db * 32, dv[db], DROP == 1 ? a.drop_scale : 1.f, h);
       }
     }
   }

@@ -289,7 +289,7 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
               const int r = 4 * gq + t;
               if (DROP == 1) {
                 const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
-                frag[sb][r >> 3][r & 7] = (T)(keep ? p * a.drop_scale : 0.f);
+                frag[sb][r >> 3][r & 7] = (T)(keep ? p : 0.f); // (drop_scale multiplies dV once, on store)
                 send[r >> 3][r & 7] = (T)(keep ? p : -p);
               } else {
                 frag[sb][r >> 3][r & 7] = (T)p;
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
     if (key < a.sk) {
       T *dst = roleG ? (T *)a.dk + RW::head(a.mdk, bh, a.sk) + (size_t)key * RW::ss(a.mdk)
                      : (T *)a.dv + RW::head(a.mdv, bh, a.sk) + (size_t)key * RW::ss(a.mdv);
-      const float f = roleG ? a.scale : 1.f;
+      const float f = roleG ? a.scale : (DROP == 1 ? a.drop_scale : 1.f);
 #pragma unroll
       for (int db = 0; db < DB; ++db) store_acc_block_row<T>(dst + db * 32, acc[db], f, h, RW::cols(a) - db * 32);
     }
