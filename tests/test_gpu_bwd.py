@@ -104,6 +104,7 @@ def test_backward_properties_at_headline_shape():
     dq2, dk2, dv2 = capi.bwd((dc.float() * 2).half(), qc, kc, vc, o, lse, mask=mc, **kw)
     for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
         assert (b.float() - 2 * a.float()).abs().max().item() <= 1e-2 * b.float().abs().max().item()
+        # (not bit for bit: many dS elements are fp16 subnormals, whose rounding does not commute with a doubling)
     # padded keys receive no gradient
     lens = (m[:, 0, 0] == 0).sum(-1)
     dkv = dk.view(B, H, S, D).float().abs() + dv.view(B, H, S, D).float().abs()

@@ -357,6 +357,13 @@ def test_size_independent_properties_at_headline_shape():
     o_a = capi.fwd(qc, kc, v2, mask=mc)[0]
     o_s = capi.fwd(qc, kc, (vc.float() + v2.float()).half(), mask=mc)[0]
     assert (o_s.float() - (o.float() + o_a.float())).abs().max().item() <= 6e-3
+    # exact ones: V = 1 gives O = 1 (the weights are the rounded probabilities over THEIR sum), and doubling V
+    # doubles O bit for bit (a power of two commutes with every rounding on the way, outside the subnormal range)
+    o_1 = capi.fwd(qc, kc, torch.ones_like(vc), mask=mc)[0]
+    assert torch.equal(o_1, torch.ones_like(o_1))
+    o_2 = capi.fwd(qc, kc, vc * 2, mask=mc)[0]
+    big = o.float().abs() >= 2.0 ** -13       # (a doubled value that leaves fp16's subnormal range carries bits its half had lost)
+    assert torch.equal(o_2[big], (o * 2)[big])
     # masked keys carry no weight: scrambling V on the padded tail changes nothing
     lens = (m[:, 0, 0] == 0).sum(-1)
     v3 = vc.clone().view(B, H, S, D)
