@@ -277,8 +277,9 @@ float fmha_drop_scale(float p_drop);
 /* Static description of a return code. */
 const char *fmha_strerror(int code);
 
-/* The FMHA_* environment variables (tuning and test overrides of the variant selection, listed in
- * INTEGRATION.md) are read once per process, on the first launch.  This reads them again; not to be
+/* The FMHA_* environment variables -- tuning and test overrides of the variant selection: FMHA_MASK_TRIM,
+ * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_BWD_SHORT, FMHA_BWD_PAIR,
+ * FMHA_BWD_FUSED -- are read once per process, on the first launch.  This reads them again; not to be
  * called while another thread is launching.  (No counterpart in the reference.) */
 void fmha_reload_overrides(void);
 
