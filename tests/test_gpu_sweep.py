@@ -6,7 +6,7 @@ exceeds 2), gradients within 1e-2 / 3e-2 of the largest oracle entry, LSE within
 -inf rows in the same places; where a per-key mask is involved, skipping the hard-masked tail must not
 change a bit.
 
-Gradients that are exactly zero.  When every query of a problem sees exactly one key (sk = 1, a valid
+Gradients that are exactly zero.  When every query of a head sees exactly one key (sk = 1, a valid
 length of 1, a causal first row alone), softmax is the constant 1 and dQ = dK = 0.  The kernels then
 compute dS_i = P_i (dP_i - delta_i) with dP_i = Z (dO_i . V_k) and delta_i = dO_i . O_i, where O_i is the
 forward's output ROUNDED to the element type: O_i = round(Z V_k).  The two terms differ by
@@ -109,17 +109,21 @@ def _run_case(it, c, rng):
     gtol = 1e-2 if dtype == "fp16" else 3e-2
     got_o = f32(o.reshape(bh, sq, d).cpu())
     assert np.abs(got_o - ref["o"]).max() <= otol, "o"
-    # the absolute bound for gradients whose true value is zero throughout (module docstring)
+    # the absolute bound for gradients whose true value is zero throughout a head (module docstring): heads of a
+    # sequence with one visible key sit beside heads with ordinary gradients, so the two criteria apply head by head
     a_rows = np.abs(f32(do) * got_o).sum(-1)                                   # A_i per (head, query)
-    zero_tol = 4 * d ** -0.5 * UNIT[dtype] * float(np.sqrt((a_rows ** 2).sum(-1)).max()) * \
-        float(max(np.abs(f32(q)).max(), np.abs(f32(k)).max()))
+    zero_tol = 4 * d ** -0.5 * UNIT[dtype] * np.sqrt((a_rows ** 2).sum(-1)) * \
+        float(max(np.abs(f32(q)).max(), np.abs(f32(k)).max()))                 # per head
     for name, t in (("dq", dq), ("dk", dk), ("dv", dv)):
         a = f32(t.reshape(ref[name].shape).cpu())
         assert np.isfinite(a).all(), name
-        if name != "dv" and np.abs(ref[name]).max() < 1e-6:
-            assert np.abs(a).max() <= max(zero_tol, 1e-6), f"{name}: zero gradient, |got| {np.abs(a).max():.3e} > {zero_tol:.3e}"
-        else:
-            assert rel_to_max(a, ref[name], floor=1e-3) <= gtol, name
+        err = np.abs(a - ref[name]).reshape(bh, -1).max(1)
+        top = np.abs(ref[name]).reshape(bh, -1).max(1)
+        zero = (top < 1e-6) if name != "dv" else np.zeros(bh, bool)
+        assert (err[zero] <= np.maximum(zero_tol[zero], 1e-6)).all(), \
+            f"{name}: zero gradient, |got| {err[zero].max():.3e} > {zero_tol[zero].min():.3e}"
+        if (~zero).any():
+            assert err[~zero].max() / max(top.max(), 1e-3) <= gtol, name
     fin = np.isfinite(ref["lse"])
     gl = lse.reshape(bh, sq).cpu().numpy()
     assert np.array_equal(np.isfinite(gl), fin), "lse: -inf rows differ"
