@@ -89,8 +89,14 @@ template <int D> struct FwdCfg {
   static constexpr int NSB = BK / 32;     // 32-key sub-blocks per tile
   static constexpr int KS = D / 16;       // contraction steps of K.Q^T
   static constexpr int DB = D / 32;       // 32-row blocks of O^T
-  static constexpr int ROWB = D * 2 + 16; // LDS row pitch in bytes (16 B pad: conflict-free b128 reads)
-  static constexpr int TILEB = BK * ROWB;
+  // LDS row pitches in bytes.  K rows are read 16 bytes per lane, a row per lane: a pad of 16 bytes puts sixteen
+  // consecutive rows on the sixteen 16-byte bank groups.  V rows are read by the transpose read, 8 bytes per lane,
+  // four lanes per row and four rows per sixteen lanes: a pad of 32 bytes sets consecutive rows 32 bytes apart in
+  // the banks, so the sixteen lanes cover 128 contiguous bytes (with the 16-byte pad rows overlapped pairwise and
+  // every such read took two passes).
+  static constexpr int ROWB = D * 2 + 16;
+  static constexpr int ROWBV = D * 2 + 32;
+  static constexpr int TILEB = BK * ROWBV; // (one size for both tiles)
   static constexpr int XROWB = 32;        // pitch of the extra-contraction-step rows (16 elements)
   static constexpr int LDS_BYTES = 4 * TILEB + 2 * BK * XROWB; // {K,V} x 2 stages + extra rows x 2 stages
 };
@@ -116,7 +122,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   using v8 = typename E::v8;
   using v4 = typename E::v4;
   using C = FwdCfg<D>;
-  constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, XROWB = C::XROWB;
+  constexpr int BK = C::BK, NSB = C::NSB, KS = C::KS, DB = C::DB, ROWB = C::ROWB, ROWBV = C::ROWBV, XROWB = C::XROWB;
   constexpr int TILEB = C::TILEB;
   constexpr int NT = NW * 64;
   constexpr int QT = NW * QB * 32;
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       const int row = c / CPR, col = c % CPR;
       const bool live = col * 8 < RW::cols(a);
       *(u32x4 *)(kd + row * ROWB + col * 16) = chunk_or_zero(kst[i], live);
-      *(u32x4 *)(vd + row * ROWB + col * 16) = chunk_or_zero(vst[i], live);
+      *(u32x4 *)(vd + row * ROWBV + col * 16) = chunk_or_zero(vst[i], live);
     }
     if (tid < BK) {
       // extra contraction step, A side: (1, mask_hi, mask_lo, 1, 0 ...); keys past the end get
@@ -512,7 +518,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
             for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
               for (int c = 0; c < 2; ++c) {
-                const v8 va = lds_load_a_transposed<T, ROWB>(ldsV, sb * 32, db * 32, c, l);
+                const v8 va = lds_load_a_transposed<T, ROWBV>(ldsV, sb * 32, db * 32, c, l);
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) o[qb][db] = E::mfma(va, pfrag[qb][sb][c], o[qb][db]);
               }
