@@ -452,6 +452,49 @@ def fp8_leg(torch, capi, L, stream, steps, warmup):
             "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)}
 
 
+DECODE_SHAPES = {  # name: (heads, query rows, keys, head dim)
+    "BH32_Sk32768_D128": (32, 1, 32768, 128),
+    "BH64_Sk8192_D128": (64, 1, 8192, 128),
+    "BH8_Sk131072_D128": (8, 1, 131072, 128),
+    "BH128_Sk16384_D64": (128, 1, 16384, 64),
+}
+
+
+def decode_sets(torch, bh, sq, sk, d):
+    """Input sets for a decode step, enough of them that K and V (the bytes that count) come from HBM."""
+    g = torch.Generator().manual_seed(31)
+    nset = max(2, int(600e6 // (4 * bh * sk * d)) + 1)
+    sets = []
+    for _ in range(nset):
+        q = torch.randn(bh, sq, d, generator=g).half().cuda()
+        k, v = (torch.randn(bh, sk, d, device="cuda", dtype=torch.float16) for _ in range(2))
+        sets.append((q, k, v, torch.empty_like(q)))
+    return sets
+
+
+def decode_leg(torch, capi, steps, warmup):
+    """Decode steps (one query row per head against a long fp16 K/V cache, no mask): HBM-bound, the bytes are K
+    and V once.  `plain` is the launch by head, `pieces` the same call with a workspace, where the library
+    cuts the key range so that the whole chip streams.  Never part of `value`."""
+    out = {}
+    for name, (bh, sq, sk, d) in DECODE_SHAPES.items():
+        sets = decode_sets(torch, bh, sq, sk, d)
+        ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+        by = 4.0 * bh * sk * d + 4.0 * bh * sq * d
+        leg = {"workload": f"bh {bh}, {sq} query row, {sk} keys, head dim {d}, fp16; {len(sets)} input sets rotated",
+               "algorithmic_MB": round(by / 1e6, 1)}
+        for mode, w in (("plain", False), ("pieces", ws)):
+            def step(i):
+                q, k, v, o = sets[i % len(sets)]
+                capi.fwd(q, k, v, out=o, workspace=w)
+            ms, _ = time_steps(torch, step, steps, warmup, blocks=9)
+            leg[mode] = {"us": round(ms * 1e3, 1), "TBps": round(by / (ms * 1e-3) / 1e12, 2),
+                         "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)}
+        out[name] = leg
+        del sets, ws
+    return out
+
+
 def profile_leg(torch, capi, L, stream, args):
     """`--profile LEG`: nothing but LEG's launches, `--steps` times after `--warmup`, for a run under
     `rocprofv3` (kernel trace or counters) in which every dispatch of a kernel belongs to one workload.
@@ -490,6 +533,14 @@ def profile_leg(torch, capi, L, stream, args):
         delta = torch.empty_like(lse)
         steps.append(lambda i: capi.fwd(q, k, v, want_lse=True, out=o, **kw))
         steps.append(lambda i: capi.bwd(do, q, k, v, o, lse, grads=grads, delta=delta, **kw))
+    elif leg in ("decode", "decode_plain"):
+        sets = decode_sets(torch, *DECODE_SHAPES["BH32_Sk32768_D128"])
+        ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda") if leg == "decode" else False
+
+        def decode_step(i):
+            q, k, v, o = sets[i % len(sets)]
+            capi.fwd(q, k, v, out=o, workspace=ws)
+        steps.append(decode_step)
     elif leg == "fp8":
         g = torch.Generator().manual_seed(21)
         q8, k8, v8 = (torch.randn(B * H, S, D, generator=g).to(torch.float8_e4m3fn).cuda() for _ in range(3))
@@ -649,7 +700,8 @@ def main():
                     help="also run a plain 256 MiB device copy a few times: under `rocprofv3 --pmc FETCH_SIZE` "
                          "(or WRITE_SIZE) its known traffic calibrates the counter for the attention kernels")
     ap.add_argument("--profile", metavar="LEG", default=None,
-                    help="run only LEG's launches (fwd, fwd_trim, train, train_one_pass, c4, c5, d256, fp8) and no "
+                    help="run only LEG's launches (fwd, fwd_trim, train, train_one_pass, c4, c5, d256, fp8, decode, "
+                         "decode_plain) and no "
                          "timing: for rocprofv3 runs in which every dispatch of a kernel is the same workload")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -834,6 +886,7 @@ def main():
     out["torch_sdpa_same_gpu"] = torch_sdpa_context(torch, args.steps, args.warmup)
     out["head_dim_256"] = head_dim_256_leg(torch, capi)
     out["fp8_e4m3_forward"] = fp8_leg(torch, capi, L, stream, args.steps, args.warmup)
+    out["decode_steps"] = decode_leg(torch, capi, args.steps, args.warmup)
     out["power"] = power
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 

@@ -348,6 +348,14 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd(const at::Tensor &q_, const at::Tens
   set_mask_and_dropout(p, m, mask, q, k.s, p_drop, seed, offset);
   at::Tensor kv_keep;
   set_kv_len(p, kv_len, q.bh, kv_keep);
+  // Few heads, few query rows and a long key range (decode steps): given room for the pieces' partial
+  // results the library cuts the key range into pieces and fills the whole chip.
+  at::Tensor workspace;
+  if (const uint64_t need = fmha_fwd_workspace_bytes(&p); need > 0) {
+    workspace = at::empty({static_cast<int64_t>(need)}, q.t.options().dtype(at::kByte));
+    p.workspace = workspace.data_ptr();
+    p.workspace_bytes = need;
+  }
   launch_fwd(p, q.t);
   return std::make_tuple(o, lse);
 }

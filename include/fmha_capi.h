@@ -154,10 +154,29 @@ typedef struct fmha_fwd_params {
    * lse (and delta) stay [bh, sq] contiguous.  Outputs must not overlap inputs. */
   int32_t heads;
   int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];
+
+  /* Optional device memory for a forward whose key range is cut into pieces (no counterpart in the
+   * reference, whose shapes are fixed at 128 x 128 per head, fmha_manual.cpp:24-29).  A decode step -- one
+   * or a few query rows per head against a long key range -- on fewer heads than the chip holds workgroups
+   * would leave most compute units idle while each busy one streams a whole K and V.  Given a workspace of
+   * at least fmha_fwd_workspace_bytes(p) bytes (16-byte aligned), such a launch runs every piece of the
+   * key range as a head of its own, keeps the pieces' normalised outputs (element type = dtype) and
+   * log-sum-exps in the workspace and merges them in a second launch:
+   *   O = sum_c exp(LSE_c - LSE) O_c,   LSE = log sum_c exp(LSE_c).
+   * Results differ from the plain launch by one more rounding to the element type (of the partial
+   * outputs).  Pieces are used without a causal mask, dropout or saved outputs, with no mask or a mask that
+   * is constant along the queries, with or without kv_len; everything else, a NULL or too small workspace
+   * included, takes the plain launch.  The workspace may be reused by the next launch on the same stream. */
+  void *workspace;
+  uint64_t workspace_bytes;
 } fmha_fwd_params;
 
 /* Enqueue the forward kernel on `hip_stream` (a hipStream_t; NULL = default stream). */
 int fmha_fwd_launch(const fmha_fwd_params *p, void *hip_stream);
+
+/* Bytes of `workspace` with which fmha_fwd_launch(p) would run its key range in pieces on the current
+ * device, or 0 where it would not (p as for the launch; the pointers are not looked at). */
+uint64_t fmha_fwd_workspace_bytes(const fmha_fwd_params *p);
 
 /*
  * Forward on 8-bit floating point inputs (no counterpart in the reference, which is fp16 only:

@@ -18,9 +18,10 @@ DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
            "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides",
-           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale", "fmha_fwd_fp8_launch")
+           "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale", "fmha_fwd_fp8_launch",
+           "fmha_fwd_workspace_bytes")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
-_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB",
+_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
 _env_seen = None
 
@@ -58,6 +59,7 @@ class FwdParams(_Params):
         ("heads", C.c_int32),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("o_stride", C.c_int64 * 3),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
     ]
 
 
@@ -115,6 +117,8 @@ def lib():
         L = C.CDLL(LIB_PATH)
         L.fmha_fwd_launch.argtypes = [C.POINTER(FwdParams), C.c_void_p]
         L.fmha_fwd_launch.restype = C.c_int
+        L.fmha_fwd_workspace_bytes.argtypes = [C.POINTER(FwdParams)]
+        L.fmha_fwd_workspace_bytes.restype = C.c_uint64
         L.fmha_bwd_launch.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         L.fmha_bwd_launch.restype = C.c_int
         L.fmha_fwd_fp8_launch.argtypes = [C.POINTER(FwdFp8Params), C.c_void_p]
@@ -221,8 +225,12 @@ def _set_rows(P, heads, **tensors):
 
 def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=False, scale=None,
         drop_kind=DROP_NONE, drop_mask=None, p_drop=0.0, drop_scale=None, seed=0, offset=0,
-        want_lse=False, save=False, flags=0, out=None, kv_len=None):
+        want_lse=False, save=False, flags=0, out=None, kv_len=None, workspace=True):
     """Launch the forward on the current stream.  Returns (o, lse|None, softmax|None, dropout|None).
+
+    workspace: True allocates what ``fmha_fwd_workspace_bytes`` asks for (nothing for most shapes: only
+    launches with few heads, few query rows and a long key range run their key range in pieces), False
+    passes none (always the plain launch), a uint8 device tensor is passed as it is.
 
     kv_len: optional int32 device tensor of B valid key counts (bh must be a multiple of B); head i
     attends keys [0, kv_len[i // (bh // B)]) only.
@@ -281,6 +289,15 @@ def fwd(q, k, v, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-10000.0, causal=F
     P.flags = flags
     _set_kv_len(P, kv_len, bh)
     _sync_env()
+    ws = None
+    if workspace is True:
+        need = lib().fmha_fwd_workspace_bytes(C.byref(P))
+        if need:
+            ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    elif workspace is not False and workspace is not None:
+        ws = workspace
+    if ws is not None:
+        P.workspace, P.workspace_bytes = ws.data_ptr(), ws.numel()
     check(lib().fmha_fwd_launch(C.byref(P), _stream_ptr()))
     return o, lse, sm, dr
 

@@ -4,6 +4,7 @@
 #include "fmha_launch.h"
 #include "fmha_fwd_fp8.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstddef>
 #include <cstring>
@@ -49,10 +50,11 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
 // one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
 // pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
-// that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call).
+// that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call), FMHA_FWD_SPLIT=0 never cuts a
+// forward's key range into pieces, FMHA_FWD_SPLIT=n (2..64) cuts it into about n wherever pieces are possible.
 // The environment is read once per process (on the first launch); fmha_reload_overrides() reads it again.
 struct Overrides {
-  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, bwd_pair, bwd_short, bwd_fused;
+  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, bwd_pair, bwd_short, bwd_fused;
 };
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
@@ -65,6 +67,7 @@ Overrides read_overrides() {
   o.fwd_save_split = env_int("FMHA_FWD_SAVE_SPLIT", 1);
   o.fwd_stream = env_int("FMHA_FWD_STREAM", 1);
   o.fwd_qb = env_int("FMHA_FWD_QB", 0);
+  o.fwd_split = env_int("FMHA_FWD_SPLIT", -1);
   o.bwd_pair = env_int("FMHA_BWD_PAIR", -1);
   o.bwd_short = env_int("FMHA_BWD_SHORT", 1);
   o.bwd_fused = env_int("FMHA_BWD_FUSED", 0);
@@ -73,6 +76,153 @@ Overrides read_overrides() {
 Overrides &overrides() {
   static Overrides o = read_overrides();
   return o;
+}
+
+constexpr int kMaxDevices = 64;
+
+// Compute units of the current device (0 if it cannot be asked), looked up once per device.
+int cu_count() {
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 0) n = 0;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+// ---- A forward whose key range is cut into pieces (few heads, long key ranges: decode steps) ----
+// With one to a few query rows per head and fewer heads than the chip has room for workgroups, a launch
+// by head leaves most compute units idle while each busy one streams a whole K and V.  Such a forward
+// runs as `pieces` forwards over `chunk` keys each (the kernels see bh * pieces heads: RowMap's third
+// level), which write normalised partial outputs and their log-sum-exps into the caller's workspace,
+// and a second launch merges them:  O = sum_c w_c O_c,  w_c = exp(LSE_c - LSE),  LSE = log sum_c exp(LSE_c).
+constexpr int kMaxPieces = 64; // what the merge kernel holds in LDS
+struct SplitPlan {
+  int pieces, chunk;
+  size_t off_lse, off_mask, bytes; // the partial outputs start at offset 0
+};
+
+size_t round256(size_t x) { return (x + 255u) & ~(size_t)255u; }
+
+// Whether the forward described by p (already validated) runs in pieces, and where its intermediates go.
+bool plan_split(const fmha_fwd_params *p, SplitPlan &pl) {
+  const int force = overrides().fwd_split;
+  if (force == 0) return false;
+  if (p->causal || p->drop_kind != FMHA_DROP_NONE || p->save_softmax || p->save_dropout) return false;
+  if (p->mask_kind != FMHA_MASK_NONE && p->mask_stride_q != 0) return false; // a [.., sq, sk] mask tensor
+  const long long sk = p->sk, sq = p->sq;
+  long long chunk;
+  if (force >= 2) {
+    const long long n = force > kMaxPieces ? kMaxPieces : force;
+    chunk = ((sk + n - 1) / n + 127) / 128 * 128;
+  } else {
+    const int cus = cu_count();
+    const long long items = (long long)p->bh * ((sq + 127) / 128); // workgroups of the plain launch
+    // Worth it while the plain launch has fewer workgroups than the chip has compute units (with one per
+    // unit it already streams at 0.66 of the HBM peak, measured) and the key range is long enough to cut.
+    if (cus <= 0 || items >= cus || sk < 2048) return false;
+    // Measured best (one to sixteen heads per compute unit's worth of work, 4k to 128k keys): about two
+    // workgroups per compute unit, pieces of at least 1024 keys.
+    const long long want = (2LL * cus + items - 1) / items;
+    chunk = ((sk + want - 1) / want + 127) / 128 * 128;
+    const long long least = (4 * sq + 127) / 128 * 128;         // partial outputs stay under an eighth of the K/V bytes
+    if (chunk < least) chunk = least;
+    if (chunk < 1024) chunk = 1024;
+    const long long cap = ((sk + kMaxPieces - 1) / kMaxPieces + 127) / 128 * 128;
+    if (chunk < cap) chunk = cap;
+  }
+  const long long pieces = (sk + chunk - 1) / chunk;
+  if (pieces < 2 || pieces > kMaxPieces || (long long)p->bh * pieces >= (1ll << 24)) return false;
+  pl.pieces = (int)pieces;
+  pl.chunk = (int)chunk;
+  const size_t vh = (size_t)p->bh * (size_t)pieces;
+  size_t off = round256(vh * (size_t)sq * (size_t)p->d * 2u);
+  pl.off_lse = off;
+  off += round256(vh * (size_t)sq * sizeof(float));
+  pl.off_mask = off;
+  if (p->mask_kind != FMHA_MASK_NONE) off += round256(vh * (size_t)chunk * 2u);
+  pl.bytes = off;
+  return true;
+}
+
+// A per-key mask's rows regrouped by piece (the kernels index mask rows by head): piece c of head i gets keys
+// [c * chunk, (c + 1) * chunk) of row i / mask_div.  One thread per (head, piece, group of 8 keys).
+__global__ void split_mask_kernel(uint16_t *mask_out, const uint16_t *mask_in, int64_t mask_sb, int32_t mask_div,
+                                  int32_t bh, int32_t sk, int32_t pieces, int32_t chunk) {
+  const int gpp = chunk / 8; // threads per piece
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)bh * pieces * gpp) return;
+  const int g = (int)(idx % gpp);
+  const long long vh = idx / gpp;
+  const int c = (int)(vh % pieces);
+  const int i = (int)(vh / pieces);
+  const uint16_t *src = mask_in + (size_t)(i / mask_div) * (size_t)mask_sb;
+  uint16_t *dst = mask_out + (size_t)vh * (size_t)chunk + g * 8;
+  for (int t = 0; t < 8; ++t) {
+    const int key = c * chunk + g * 8 + t;
+    dst[t] = key < sk ? src[key] : (uint16_t)0; // (keys past the end are excluded by the pieces' key counts)
+  }
+}
+
+// Merges the pieces: one workgroup of kMergeThreads per (head, query row).  Thread t owns 8 output columns
+// (t % cpr) and every (kMergeThreads / cpr)-th piece, so that the loads of all pieces are in flight together
+// (a thread walking the pieces one after the other pays a trip to memory per piece); the threads' sums meet in LDS.
+constexpr int kMergeThreads = 256;
+template <typename T>
+__global__ void __launch_bounds__(kMergeThreads)
+split_merge_kernel(const T *o_part, const float *lse_part, T *o, float *lse, RowMap mo, int32_t sq, int32_t d,
+                   int32_t pieces) {
+  __shared__ float s_lse[kMaxPieces];
+  __shared__ float s_acc[kMergeThreads][9];
+  const int t = threadIdx.x;
+  const int cpr = d / 8;          // 16-byte column groups per row (1..32)
+  const int lanes = kMergeThreads / cpr; // threads per column group
+  const int c8 = t % cpr, pl = t / cpr;  // (threads with pl >= lanes have no work)
+  const int h = blockIdx.x / sq, q = blockIdx.x - h * sq;
+  const size_t row0 = (size_t)h * pieces * sq + q; // piece c: row0 + c * sq
+  if (t < pieces) s_lse[t] = lse_part[row0 + (size_t)t * sq];
+  __syncthreads();
+  float m = -INFINITY;
+  for (int c = 0; c < pieces; ++c) m = fmaxf(m, s_lse[c]);
+  float acc[9] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; // eight columns and the sum of the weights
+  if (m != -INFINITY && pl < lanes) { // (a head without any visible key: O = 0, LSE = -inf, like the plain launch)
+    for (int c = pl; c < pieces; c += lanes) {
+      const float l = s_lse[c];
+      if (l == -INFINITY) continue; // an empty piece
+      const float w = expf(l - m);
+      Pack16 x;
+      x.u = *(const u32x4 *)(o_part + (row0 + (size_t)c * sq) * d + c8 * 8);
+      acc[8] += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float xv;
+        if constexpr (__is_same(T, _Float16)) xv = (float)x.h[e];
+        else xv = (float)x.b[e];
+        acc[e] += w * xv;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 9; ++e) s_acc[t][e] = acc[e];
+  __syncthreads();
+  if (pl != 0) return;
+  for (int j = 1; j < lanes; ++j) {
+#pragma unroll
+    for (int e = 0; e < 9; ++e) acc[e] += s_acc[j * cpr + c8][e];
+  }
+  const float tot = acc[8];
+  const float inv = tot > 0.f ? 1.f / tot : 0.f;
+  Pack16 y;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    if constexpr (__is_same(T, _Float16)) y.h[e] = (_Float16)(acc[e] * inv);
+    else y.b[e] = (__bf16)(acc[e] * inv);
+  }
+  *(u32x4 *)(o + mo.head(h) + (size_t)q * (size_t)mo.ss + c8 * 8) = y.u;
+  if (lse && c8 == 0) lse[(size_t)h * sq + q] = tot > 0.f ? m + logf(tot) : -INFINITY;
 }
 
 } // namespace
@@ -136,6 +286,9 @@ static int built_head_dim(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 static int make_row_map(RowMap &m, int32_t heads, const int64_t st[3], int32_t bh, int32_t rows, int32_t d,
                         bool &strided) {
   m.heads_rcp = 0;
+  m.sp = 0;
+  m.pieces = 1;
+  m.pieces_rcp = 0;
   if (heads == 0) {
     m.sb = (int64_t)rows * d;
     m.sh = 0;
@@ -157,7 +310,89 @@ static int make_row_map(RowMap &m, int32_t heads, const int64_t st[3], int32_t b
   return FMHA_OK;
 }
 
+static int fwd_dispatch_strided(FwdArgs &a, const FwdVariant &v, int dtype, int D, hipStream_t s) {
+  if (dtype == FMHA_DTYPE_F16)
+    return D == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_f16_d128_strided(a, v, s) : fwd_dispatch_f16_d256_strided(a, v, s);
+  return D == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_bf16_d128_strided(a, v, s) : fwd_dispatch_bf16_d256_strided(a, v, s);
+}
+
+// The forward in pieces (plan_split): a per-key mask's rows regrouped by piece, the forward kernels over bh * pieces
+// heads of `chunk` keys on the run-time-layout code path, then the merge.  `a` describes the whole launch.
+static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const SplitPlan &pl, int D, hipStream_t s) {
+  unsigned char *ws = (unsigned char *)p->workspace;
+  float *lse_part = (float *)(ws + pl.off_lse);
+  uint16_t *mask_part = a.mask ? (uint16_t *)(ws + pl.off_mask) : nullptr;
+  const long long vh = (long long)p->bh * pl.pieces;
+  if (a.mask) {
+    const long long threads = vh * (pl.chunk / 8);
+    const int nt = 256;
+    hipLaunchKernelGGL(split_mask_kernel, dim3((unsigned)((threads + nt - 1) / nt)), dim3(nt), 0, s, mask_part,
+                       (const uint16_t *)a.mask, a.mask_sb, a.mask_div, p->bh, p->sk, pl.pieces, pl.chunk);
+    if (hipGetLastError() != hipSuccess) return FMHA_E_LAUNCH;
+  }
+  FwdArgs b = a;
+  b.o = ws;
+  b.lse = lse_part;
+  b.sk_whole = p->sk; // the kernels work out each piece's own key count (from the head's valid count, if any)
+  if (a.mask) {
+    b.mask = mask_part;
+    b.mask_sb = pl.chunk;
+    b.mask_sq = 0;
+    b.mask_div = 1;
+  }
+  b.mask_vec = 1; // pieces are multiples of 128 keys and start on 256-byte boundaries
+  b.bh = (int32_t)vh;
+  b.sk = pl.chunk;
+  b.drop = make_drop_ctx(0, 0, 0.f, p->sq, pl.chunk);
+  b.clock_probe = nullptr;
+  const uint32_t rcp = (uint32_t)((1ull << 32) / (uint64_t)pl.pieces) + 1u;
+  for (RowMap *m : {&b.mq, &b.mk, &b.mv}) {
+    m->pieces = pl.pieces;
+    m->pieces_rcp = rcp;
+  }
+  b.mq.sp = 0;
+  b.mk.sp = (int64_t)pl.chunk * a.mk.ss;
+  b.mv.sp = (int64_t)pl.chunk * a.mv.ss;
+  b.mo.heads = 1; // the partial outputs: [bh * pieces, sq, d] contiguous
+  b.mo.heads_rcp = 0;
+  b.mo.sb = (int64_t)p->sq * p->d;
+  b.mo.sh = 0;
+  b.mo.ss = p->d;
+  FwdVariant v;
+  v.qb = 1;
+  v.mask = a.mask ? kMaskPerKey : kMaskNone;
+  v.causal = false;
+  v.drop = 0;
+  v.saving = v.save_split = v.stream = v.short_keys = false;
+  const int rc = fwd_dispatch_strided(b, v, p->dtype, D, s);
+  if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
+  {
+    const long long rows = (long long)p->bh * p->sq;
+    const dim3 grid((unsigned)rows);
+    if (p->dtype == FMHA_DTYPE_F16)
+      hipLaunchKernelGGL(split_merge_kernel<_Float16>, grid, dim3(kMergeThreads), 0, s, (const _Float16 *)ws, lse_part,
+                         (_Float16 *)p->o, p->lse, a.mo, p->sq, p->d, pl.pieces);
+    else
+      hipLaunchKernelGGL(split_merge_kernel<__bf16>, grid, dim3(kMergeThreads), 0, s, (const __bf16 *)ws, lse_part,
+                         (__bf16 *)p->o, p->lse, a.mo, p->sq, p->d, pl.pieces);
+    if (hipGetLastError() != hipSuccess) return FMHA_E_LAUNCH;
+  }
+  return FMHA_OK;
+}
+
 extern "C" {
+
+uint64_t fmha_fwd_workspace_bytes(const fmha_fwd_params *caller) {
+  if (!caller || caller->struct_bytes < offsetof(fmha_fwd_params, kv_len)) return 0;
+  fmha_fwd_params local;
+  std::memset(&local, 0, sizeof local);
+  std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
+  if (local.bh <= 0 || local.sq <= 0 || local.sk <= 0 || local.d < 8 || local.d > 256 || (local.d & 7) != 0) return 0;
+  if (local.drop_kind == FMHA_DROP_PHILOX && fmha_drop_threshold(local.p_drop) == 0) local.drop_kind = FMHA_DROP_NONE;
+  if (local.sq == 1) local.mask_stride_q = 0;
+  SplitPlan pl;
+  return plan_split(&local, pl) ? (uint64_t)pl.bytes : 0;
+}
 
 int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   // the caller's struct may be shorter (older header) or longer (newer) than this library's
@@ -189,6 +424,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
     if (fmha_drop_threshold(p->p_drop) == 0) local.drop_kind = FMHA_DROP_NONE;
     else if (p->drop_scale == 0.f) local.drop_scale = fmha_drop_scale(p->p_drop);
   }
+  if (p->sq == 1) local.mask_stride_q = 0; // one query row: any mask is a per-key mask
   const bool saving = p->save_softmax || p->save_dropout;
   if (saving && (p->drop_kind == FMHA_DROP_PHILOX || p->causal)) return FMHA_E_UNSUPPORTED;
   if (p->drop_kind == FMHA_DROP_TENSOR && p->causal) return FMHA_E_UNSUPPORTED;
@@ -231,6 +467,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (!overrides().mask_trim) a.flags |= kFwdFlagNoTrim;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
+  a.sk_whole = 0;
   a.clock_probe = (unsigned long long *)p->clock_probe;
   int mrc;
   bool strided = false;
@@ -242,6 +479,11 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   a.dcols = p->d;
   if (a.mk.ss != a.mv.ss) return FMHA_E_UNSUPPORTED;
   if (strided && (saving || p->drop_kind == FMHA_DROP_TENSOR)) return FMHA_E_UNSUPPORTED;
+
+  hipStream_t s = (hipStream_t)hip_stream;
+  SplitPlan pl;
+  if (p->workspace && ((uintptr_t)p->workspace & 15u) == 0 && plan_split(p, pl) && p->workspace_bytes >= pl.bytes)
+    return fwd_split_launch(p, a, pl, D, s);
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);
@@ -277,13 +519,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   // so one block per wave is faster there.
   v.qb = 1;
   if (p->d == 64 && !v.causal && v.drop == 0 && v.mask == kMaskNone) {
-    static const int cus = [] {
-      int dev = 0, n = 0;
-      if (hipGetDevice(&dev) != hipSuccess ||
-          hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-        n = 0;
-      return n;
-    }();
+    const int cus = cu_count();
     const int tiles2 = (p->sq + 255) / 256;
     const long long items2 = (long long)p->bh * tiles2;
     const bool little_padding = tiles2 * 256 - p->sq <= p->sq / 8;
@@ -293,14 +529,9 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;
   if (strided) v.qb = 1; // the two-block variant is built for the folded layout only
 
-  hipStream_t s = (hipStream_t)hip_stream;
   int rc;
-  if (strided) {
-    if (p->dtype == FMHA_DTYPE_F16)
-      rc = D == 64 ? fwd_dispatch_f16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_f16_d128_strided(a, v, s) : fwd_dispatch_f16_d256_strided(a, v, s);
-    else
-      rc = D == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_bf16_d128_strided(a, v, s) : fwd_dispatch_bf16_d256_strided(a, v, s);
-  } else if (p->dtype == FMHA_DTYPE_F16)
+  if (strided) rc = fwd_dispatch_strided(a, v, p->dtype, D, s);
+  else if (p->dtype == FMHA_DTYPE_F16)
     rc = D == 64 ? fwd_dispatch_f16_d64(a, v, s) : D == 128 ? fwd_dispatch_f16_d128(a, v, s) : fwd_dispatch_f16_d256(a, v, s);
   else
     rc = D == 64 ? fwd_dispatch_bf16_d64(a, v, s) : D == 128 ? fwd_dispatch_bf16_d128(a, v, s) : fwd_dispatch_bf16_d256(a, v, s);
@@ -319,7 +550,6 @@ uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d)
 // device address is looked up once per device (the array's name is only a host-side handle).
 namespace {
 constexpr size_t kScratchBytes = 8u << 20;
-constexpr int kMaxDevices = 64;
 } // namespace
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 namespace {

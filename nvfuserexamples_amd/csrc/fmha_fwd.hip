@@ -78,7 +78,7 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
     const bool mask_ok = a.mask_a == FMHA_LOG2E && a.mask_b == 0.f && a.sk % 8 == 0 && a.sk > 128 && a.sk <= 1024 &&
                          rows * ((a.sk + 511) / 512) <= 64 && a.mask_sb % 8 == 0 &&
                          (reinterpret_cast<uintptr_t>(a.mask) & 15) == 0;
-    if (shape && mask_ok && !a.kv_len && !(a.flags & kFwdFlagNoTrim)) {
+    if (shape && mask_ok && !a.kv_len && a.sk_whole == 0 && !(a.flags & kFwdFlagNoTrim)) {
       a.bal_rows = (int32_t)rows;
       a.bal_ipr = (int32_t)ipr;
       a.bal_R = (int32_t)(nblk / ipr);

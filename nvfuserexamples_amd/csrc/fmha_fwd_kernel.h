@@ -64,6 +64,7 @@ struct FwdArgs {
   int32_t flags;
   const int32_t *kv_len; // optional valid key count per group of kv_div heads (not with tensor dropout / saved outputs)
   int32_t kv_div;
+  int32_t sk_whole;      // key range cut into pieces (mk.pieces > 1): its whole length; sk is then the length of a piece
   unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
   RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
   int32_t dcols;         // elements per row that exist (<= the kernel's head dim; run-time layouts only)
@@ -83,6 +84,27 @@ enum { kFwdFlagNoTrim = 1 }; // visit every key tile even where a per-key mask h
 
 // how the mask tensor is read
 enum { kMaskNone = 0, kMaskPerKey = 1, kMaskFull = 2 };
+
+// Keys head `bh` may see at all: all sk, or the head's valid count (possibly 0).  With the key range cut into
+// pieces that run as heads of their own (RowMap::pieces of k; counts are per real head), what is left of
+// either in this head's piece.
+template <bool STRIDED> FMHA_DEV int visible_keys(const FwdArgs &a, int bh) {
+  int whole = a.sk, head = bh, first = 0;
+  if constexpr (STRIDED) {
+    if (a.mk.pieces > 1) {
+      head = (int)__umulhi((uint32_t)bh, a.mk.pieces_rcp);
+      first = (bh - head * a.mk.pieces) * a.sk;
+      whole = a.sk_whole;
+    }
+  }
+  int n = whole;
+  if (a.kv_len) {
+    const int m = a.kv_len[head / a.kv_div];
+    n = m < 0 ? 0 : (m < n ? m : n);
+  }
+  n -= first;
+  return n < 0 ? 0 : (n < a.sk ? n : a.sk);
+}
 
 template <int D> struct FwdCfg {
   static constexpr int BK = 64;           // keys per LDS tile
@@ -177,11 +199,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
   // ---- key range: all sk keys, or the head's valid count (keys at or past it get a -inf mask term, whole
   // tiles past it are not visited; a count of 0 visits one tile that is masked throughout: O = 0, LSE = -inf)
-  int skv = a.sk;
-  if (a.kv_len) {
-    const int n = a.kv_len[bh / a.kv_div];
-    skv = n < 0 ? 0 : (n < a.sk ? n : a.sk);
-  }
+  const int skv = visible_keys<STRIDED>(a, bh);
   int nkt = (skv + BK - 1) / BK;
   if (nkt < 1) nkt = 1;
   if (CAUSAL) {

@@ -240,11 +240,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     if (CAUSAL && ((idx / G) & 1) == 0) it.qt = a.nqt - 1 - it.qt;
     // keys this head may see at all: [0, sk) or its valid count (possibly 0: then every key is
     // treated as past the end, which yields O = 0 and LSE = -inf)
-    int sk = a.sk;
-    if (a.kv_len) {
-      const int n = a.kv_len[it.bh / a.kv_div];
-      sk = n < 0 ? 0 : (n < sk ? n : sk);
-    }
+    const int sk = visible_keys<STRIDED>(a, it.bh);
     int nkt = (sk + BK - 1) / BK;
     if (nkt < 1) nkt = 1;
     if (CAUSAL) {

@@ -42,6 +42,21 @@ def test_strerror_and_threshold():
     assert L.fmha_bwd_noalloc_max_rows() * 4 == 8 << 20
 
 
+def test_workspace_query_without_a_gpu_says_no_pieces():
+    """Where the device cannot be asked for its size (no GPU here) the forward never asks for a workspace,
+    and nonsense parameter blocks get 0, not a crash."""
+    L = capi.lib()
+    P = capi.FwdParams()
+    P.bh, P.sq, P.sk, P.d, P.scale = 4, 1, 8192, 64, 0.125
+    if not torch.cuda.is_available():
+        assert L.fmha_fwd_workspace_bytes(C.byref(P)) == 0
+    P.d = 12
+    assert L.fmha_fwd_workspace_bytes(C.byref(P)) == 0
+    P.struct_bytes = 8
+    assert L.fmha_fwd_workspace_bytes(C.byref(P)) == 0
+    assert L.fmha_fwd_workspace_bytes(None) == 0
+
+
 def _valid_params():
     P = capi.FwdParams()
     P.q = P.k = P.v = P.o = 0x1000  # never dereferenced: every call below fails validation first
