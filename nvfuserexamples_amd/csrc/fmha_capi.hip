@@ -96,8 +96,7 @@ int cu_count() {
 // ---- A forward whose key range is cut into pieces (few heads, long key ranges: decode steps) ----
 // With one to a few query rows per head and fewer heads than the chip has room for workgroups, a launch
 // by head leaves most compute units idle while each busy one streams a whole K and V.  Such a forward
-// runs as `pieces` forwards over `chunk` keys each (the kernels see bh * pieces heads: RowMap's third
-// level), which write normalised partial outputs and their log-sum-exps into the caller's workspace,
+// runs as `pieces` forwards over `chunk` keys each (the kernels see bh * pieces heads: FwdArgs::pieces), which write normalised partial outputs and their log-sum-exps into the caller's workspace,
 // and a second launch merges them:  O = sum_c w_c O_c,  w_c = exp(LSE_c - LSE),  LSE = log sum_c exp(LSE_c).
 constexpr int kMaxPieces = 64; // what the merge kernel holds in LDS
 struct SplitPlan {
@@ -286,9 +285,6 @@ static int built_head_dim(int d) { return d <= 64 ? 64 : d <= 128 ? 128 : 256; }
 static int make_row_map(RowMap &m, int32_t heads, const int64_t st[3], int32_t bh, int32_t rows, int32_t d,
                         bool &strided) {
   m.heads_rcp = 0;
-  m.sp = 0;
-  m.pieces = 1;
-  m.pieces_rcp = 0;
   if (heads == 0) {
     m.sb = (int64_t)rows * d;
     m.sh = 0;
@@ -345,14 +341,9 @@ static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const Sp
   b.sk = pl.chunk;
   b.drop = make_drop_ctx(0, 0, 0.f, p->sq, pl.chunk);
   b.clock_probe = nullptr;
-  const uint32_t rcp = (uint32_t)((1ull << 32) / (uint64_t)pl.pieces) + 1u;
-  for (RowMap *m : {&b.mq, &b.mk, &b.mv}) {
-    m->pieces = pl.pieces;
-    m->pieces_rcp = rcp;
-  }
-  b.mq.sp = 0;
-  b.mk.sp = (int64_t)pl.chunk * a.mk.ss;
-  b.mv.sp = (int64_t)pl.chunk * a.mv.ss;
+  b.pieces = pl.pieces;
+  b.pieces_rcp = (uint32_t)((1ull << 32) / (uint64_t)pl.pieces) + 1u;
+  b.piece_stride = (int64_t)pl.chunk * a.mk.ss; // (k and v rows are equally far apart)
   b.mo.heads = 1; // the partial outputs: [bh * pieces, sq, d] contiguous
   b.mo.heads_rcp = 0;
   b.mo.sb = (int64_t)p->sq * p->d;
@@ -467,7 +458,10 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   if (!overrides().mask_trim) a.flags |= kFwdFlagNoTrim;
   a.kv_len = p->kv_len;
   a.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
+  a.pieces = 0;
+  a.pieces_rcp = 0;
   a.sk_whole = 0;
+  a.piece_stride = 0;
   a.clock_probe = (unsigned long long *)p->clock_probe;
   int mrc;
   bool strided = false;

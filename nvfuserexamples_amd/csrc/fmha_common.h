@@ -152,26 +152,13 @@ FMHA_DEV void dma_global_to_lds_b128(const void *uniform_base, uint32_t lane_off
 // ss = D; a [B, rows, H, D] tensor is heads = H, sb = rows * H * D, sh = D, ss = H * D.
 // heads_rcp = floor(2^32 / heads) + 1 turns the division into a multiplication (exact while
 // bh * heads < 2^32, which the host checks); offsets inside one head fit 31 bits (also checked).
-// Optional third level, for a key range that is cut into `pieces` runs of rows which the kernels treat as
-// heads of their own: head index = real head * pieces + piece, and piece c starts sp * c elements into the
-// real head's rows (sp = 0 for a tensor every piece shares, such as q).  pieces = 1: no third level.
 struct RowMap {
   int64_t sb, sh, ss;
   int32_t heads;
   uint32_t heads_rcp;
-  int64_t sp;
-  int32_t pieces;
-  uint32_t pieces_rcp; // floor(2^32 / pieces) + 1
   FMHA_DEV size_t head(int bh) const {
-    uint32_t i = (uint32_t)bh;
-    size_t off = 0;
-    if (pieces > 1) {
-      const uint32_t r = __umulhi(i, pieces_rcp);
-      off = (size_t)(i - r * (uint32_t)pieces) * (size_t)sp;
-      i = r;
-    }
-    const uint32_t b = heads == 1 ? i : __umulhi(i, heads_rcp);
-    return off + (size_t)b * (size_t)sb + (size_t)(i - b * (uint32_t)heads) * (size_t)sh;
+    const uint32_t b = heads == 1 ? (uint32_t)bh : __umulhi((uint32_t)bh, heads_rcp);
+    return (size_t)b * (size_t)sb + (size_t)((uint32_t)bh - b * (uint32_t)heads) * (size_t)sh;
   }
 };
 // Kernels are built twice: for the folded contiguous layout, whose strides are compile-time

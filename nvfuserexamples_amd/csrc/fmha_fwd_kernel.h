@@ -64,7 +64,14 @@ struct FwdArgs {
   int32_t flags;
   const int32_t *kv_len; // optional valid key count per group of kv_div heads (not with tensor dropout / saved outputs)
   int32_t kv_div;
-  int32_t sk_whole;      // key range cut into pieces (mk.pieces > 1): its whole length; sk is then the length of a piece
+  // A key range cut into pieces that run as heads of their own (run-time layouts only; pieces <= 1: off).
+  // Head index = real head * pieces + piece; q, k, v (and kv_len) belong to the real head, piece c starts
+  // piece_stride * c elements into the real head's k and v rows and covers sk of the sk_whole keys; o, lse
+  // and the mask are indexed by the head index as always.
+  int32_t pieces;
+  uint32_t pieces_rcp;   // floor(2^32 / pieces) + 1
+  int32_t sk_whole;
+  int64_t piece_stride;
   unsigned long long *clock_probe; // optional: counters at the start and end of workgroup 0 (pipelined kernel only)
   RowMap mq, mk, mv, mo; // row layout of q, k, v, o (mk.ss == mv.ss)
   int32_t dcols;         // elements per row that exist (<= the kernel's head dim; run-time layouts only)
@@ -85,24 +92,29 @@ enum { kFwdFlagNoTrim = 1 }; // visit every key tile even where a per-key mask h
 // how the mask tensor is read
 enum { kMaskNone = 0, kMaskPerKey = 1, kMaskFull = 2 };
 
-// Keys head `bh` may see at all: all sk, or the head's valid count (possibly 0).  With the key range cut into
-// pieces that run as heads of their own (RowMap::pieces of k; counts are per real head), what is left of
-// either in this head's piece.
-template <bool STRIDED> FMHA_DEV int visible_keys(const FwdArgs &a, int bh) {
-  int whole = a.sk, head = bh, first = 0;
+// Head index -> (real head, first key of its piece); see FwdArgs::pieces.
+template <bool STRIDED> FMHA_DEV void real_head(const FwdArgs &a, int bh, int &head, int &piece) {
+  head = bh;
+  piece = 0;
   if constexpr (STRIDED) {
-    if (a.mk.pieces > 1) {
-      head = (int)__umulhi((uint32_t)bh, a.mk.pieces_rcp);
-      first = (bh - head * a.mk.pieces) * a.sk;
-      whole = a.sk_whole;
+    if (a.pieces > 1) {
+      head = (int)__umulhi((uint32_t)bh, a.pieces_rcp);
+      piece = bh - head * a.pieces;
     }
   }
-  int n = whole;
+}
+// Keys a head may see at all: all sk, or the real head's valid count (possibly 0); of a piece: what is left
+// of either in it.
+template <bool STRIDED> FMHA_DEV int visible_keys(const FwdArgs &a, int head, int piece) {
+  int n = a.sk;
+  if constexpr (STRIDED) {
+    if (a.pieces > 1) n = a.sk_whole;
+  }
   if (a.kv_len) {
     const int m = a.kv_len[head / a.kv_div];
     n = m < 0 ? 0 : (m < n ? m : n);
   }
-  n -= first;
+  n -= piece * a.sk;
   return n < 0 ? 0 : (n < a.sk ? n : a.sk);
 }
 
@@ -175,9 +187,11 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   if (CAUSAL) qt = a.nqt - 1 - qt; // longest rows first
   const int q0w = qt * QT + w * (QB * 32);
 
-  const T *Qb = (const T *)a.q + RW::head(a.mq, bh, a.sq);
-  const T *Kb = (const T *)a.k + RW::head(a.mk, bh, a.sk);
-  const T *Vb = (const T *)a.v + RW::head(a.mv, bh, a.sk);
+  int rh, piece;
+  real_head<STRIDED>(a, bh, rh, piece);
+  const T *Qb = (const T *)a.q + RW::head(a.mq, rh, a.sq);
+  const T *Kb = (const T *)a.k + RW::head(a.mk, rh, a.sk) + (STRIDED ? (size_t)piece * (size_t)a.piece_stride : 0);
+  const T *Vb = (const T *)a.v + RW::head(a.mv, rh, a.sk) + (STRIDED ? (size_t)piece * (size_t)a.piece_stride : 0);
   const T *mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb : nullptr;
 
   // ---- Q' = Q * scale * log2(e) as B-operand registers
@@ -199,7 +213,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
 
   // ---- key range: all sk keys, or the head's valid count (keys at or past it get a -inf mask term, whole
   // tiles past it are not visited; a count of 0 visits one tile that is masked throughout: O = 0, LSE = -inf)
-  const int skv = visible_keys<STRIDED>(a, bh);
+  const int skv = visible_keys<STRIDED>(a, rh, piece);
   int nkt = (skv + BK - 1) / BK;
   if (nkt < 1) nkt = 1;
   if (CAUSAL) {

@@ -216,7 +216,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   // is padded to even (nkt2) with an all-masked phantom tile so that the two x / P buffers and
   // the two LDS stages alternate with fixed roles across items as well.
   struct Item {
-    int bh, qt, nkt2, kend;
+    int bh, rh, qt, nkt2, kend; // rh: the head q, k and v belong to (= bh unless the key range is cut into pieces)
     const T *Kb, *Vb, *mkey;
   };
   auto make_item = [&](int idx, int ord) {
@@ -240,7 +240,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     if (CAUSAL && ((idx / G) & 1) == 0) it.qt = a.nqt - 1 - it.qt;
     // keys this head may see at all: [0, sk) or its valid count (possibly 0: then every key is
     // treated as past the end, which yields O = 0 and LSE = -inf)
-    const int sk = visible_keys<STRIDED>(a, it.bh);
+    int piece;
+    real_head<STRIDED>(a, it.bh, it.rh, piece);
+    const int sk = visible_keys<STRIDED>(a, it.rh, piece);
     int nkt = (sk + BK - 1) / BK;
     if (nkt < 1) nkt = 1;
     if (CAUSAL) {
@@ -251,8 +253,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     }
     it.kend = nkt * BK < sk ? nkt * BK : sk;
     it.nkt2 = (nkt + 1) & ~1;
-    it.Kb = (const T *)a.k + RW::head(a.mk, it.bh, a.sk);
-    it.Vb = (const T *)a.v + RW::head(a.mv, it.bh, a.sk);
+    const size_t poff = STRIDED ? (size_t)piece * (size_t)a.piece_stride : 0;
+    it.Kb = (const T *)a.k + RW::head(a.mk, it.rh, a.sk) + poff;
+    it.Vb = (const T *)a.v + RW::head(a.mv, it.rh, a.sk) + poff;
     it.mkey = (MASK == kMaskPerKey) ? (const T *)a.mask + (size_t)mrow * a.mask_sb : nullptr;
     return it;
   };
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
   auto q_row = [&](const Item &it, int qb) {
     int q = it.qt * QT + w * (QB * 32) + qb * 32 + ql;
     q = q < a.sq ? q : a.sq - 1; // rows past the end repeat the last valid row and are never stored
-    return (const T *)a.q + RW::head(a.mq, it.bh, a.sq) + (size_t)q * RW::ss(a.mq) + h * 8;
+    return (const T *)a.q + RW::head(a.mq, it.rh, a.sq) + (size_t)q * RW::ss(a.mq) + h * 8;
   };
   auto dmaQ = [&](const Item &it) {
 #pragma unroll
