@@ -223,6 +223,12 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
     if (need < nkt) nkt = need;
   }
 
+  // rows of K and V that exist from Kb / Vb on: all sk, or what the whole key range leaves for this piece (>= 1)
+  int krows = a.sk;
+  if constexpr (STRIDED) {
+    if (a.pieces > 1 && a.sk_whole - piece * a.sk < krows) krows = a.sk_whole - piece * a.sk;
+  }
+
   // ---- tile staging: global -> registers -> LDS
   u32x4 kst[CPT], vst[CPT];
   T mraw = (T)0.f;     // raw per-key mask element in flight (converted when it is written to LDS,
@@ -235,7 +241,7 @@ __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
       // keys past the end re-read the last row: their scores get -inf through the extra step, so P = 0
       // meets finite values of V (unconditional loads do not stall on each other)
       int kr = k0 + row;
-      kr = kr < a.sk ? kr : a.sk - 1;
+      kr = kr < krows ? kr : krows - 1;
       const int cc = col * 8 < RW::cols(a) ? col * 8 : 0; // padding chunks: zeroed when they are written to LDS
       kst[i] = *(const u32x4 *)(Kb + (size_t)kr * RW::ss(a.mk) + cc);
       vst[i] = *(const u32x4 *)(Vb + (size_t)kr * RW::ss(a.mv) + cc);

@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 
 O_TOL = {"fp16": 2e-3, "bf16": 2e-2}
 SELF_TOL = {"fp16": 1.5e-3, "bf16": 1.2e-2}   # one more rounding of values up to ~1: 2^-11 resp. 2^-8, both ways
-STD = {64: 1.0, 96: 0.7, 128: 0.5, 256: 0.35}
+STD = {64: 1.0, 96: 0.7, 128: 0.5, 200: 0.35, 256: 0.35}
 
 
 @pytest.fixture
@@ -195,3 +195,24 @@ def test_operator_allocates_the_workspace_itself():
     torch.cuda.synchronize()
     for a, b in ((qg.grad, dq0), (kg.grad, dk0), (vg.grad, dv0)):
         assert (a.float() - b.float()).abs().max().item() <= 2e-3 * max(1.0, b.float().abs().max().item())
+
+
+@pytest.mark.parametrize("d", [64, 200])
+def test_ragged_last_piece_reads_no_row_past_the_end(d, pieces):
+    """The last piece of the last head has fewer rows than the others (300 keys = 256 + 44): K and V sit at the
+    end of buffers whose tails hold NaN, so a row read past the 300th would poison the output (head dim 200
+    runs on the plain forward loop, 64 on the pipelined one)."""
+    bh, sq, sk = 4, 129, 300
+    q, k, v = make_qkv(bh, sq, sk, d, seed=17, std=STD[d])
+    bufs = []
+    for t in (k, v):
+        buf = torch.full((bh * sk + 1024, d), float("nan"), dtype=torch.float16, device="cuda")
+        buf[:bh * sk] = t.reshape(bh * sk, d).cuda()
+        bufs.append(buf)
+    kc, vc = (b[:bh * sk].view(bh, sk, d) for b in bufs)
+    pieces(2)
+    o, lse, _, _ = capi.fwd(q.cuda(), kc, vc, want_lse=True)
+    torch.cuda.synchronize()
+    ref = oracle.attention(f32(q), f32(k), f32(v), want=("o", "lse"))
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= O_TOL["fp16"]

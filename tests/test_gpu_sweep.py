@@ -17,6 +17,7 @@ that.  Hence |dQ_id| <= scale * u * A_i * |K_kd| and, the signs of the row error
 |dK_kd| is of the order scale * u * sqrt(sum_i A_i^2) * max|Q|.  Such all-zero gradients are judged on
 ABSOLUTE error against 4 * scale * u * sqrt(sum_i A_i^2) * max(|Q|, |K|) instead of relative to a
 maximum that does not exist."""
+import os
 import random
 
 import numpy as np
@@ -129,6 +130,21 @@ def _run_case(it, c, rng):
     assert np.array_equal(np.isfinite(gl), fin), "lse: -inf rows differ"
     if fin.any():
         assert np.abs(gl[fin] - ref["lse"][fin]).max() <= 5e-3 + 2.0 ** -8 * np.abs(ref["lse"][fin]).max(), "lse"
+    # the same forward with its key range cut into pieces (decode steps take this route by themselves; here it is
+    # forced on every third eligible problem): same bars, one more rounding of the partial outputs included
+    pr = random.Random(it * 7919 + 13)
+    if not causal and not p and maskk != "full" and sk > 128 and pr.random() < 0.34:
+        os.environ["FMHA_FWD_SPLIT"] = str(pr.choice([2, 3, 5]))
+        try:
+            o3, lse3, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, **kw)
+            torch.cuda.synchronize()
+        finally:
+            del os.environ["FMHA_FWD_SPLIT"]
+        assert np.abs(f32(o3.reshape(bh, sq, d).cpu()) - ref["o"]).max() <= otol, "o in pieces"
+        gl3 = lse3.reshape(bh, sq).cpu().numpy()
+        assert np.array_equal(np.isfinite(gl3), fin), "lse in pieces: -inf rows differ"
+        if fin.any():
+            assert np.abs(gl3[fin] - ref["lse"][fin]).max() <= 5e-3 + 2.0 ** -8 * np.abs(ref["lse"][fin]).max(), "lse in pieces"
 
 
 # problems whose gradients with respect to q and k are zero throughout (every query sees one key)
