@@ -78,3 +78,31 @@ def test_reference_operators_replay_from_a_graph():
         torch.cuda.synchronize()
         for a, b_ in zip(got, want):
             assert torch.equal(a, b_), r
+
+
+def test_decode_step_in_pieces_replays_from_a_graph():
+    """A decode step whose key range runs in pieces (mask regrouping, the forward on the pieces, the merge; the
+    operator allocates the workspace inside the capture) with valid key counts that change between replays."""
+    from nvfuserexamples_amd import load_ops
+    ops = load_ops()
+    b, h, sk, d = 2, 4, 4096, 128
+    q, k, v = (t.cuda() for t in make_qkv(b * h, 1, sk, d, seed=3, std=0.5))
+    m = pad_mask(b, sk, sk // 2, sk).half().cuda()
+    lens = torch.tensor([sk, sk // 3], dtype=torch.int32, device="cuda")
+
+    def step():
+        return ops.fmha_fwd(q, k, v, m, 0.0, False, 0.0, 0, 0, lens)
+
+    g, outs = _capture(step)
+    for r in range(4):
+        fresh = [t.cuda() for t in make_qkv(b * h, 1, sk, d, seed=20 + r, std=0.5)]
+        for dst, src in zip((q, k, v), fresh):
+            dst.copy_(src)
+        lens.copy_(torch.tensor([sk - 500 * r, 100 + 700 * r], dtype=torch.int32))
+        g.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()
+        torch.cuda.synchronize()
+        for a, b_ in zip(got, want):
+            assert torch.equal(a, b_), r
