@@ -457,6 +457,7 @@ DECODE_SHAPES = {  # name: (heads, query rows, keys, head dim)
     "BH64_Sk8192_D128": (64, 1, 8192, 128),
     "BH8_Sk131072_D128": (8, 1, 131072, 128),
     "BH128_Sk16384_D64": (128, 1, 16384, 64),
+    "BH512_Sk4096_D128": (512, 1, 4096, 128),   # enough heads to fill the chip: never cut
 }
 
 
@@ -473,9 +474,10 @@ def decode_sets(torch, bh, sq, sk, d):
 
 
 def decode_leg(torch, capi, steps, warmup):
-    """Decode steps (one query row per head against a long fp16 K/V cache, no mask): HBM-bound, the bytes are K
-    and V once.  `plain` is the launch by head, `pieces` the same call with a workspace, where the library
-    cuts the key range so that the whole chip streams.  Never part of `value`."""
+    """Decode steps (one query row per head against a long fp16 K/V cache, no mask) on the decode kernel: HBM-bound,
+    the bytes are K and V once.  `plain` is the launch by head, `pieces` the same call with a workspace, where the
+    library cuts the key range so that the whole chip streams (not needed, and not done, with enough heads).
+    Never part of `value`."""
     out = {}
     for name, (bh, sq, sk, d) in DECODE_SHAPES.items():
         sets = decode_sets(torch, bh, sq, sk, d)

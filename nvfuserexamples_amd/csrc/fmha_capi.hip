@@ -3,6 +3,7 @@
 #include "../../include/fmha_capi.h"
 #include "fmha_launch.h"
 #include "fmha_fwd_fp8.h"
+#include "fmha_fwd_decode.h"
 
 #include <atomic>
 #include <cmath>
@@ -10,6 +11,7 @@
 #include <cstring>
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 using namespace fmha;
 
@@ -51,10 +53,11 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
 // pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
 // that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call), FMHA_FWD_SPLIT=0 never cuts a
-// forward's key range into pieces, FMHA_FWD_SPLIT=n (2..64) cuts it into about n wherever pieces are possible.
+// forward's key range into pieces, FMHA_FWD_SPLIT=n (2..64) cuts it into about n wherever pieces are possible,
+// FMHA_FWD_DECODE=0 keeps forwards of one to four query rows on the matrix-pipe kernels.
 // The environment is read once per process (on the first launch); fmha_reload_overrides() reads it again.
 struct Overrides {
-  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, bwd_pair, bwd_short, bwd_fused;
+  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, fwd_decode, bwd_pair, bwd_short, bwd_fused;
 };
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
@@ -68,6 +71,7 @@ Overrides read_overrides() {
   o.fwd_stream = env_int("FMHA_FWD_STREAM", 1);
   o.fwd_qb = env_int("FMHA_FWD_QB", 0);
   o.fwd_split = env_int("FMHA_FWD_SPLIT", -1);
+  o.fwd_decode = env_int("FMHA_FWD_DECODE", 1);
   o.bwd_pair = env_int("FMHA_BWD_PAIR", -1);
   o.bwd_short = env_int("FMHA_BWD_SHORT", 1);
   o.bwd_fused = env_int("FMHA_BWD_FUSED", 0);
@@ -106,8 +110,19 @@ struct SplitPlan {
 
 size_t round256(size_t x) { return (x + 255u) & ~(size_t)255u; }
 
+// Forwards the decode kernel serves (fmha_fwd_decode.h): one to four query rows, head dim 64 or 128, no causal
+// mask, dropout or saved outputs, no mask or one that is constant along the queries.
+bool decode_eligible(const fmha_fwd_params *p) {
+  return overrides().fwd_decode != 0 && p->sq <= 4 && (p->d == 64 || p->d == 128) && !p->causal &&
+         p->drop_kind == FMHA_DROP_NONE && !p->save_softmax && !p->save_dropout &&
+         (p->mask_kind == FMHA_MASK_NONE || p->mask_stride_q == 0);
+}
+
 // Whether the forward described by p (already validated) runs in pieces, and where its intermediates go.
+// The decode kernel's pieces are fp32 and read the caller's mask where it is; the matrix-pipe kernels' pieces
+// have the element type and a regrouped copy of the mask.
 bool plan_split(const fmha_fwd_params *p, SplitPlan &pl) {
+  const bool decode = decode_eligible(p);
   const int force = overrides().fwd_split;
   if (force == 0) return false;
   if (p->causal || p->drop_kind != FMHA_DROP_NONE || p->save_softmax || p->save_dropout) return false;
@@ -138,11 +153,11 @@ bool plan_split(const fmha_fwd_params *p, SplitPlan &pl) {
   pl.pieces = (int)pieces;
   pl.chunk = (int)chunk;
   const size_t vh = (size_t)p->bh * (size_t)pieces;
-  size_t off = round256(vh * (size_t)sq * (size_t)p->d * 2u);
+  size_t off = round256(vh * (size_t)sq * (size_t)p->d * (decode ? 4u : 2u));
   pl.off_lse = off;
   off += round256(vh * (size_t)sq * sizeof(float));
   pl.off_mask = off;
-  if (p->mask_kind != FMHA_MASK_NONE) off += round256(vh * (size_t)chunk * 2u);
+  if (p->mask_kind != FMHA_MASK_NONE && !decode) off += round256(vh * (size_t)chunk * 2u);
   pl.bytes = off;
   return true;
 }
@@ -170,9 +185,9 @@ __global__ void split_mask_kernel(uint16_t *mask_out, const uint16_t *mask_in, i
 // (t % cpr) and every (kMergeThreads / cpr)-th piece, so that the loads of all pieces are in flight together
 // (a thread walking the pieces one after the other pays a trip to memory per piece); the threads' sums meet in LDS.
 constexpr int kMergeThreads = 256;
-template <typename T>
+template <typename T, typename TP>
 __global__ void __launch_bounds__(kMergeThreads)
-split_merge_kernel(const T *o_part, const float *lse_part, T *o, float *lse, RowMap mo, int32_t sq, int32_t d,
+split_merge_kernel(const TP *o_part, const float *lse_part, T *o, float *lse, RowMap mo, int32_t sq, int32_t d,
                    int32_t pieces) {
   __shared__ float s_lse[kMaxPieces];
   __shared__ float s_acc[kMergeThreads][9];
@@ -192,16 +207,21 @@ split_merge_kernel(const T *o_part, const float *lse_part, T *o, float *lse, Row
       const float l = s_lse[c];
       if (l == -INFINITY) continue; // an empty piece
       const float w = expf(l - m);
-      Pack16 x;
-      x.u = *(const u32x4 *)(o_part + (row0 + (size_t)c * sq) * d + c8 * 8);
+      const TP *src = o_part + (row0 + (size_t)c * sq) * d + c8 * 8;
+      float xv[8];
+      if constexpr (__is_same(TP, float)) {
+        const f32x4 lo = *(const f32x4 *)src, hi = *(const f32x4 *)(src + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          xv[e] = lo[e];
+          xv[4 + e] = hi[e];
+        }
+      } else {
+        unpack8<TP>(*(const u32x4 *)src, xv);
+      }
       acc[8] += w;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float xv;
-        if constexpr (__is_same(T, _Float16)) xv = (float)x.h[e];
-        else xv = (float)x.b[e];
-        acc[e] += w * xv;
-      }
+      for (int e = 0; e < 8; ++e) acc[e] += w * xv[e];
     }
   }
 #pragma unroll
@@ -312,6 +332,56 @@ static int fwd_dispatch_strided(FwdArgs &a, const FwdVariant &v, int dtype, int 
   return D == 64 ? fwd_dispatch_bf16_d64_strided(a, v, s) : D == 128 ? fwd_dispatch_bf16_d128_strided(a, v, s) : fwd_dispatch_bf16_d256_strided(a, v, s);
 }
 
+// The merge of `pieces` partial results (fp32 from the decode kernel, element type otherwise) into o and lse.
+template <bool F32> static int merge_launch(const fmha_fwd_params *p, const void *o_part, const float *lse_part,
+                                            const RowMap &mo, int pieces, hipStream_t s) {
+  const dim3 grid((unsigned)((long long)p->bh * p->sq)), block(kMergeThreads);
+  if (p->dtype == FMHA_DTYPE_F16) {
+    using TP = std::conditional_t<F32, float, _Float16>;
+    hipLaunchKernelGGL((split_merge_kernel<_Float16, TP>), grid, block, 0, s, (const TP *)o_part, lse_part,
+                       (_Float16 *)p->o, p->lse, mo, p->sq, p->d, pieces);
+  } else {
+    using TP = std::conditional_t<F32, float, __bf16>;
+    hipLaunchKernelGGL((split_merge_kernel<__bf16, TP>), grid, block, 0, s, (const TP *)o_part, lse_part, (__bf16 *)p->o,
+                       p->lse, mo, p->sq, p->d, pieces);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// One to four query rows (decode_eligible): the decode kernel on the whole key range, or -- with a plan -- on its
+// pieces, followed by the merge.
+static int fwd_decode_launch(const fmha_fwd_params *p, const FwdArgs &a, const SplitPlan *pl, hipStream_t s) {
+  DecodeArgs d;
+  d.q = a.q; d.k = a.k; d.v = a.v;
+  d.o = a.o;
+  d.lse = a.lse;
+  d.o_part = nullptr;
+  d.lse_part = nullptr;
+  d.mask = a.mask;
+  d.mask_sb = a.mask_sb;
+  d.mask_div = a.mask_div;
+  d.mask_a = a.mask_a;
+  d.mask_b = a.mask_b;
+  d.kv_len = a.kv_len;
+  d.kv_div = a.kv_div;
+  d.bh = p->bh; d.sq = p->sq; d.sk = p->sk;
+  d.pieces = 1;
+  d.chunk = p->sk;
+  d.scale_l2 = a.scale_l2;
+  d.mq = a.mq; d.mk = a.mk; d.mv = a.mv; d.mo = a.mo;
+  if (pl) {
+    unsigned char *ws = (unsigned char *)p->workspace;
+    d.pieces = pl->pieces;
+    d.chunk = pl->chunk;
+    d.o_part = (float *)ws;
+    d.lse_part = (float *)(ws + pl->off_lse);
+  }
+  const int rc = fwd_decode_dispatch(d, p->d, p->dtype == FMHA_DTYPE_BF16, s);
+  if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
+  if (pl && merge_launch<true>(p, d.o_part, d.lse_part, a.mo, pl->pieces, s) != 0) return FMHA_E_LAUNCH;
+  return FMHA_OK;
+}
+
 // The forward in pieces (plan_split): a per-key mask's rows regrouped by piece, the forward kernels over bh * pieces
 // heads of `chunk` keys on the run-time-layout code path, then the merge.  `a` describes the whole launch.
 static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const SplitPlan &pl, int D, hipStream_t s) {
@@ -358,15 +428,7 @@ static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const Sp
   const int rc = fwd_dispatch_strided(b, v, p->dtype, D, s);
   if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
   {
-    const long long rows = (long long)p->bh * p->sq;
-    const dim3 grid((unsigned)rows);
-    if (p->dtype == FMHA_DTYPE_F16)
-      hipLaunchKernelGGL(split_merge_kernel<_Float16>, grid, dim3(kMergeThreads), 0, s, (const _Float16 *)ws, lse_part,
-                         (_Float16 *)p->o, p->lse, a.mo, p->sq, p->d, pl.pieces);
-    else
-      hipLaunchKernelGGL(split_merge_kernel<__bf16>, grid, dim3(kMergeThreads), 0, s, (const __bf16 *)ws, lse_part,
-                         (__bf16 *)p->o, p->lse, a.mo, p->sq, p->d, pl.pieces);
-    if (hipGetLastError() != hipSuccess) return FMHA_E_LAUNCH;
+    if (merge_launch<false>(p, ws, lse_part, a.mo, pl.pieces, s) != 0) return FMHA_E_LAUNCH;
   }
   return FMHA_OK;
 }
@@ -476,8 +538,10 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
 
   hipStream_t s = (hipStream_t)hip_stream;
   SplitPlan pl;
-  if (p->workspace && ((uintptr_t)p->workspace & 15u) == 0 && plan_split(p, pl) && p->workspace_bytes >= pl.bytes)
-    return fwd_split_launch(p, a, pl, D, s);
+  const bool split = p->workspace && ((uintptr_t)p->workspace & 15u) == 0 && plan_split(p, pl) &&
+                     p->workspace_bytes >= pl.bytes;
+  if (decode_eligible(p)) return fwd_decode_launch(p, a, split ? &pl : nullptr, s);
+  if (split) return fwd_split_launch(p, a, pl, D, s);
 
   FwdVariant v;
   v.mask = a.mask == nullptr ? kMaskNone : (a.mask_sq == 0 ? kMaskPerKey : kMaskFull);

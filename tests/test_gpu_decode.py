@@ -28,13 +28,20 @@ STD = {64: 1.0, 96: 0.7, 128: 0.5, 200: 0.35, 256: 0.35}
 
 @pytest.fixture
 def pieces(monkeypatch):
-    def force(n):
+    """force(n): about n pieces (None: the library's own choice); force(n, decode_kernel=False) also keeps
+    launches of one to four query rows off the decode kernel, on the matrix-pipe kernels."""
+    def force(n, decode_kernel=True):
         if n is None:
             monkeypatch.delenv("FMHA_FWD_SPLIT", raising=False)
         else:
             monkeypatch.setenv("FMHA_FWD_SPLIT", str(n))
+        if decode_kernel:
+            monkeypatch.delenv("FMHA_FWD_DECODE", raising=False)
+        else:
+            monkeypatch.setenv("FMHA_FWD_DECODE", "0")
     yield force
     monkeypatch.delenv("FMHA_FWD_SPLIT", raising=False)
+    monkeypatch.delenv("FMHA_FWD_DECODE", raising=False)
     capi.lib().fmha_reload_overrides()
 
 
@@ -59,6 +66,9 @@ CASES = [
     (2, 1, 1500, 96, "fp16", 4, None, False),          # a head dim between the built ones
     (2, 2, 1100, 256, "bf16", 3, "pad", True),         # head dim 256: the plain forward loop
     (2, 1, 2048, 64, "fp16", 64, None, False),         # as many pieces as there are 128-key runs
+    (5, 2, 777, 128, "bf16", 2, "perhead", True),      # two query rows
+    (4, 4, 1234, 64, "fp16", 3, "pad", True),          # four
+    (3, 3, 333, 128, "fp16", 2, None, False),          # three (run as four)
 ]
 
 
@@ -92,13 +102,18 @@ def _oracle_mask(m, lens, bh, sq, sk):
     return full.numpy()
 
 
+@pytest.mark.parametrize("decode_kernel", [True, False])
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,force,mask,kvl", CASES)
-def test_pieces_match_oracle_and_plain_launch(bh, sq, sk, d, dtype, force, mask, kvl, pieces):
+def test_pieces_match_oracle_and_plain_launch(bh, sq, sk, d, dtype, force, mask, kvl, decode_kernel, pieces):
+    """Rows of one to four queries at head dim 64 / 128 run on the decode kernel (fp32 pieces), everything else --
+    and everything with decode_kernel = False -- on the matrix-pipe kernels (pieces in the element type)."""
+    if not decode_kernel and (sq > 4 or d not in (64, 128)):
+        pytest.skip("not a decode-kernel shape: same route as with decode_kernel = True")
     q, k, v, m, lens = _inputs(bh, sq, sk, d, dtype, mask, kvl, seed=bh * 1000 + sk)
     tdt = q.dtype
     qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
     kw = dict(mask=None if m is None else m.to(tdt).cuda(), kv_len=None if lens is None else lens.cuda(), want_lse=True)
-    pieces(force)
+    pieces(force, decode_kernel)
     P = _params(bh, sq, sk, d, dtype=capi.F16 if dtype == "fp16" else capi.BF16)
     if m is not None:
         P.mask_kind, P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = capi.MASK_ADDITIVE, bh // m.shape[0], sk, 0
@@ -131,10 +146,12 @@ def test_run_time_layouts_and_too_small_workspaces(pieces):
     o0, lse0, _, _ = capi.fwd(q, k, v, kv_len=lens, want_lse=True, workspace=False)
     tiny = torch.empty(64, dtype=torch.uint8, device="cuda")
     o1, _, _, _ = capi.fwd(q, k, v, kv_len=lens, workspace=tiny)
+    big = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    o2, _, _, _ = capi.fwd(q, k, v, kv_len=lens, workspace=big)
     torch.cuda.synchronize()
     assert o.shape == o0.shape == (B, H, sq, d)
     assert torch.equal(o1, o0)
-    assert not torch.equal(o, o0)            # the pieces did run
+    assert torch.equal(o2, o) and big.any()  # the pieces did run: their partial results are in the workspace
     assert (o.float() - o0.float()).abs().max().item() <= SELF_TOL["fp16"]
     assert (lse - lse0).abs().max().item() <= 5e-4
     m = torch.zeros(B * H, sq, sk)
