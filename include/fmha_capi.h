@@ -157,16 +157,18 @@ typedef struct fmha_fwd_params {
 
   /* Optional device memory for a forward whose key range is cut into pieces (no counterpart in the
    * reference, whose shapes are fixed at 128 x 128 per head, fmha_manual.cpp:24-29).  A decode step -- one
-   * or a few query rows per head against a long key range -- on fewer heads than the chip holds workgroups
-   * would leave most compute units idle while each busy one streams a whole K and V.  Given a workspace of
-   * at least fmha_fwd_workspace_bytes(p) bytes (16-byte aligned), such a launch runs every piece of the
-   * key range as a head of its own, keeps the pieces' normalised outputs (element type = dtype) and
-   * log-sum-exps in the workspace and merges them in a second launch:
+   * or a few query rows per head against a long key range -- on fewer heads than the chip has compute units
+   * would leave most of them idle while each busy one streams a whole K and V.  Given a workspace of at
+   * least fmha_fwd_workspace_bytes(p) bytes (16-byte aligned), such a launch runs every piece of the key
+   * range as a workgroup (or head) of its own, keeps the pieces' normalised outputs and log-sum-exps in the
+   * workspace and merges them in a second launch:
    *   O = sum_c exp(LSE_c - LSE) O_c,   LSE = log sum_c exp(LSE_c).
-   * Results differ from the plain launch by one more rounding to the element type (of the partial
-   * outputs).  Pieces are used without a causal mask, dropout or saved outputs, with no mask or a mask that
-   * is constant along the queries, with or without kv_len; everything else, a NULL or too small workspace
-   * included, takes the plain launch.  The workspace may be reused by the next launch on the same stream. */
+   * Launches of one to four query rows at head dim 64 or 128 (which have a streaming kernel of their own,
+   * with or without pieces) keep their pieces in fp32; other shapes keep them in the element type, so their
+   * results differ from the plain launch by one more rounding to that type.  Pieces are used without a
+   * causal mask, dropout or saved outputs, with no mask or a mask that is constant along the queries, with
+   * or without kv_len; everything else, a NULL or too small workspace included, takes the plain launch.
+   * The workspace may be reused by the next launch on the same stream. */
   void *workspace;
   uint64_t workspace_bytes;
 } fmha_fwd_params;
@@ -297,7 +299,7 @@ float fmha_drop_scale(float p_drop);
 const char *fmha_strerror(int code);
 
 /* The FMHA_* environment variables -- tuning and test overrides of the variant selection: FMHA_MASK_TRIM,
- * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_BWD_SHORT, FMHA_BWD_PAIR,
+ * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_BWD_SHORT, FMHA_BWD_PAIR,
  * FMHA_BWD_FUSED -- are read once per process, on the first launch.  This reads them again; not to be
  * called while another thread is launching.  (No counterpart in the reference.) */
 void fmha_reload_overrides(void);
