@@ -57,6 +57,38 @@ def test_workspace_query_without_a_gpu_says_no_pieces():
     assert L.fmha_fwd_workspace_bytes(None) == 0
 
 
+@pytest.mark.parametrize("bh,sq,sk,d,n,masked", [
+    (4, 1, 4096, 64, 4, False), (3, 1, 1000, 128, 3, True), (2, 130, 520, 64, 2, True), (5, 3, 777, 96, 64, False),
+    (1, 1, 131072, 128, 200, False), (7, 4, 300, 256, 2, True)])
+def test_forced_pieces_size_their_workspace(bh, sq, sk, d, n, masked, monkeypatch):
+    """FMHA_FWD_SPLIT=n needs no device: about n pieces (at most 64) of a multiple of 128 keys.  The workspace
+    holds the partial outputs (fp32 for the decode kernel's shapes -- up to four query rows at head dim 64 /
+    128 -- else the element type), their log-sum-exps and, for the matrix-pipe kernels only, a regrouped copy
+    of a per-key mask; every part starts on a 256-byte boundary."""
+    monkeypatch.setenv("FMHA_FWD_SPLIT", str(n))
+    L = capi.lib()
+    L.fmha_reload_overrides()
+    try:
+        P = capi.FwdParams()
+        P.bh, P.sq, P.sk, P.d, P.scale = bh, sq, sk, d, 0.125
+        if masked:
+            P.mask_kind, P.mask_bh_div, P.mask_stride_b = capi.MASK_ADDITIVE, 1, sk
+        got = L.fmha_fwd_workspace_bytes(C.byref(P))
+        chunk = -(-(-(-sk // min(n, 64))) // 128) * 128
+        pieces = -(-sk // chunk)
+        decode = sq <= 4 and d in (64, 128)
+        r256 = lambda x: (x + 255) // 256 * 256
+        want = r256(bh * pieces * sq * d * (4 if decode else 2)) + r256(bh * pieces * sq * 4)
+        if masked and not decode:
+            want += r256(bh * pieces * chunk * 2)
+        assert pieces >= 2 and got == want
+        P.causal = 1
+        assert L.fmha_fwd_workspace_bytes(C.byref(P)) == 0
+    finally:
+        monkeypatch.delenv("FMHA_FWD_SPLIT")
+        L.fmha_reload_overrides()
+
+
 def _valid_params():
     P = capi.FwdParams()
     P.q = P.k = P.v = P.o = 0x1000  # never dereferenced: every call below fails validation first
