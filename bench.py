@@ -494,6 +494,23 @@ def decode_leg(torch, capi, steps, warmup):
                          "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)}
         out[name] = leg
         del sets, ws
+    # the same steps on an e4m3 cache (q, k, v e4m3, O fp16): half the bytes
+    for name in ("BH32_Sk32768_D128", "BH512_Sk4096_D128"):
+        bh, sq, sk, d = DECODE_SHAPES[name]
+        nset = max(2, int(600e6 // (2 * bh * sk * d)) + 1)
+        sets = [tuple(torch.randn(bh, s_, d, device="cuda").to(torch.float8_e4m3fn) for s_ in (sq, sk, sk))
+                for _ in range(nset)]
+        ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+        by = 2.0 * bh * sk * d + bh * sq * d * 3.0
+
+        def step8(i):
+            q8, k8, v8 = sets[i % len(sets)]
+            capi.fwd_fp8(q8, k8, v8, workspace=ws)
+        ms, _ = time_steps(torch, step8, steps, warmup, blocks=9)
+        out[name]["e4m3_cache"] = {"us": round(ms * 1e3, 1), "algorithmic_MB": round(by / 1e6, 1),
+                                   "TBps": round(by / (ms * 1e-3) / 1e12, 2),
+                                   "hbm_frac": round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)}
+        del sets, ws
     return out
 
 

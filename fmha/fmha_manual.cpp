@@ -442,7 +442,7 @@ fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, co
 std::tuple<at::Tensor, at::Tensor> fmha_fwd_fp8(const at::Tensor &q8, const at::Tensor &k8, const at::Tensor &v8,
                                                 double descale_q, double descale_k, double descale_v,
                                                 const c10::optional<at::Tensor> &mask, double scale, bool is_causal,
-                                                bool out_bf16) {
+                                                bool out_bf16, const c10::optional<at::Tensor> &kv_len) {
   for (const at::Tensor *t : {&q8, &k8, &v8})
     TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat8_e4m3fn && t->dim() == 3 && t->is_contiguous(),
                 "mha_manual: q, k, v must be contiguous [B*H,S,D] float8_e4m3fn GPU tensors");
@@ -476,6 +476,14 @@ std::tuple<at::Tensor, at::Tensor> fmha_fwd_fp8(const at::Tensor &q8, const at::
     p.mask = m.t.data_ptr();
     p.mask_bh_div = m.bh_div;
     p.mask_stride_b = m.stride_b;
+  }
+  // valid key counts and the key range in pieces: launches of one to four query rows (the decode kernel) only
+  at::Tensor kv_keep, workspace;
+  set_kv_len(p, kv_len, q8.size(0), kv_keep);
+  if (const uint64_t need = fmha_fwd_fp8_workspace_bytes(&p); need > 0) {
+    workspace = at::empty({static_cast<int64_t>(need)}, q8.options().dtype(at::kByte));
+    p.workspace = workspace.data_ptr();
+    p.workspace_bytes = need;
   }
   const int rc = fmha_fwd_fp8_launch(&p, current_stream(q8));
   TORCH_CHECK(rc == FMHA_OK, "mha_manual e4m3 forward: ", fmha_strerror(rc));
@@ -557,7 +565,7 @@ TORCH_LIBRARY(mha_manual, m) {
         "is_causal, float p_drop, int seed, int offset, Tensor? kv_len=None) -> (Tensor, Tensor, Tensor)");
   m.def("fmha_philox_keep_mask(Tensor like, int bh, int sq, int sk, float p_drop, int seed, int offset) -> Tensor");
   m.def("fmha_fwd_fp8(Tensor q8, Tensor k8, Tensor v8, float descale_q, float descale_k, float descale_v, Tensor? mask, "
-        "float scale, bool is_causal, bool out_bf16=False) -> (Tensor, Tensor)");
+        "float scale, bool is_causal, bool out_bf16=False, Tensor? kv_len=None) -> (Tensor, Tensor)");
 }
 
 // On ROCm builds of PyTorch the CUDA dispatch key is the HIP device's key.

@@ -206,9 +206,22 @@ typedef struct fmha_fwd_fp8_params {
   int32_t out_dtype; /* FMHA_DTYPE_F16 / FMHA_DTYPE_BF16 */
   float scale, descale_q, descale_k, descale_v;
   int32_t causal;
+  /* Decode steps on an e4m3 K/V cache: launches of one to four query rows without a causal mask run on the
+   * streaming kernel of the 16-bit decode steps (8-byte row loads, fp32 arithmetic), which keeps the
+   * probabilities in fp32 -- no e4m3 rounding of P~, so O = descale_v * softmax(y) v8 up to fp32 rounding --
+   * and moves half the bytes of the fp16 cache.  Such launches (and only they) also take valid key counts
+   * (kv_len, kv_len_bh_div) and a workspace (workspace, workspace_bytes, fmha_fwd_fp8_workspace_bytes), all
+   * as in fmha_fwd_params. */
+  const int32_t *kv_len;
+  int32_t kv_len_bh_div;
+  void *workspace;
+  uint64_t workspace_bytes;
 } fmha_fwd_fp8_params;
 
 int fmha_fwd_fp8_launch(const fmha_fwd_fp8_params *p, void *hip_stream);
+
+/* As fmha_fwd_workspace_bytes, for fmha_fwd_fp8_launch. */
+uint64_t fmha_fwd_fp8_workspace_bytes(const fmha_fwd_fp8_params *p);
 
 /*
  * Backward (no counterpart in the reference, which has no backward kernel:

@@ -19,7 +19,7 @@ DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
            "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides",
            "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale", "fmha_fwd_fp8_launch",
-           "fmha_fwd_workspace_bytes")
+           "fmha_fwd_workspace_bytes", "fmha_fwd_fp8_workspace_bytes")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
 _ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT", "FMHA_FWD_DECODE",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
@@ -94,6 +94,8 @@ class FwdFp8Params(_Params):
         ("out_dtype", C.c_int32),
         ("scale", C.c_float), ("descale_q", C.c_float), ("descale_k", C.c_float), ("descale_v", C.c_float),
         ("causal", C.c_int32),
+        ("kv_len", C.c_void_p), ("kv_len_bh_div", C.c_int32),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64),
     ]
 
 
@@ -123,6 +125,8 @@ def lib():
         L.fmha_bwd_launch.restype = C.c_int
         L.fmha_fwd_fp8_launch.argtypes = [C.POINTER(FwdFp8Params), C.c_void_p]
         L.fmha_fwd_fp8_launch.restype = C.c_int
+        L.fmha_fwd_fp8_workspace_bytes.argtypes = [C.POINTER(FwdFp8Params)]
+        L.fmha_fwd_fp8_workspace_bytes.restype = C.c_uint64
         L.fmha_bwd_launch_noalloc.argtypes = [C.POINTER(BwdParams), C.c_void_p]
         L.fmha_bwd_launch_noalloc.restype = C.c_int
         L.fmha_bwd_noalloc_max_rows.argtypes = []
@@ -367,10 +371,11 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
 
 
 def fwd_fp8(q8, k8, v8, descale_q=1.0, descale_k=1.0, descale_v=1.0, mask=None, causal=False, scale=None,
-            out_dtype=None, want_lse=False):
+            out_dtype=None, want_lse=False, kv_len=None, workspace=True):
     """Forward on e4m3 inputs (torch.float8_e4m3fn, contiguous [bh, s, d]) on the current stream.
     Returns (o, lse|None); o is float16 unless out_dtype says bfloat16.  mask: additive [bh|B, 1, sk] /
-    [B,1,1,sk] in o's dtype."""
+    [B,1,1,sk] in o's dtype.  kv_len (valid key counts, as in fwd) and workspace (as in fwd) apply to launches
+    of one to four query rows without a causal mask, which run on the streaming decode kernel."""
     import torch
     out_dtype = out_dtype or torch.float16
     for t in (q8, k8, v8):
@@ -395,6 +400,17 @@ def fwd_fp8(q8, k8, v8, descale_q=1.0, descale_k=1.0, descale_v=1.0, mask=None, 
         if mask.dtype != out_dtype or sqs != 0:
             raise FmhaError(-5, "the e4m3 forward takes a per-key mask ([.., 1, sk]) of o's dtype")
         P.mask, P.mask_bh_div, P.mask_stride_b = mask.data_ptr(), div, sb
+    _set_kv_len(P, kv_len, bh)
+    _sync_env()
+    ws = None
+    if workspace is True:
+        need = lib().fmha_fwd_fp8_workspace_bytes(C.byref(P))
+        if need:
+            ws = torch.empty(need, dtype=torch.uint8, device=q8.device)
+    elif workspace is not False and workspace is not None:
+        ws = workspace
+    if ws is not None:
+        P.workspace, P.workspace_bytes = ws.data_ptr(), ws.numel()
     check(lib().fmha_fwd_fp8_launch(C.byref(P), _stream_ptr()))
     return o, lse
 

@@ -333,17 +333,17 @@ static int fwd_dispatch_strided(FwdArgs &a, const FwdVariant &v, int dtype, int 
 }
 
 // The merge of `pieces` partial results (fp32 from the decode kernel, element type otherwise) into o and lse.
-template <bool F32> static int merge_launch(const fmha_fwd_params *p, const void *o_part, const float *lse_part,
-                                            const RowMap &mo, int pieces, hipStream_t s) {
-  const dim3 grid((unsigned)((long long)p->bh * p->sq)), block(kMergeThreads);
-  if (p->dtype == FMHA_DTYPE_F16) {
+template <bool F32> static int merge_launch(int dtype, void *o, float *lse, int bh, int sq, int d, const void *o_part,
+                                            const float *lse_part, const RowMap &mo, int pieces, hipStream_t s) {
+  const dim3 grid((unsigned)((long long)bh * sq)), block(kMergeThreads);
+  if (dtype == FMHA_DTYPE_F16) {
     using TP = std::conditional_t<F32, float, _Float16>;
     hipLaunchKernelGGL((split_merge_kernel<_Float16, TP>), grid, block, 0, s, (const TP *)o_part, lse_part,
-                       (_Float16 *)p->o, p->lse, mo, p->sq, p->d, pieces);
+                       (_Float16 *)o, lse, mo, sq, d, pieces);
   } else {
     using TP = std::conditional_t<F32, float, __bf16>;
-    hipLaunchKernelGGL((split_merge_kernel<__bf16, TP>), grid, block, 0, s, (const TP *)o_part, lse_part, (__bf16 *)p->o,
-                       p->lse, mo, p->sq, p->d, pieces);
+    hipLaunchKernelGGL((split_merge_kernel<__bf16, TP>), grid, block, 0, s, (const TP *)o_part, lse_part, (__bf16 *)o,
+                       lse, mo, sq, d, pieces);
   }
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
@@ -368,6 +368,7 @@ static int fwd_decode_launch(const fmha_fwd_params *p, const FwdArgs &a, const S
   d.pieces = 1;
   d.chunk = p->sk;
   d.scale_l2 = a.scale_l2;
+  d.out_scale = 1.f;
   d.mq = a.mq; d.mk = a.mk; d.mv = a.mv; d.mo = a.mo;
   if (pl) {
     unsigned char *ws = (unsigned char *)p->workspace;
@@ -378,7 +379,8 @@ static int fwd_decode_launch(const fmha_fwd_params *p, const FwdArgs &a, const S
   }
   const int rc = fwd_decode_dispatch(d, p->d, p->dtype == FMHA_DTYPE_BF16, s);
   if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
-  if (pl && merge_launch<true>(p, d.o_part, d.lse_part, a.mo, pl->pieces, s) != 0) return FMHA_E_LAUNCH;
+  if (pl && merge_launch<true>(p->dtype, p->o, p->lse, p->bh, p->sq, p->d, d.o_part, d.lse_part, a.mo, pl->pieces, s) != 0)
+    return FMHA_E_LAUNCH;
   return FMHA_OK;
 }
 
@@ -428,7 +430,8 @@ static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const Sp
   const int rc = fwd_dispatch_strided(b, v, p->dtype, D, s);
   if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
   {
-    if (merge_launch<false>(p, ws, lse_part, a.mo, pl.pieces, s) != 0) return FMHA_E_LAUNCH;
+    if (merge_launch<false>(p->dtype, p->o, p->lse, p->bh, p->sq, p->d, ws, lse_part, a.mo, pl.pieces, s) != 0)
+      return FMHA_E_LAUNCH;
   }
   return FMHA_OK;
 }
@@ -630,7 +633,27 @@ void *scratch_on_current_device() {
 int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_scratch);
 } // namespace
 
+// Whether an e4m3 forward (validated) runs on the decode kernel; `shape` then describes it to plan_split.
+static bool fp8_decode_shape(const fmha_fwd_fp8_params *p, fmha_fwd_params &shape) {
+  std::memset(&shape, 0, sizeof shape);
+  shape.bh = p->bh; shape.sq = p->sq; shape.sk = p->sk; shape.d = p->d;
+  shape.causal = p->causal;
+  shape.mask_kind = p->mask ? FMHA_MASK_ADDITIVE : FMHA_MASK_NONE;
+  return decode_eligible(&shape);
+}
+
 extern "C" {
+
+uint64_t fmha_fwd_fp8_workspace_bytes(const fmha_fwd_fp8_params *caller) {
+  if (!caller || caller->struct_bytes < offsetof(fmha_fwd_fp8_params, causal) + sizeof(int32_t)) return 0;
+  fmha_fwd_fp8_params local;
+  std::memset(&local, 0, sizeof local);
+  std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
+  if (local.bh <= 0 || local.sq <= 0 || local.sk <= 0 || (local.d != 64 && local.d != 128)) return 0;
+  fmha_fwd_params shape;
+  SplitPlan pl;
+  return fp8_decode_shape(&local, shape) && plan_split(&shape, pl) ? (uint64_t)pl.bytes : 0;
+}
 
 int fmha_fwd_fp8_launch(const fmha_fwd_fp8_params *caller, void *hip_stream) {
   if (!caller) return FMHA_E_NULL;
@@ -649,6 +672,53 @@ int fmha_fwd_fp8_launch(const fmha_fwd_fp8_params *caller, void *hip_stream) {
   for (float f : {p->descale_q, p->descale_k, p->descale_v})
     if (!(f > 0.f) || !std::isfinite(f)) return FMHA_E_ARG;
   if (p->mask && (p->mask_bh_div < 1 || p->mask_stride_b < 0)) return FMHA_E_ARG;
+  if (p->kv_len && (p->kv_len_bh_div < 1 || ((uintptr_t)p->kv_len & 3u))) return FMHA_E_ARG;
+  fmha_fwd_params shape; // what the piece planning looks at
+  if (fp8_decode_shape(p, shape)) {
+    // one to four query rows: the streaming decode kernel on e4m3 rows, whole key range or pieces
+    DecodeArgs d;
+    d.q = p->q; d.k = p->k; d.v = p->v;
+    d.o = p->o;
+    d.lse = p->lse;
+    d.o_part = nullptr;
+    d.lse_part = nullptr;
+    d.mask = p->mask;
+    d.mask_sb = p->mask_stride_b;
+    d.mask_div = p->mask ? (int32_t)p->mask_bh_div : 1;
+    d.mask_a = FMHA_LOG2E;
+    d.mask_b = 0.f;
+    d.kv_len = p->kv_len;
+    d.kv_div = p->kv_len ? p->kv_len_bh_div : 1;
+    d.bh = p->bh; d.sq = p->sq; d.sk = p->sk;
+    d.pieces = 1;
+    d.chunk = p->sk;
+    d.scale_l2 = p->scale * p->descale_q * p->descale_k * FMHA_LOG2E;
+    d.out_scale = p->descale_v;
+    bool strided = false;
+    int mrc;
+    if ((mrc = make_row_map(d.mq, 0, nullptr, p->bh, p->sq, p->d, strided)) != FMHA_OK) return mrc;
+    if ((mrc = make_row_map(d.mk, 0, nullptr, p->bh, p->sk, p->d, strided)) != FMHA_OK) return mrc;
+    d.mv = d.mk;
+    d.mo = d.mq;
+    SplitPlan pl;
+    const bool split = p->workspace && ((uintptr_t)p->workspace & 15u) == 0 && plan_split(&shape, pl) &&
+                       p->workspace_bytes >= pl.bytes;
+    if (split) {
+      unsigned char *ws = (unsigned char *)p->workspace;
+      d.pieces = pl.pieces;
+      d.chunk = pl.chunk;
+      d.o_part = (float *)ws;
+      d.lse_part = (float *)(ws + pl.off_lse);
+    }
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int rc = fwd_decode_fp8_dispatch(d, p->d, p->out_dtype == FMHA_DTYPE_BF16, s);
+    if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
+    if (split && merge_launch<true>(p->out_dtype, p->o, p->lse, p->bh, p->sq, p->d, d.o_part, d.lse_part, d.mo,
+                                    pl.pieces, s) != 0)
+      return FMHA_E_LAUNCH;
+    return FMHA_OK;
+  }
+  if (p->kv_len) return FMHA_E_UNSUPPORTED; // the matrix-pipe e4m3 kernel takes no key counts
   Fp8Args a;
   a.q = (const uint8_t *)p->q; a.k = (const uint8_t *)p->k; a.v = (const uint8_t *)p->v;
   a.o = p->o; a.lse = p->lse;

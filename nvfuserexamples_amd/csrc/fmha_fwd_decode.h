@@ -19,6 +19,9 @@
 
 namespace fmha {
 
+// q, k and v may also hold e4m3 bytes (element type uint8_t here; o and the mask then have a 16-bit type of
+// their own): the same kernel with 8-byte row loads, twice as many of them in flight, and the dequantisation
+// factors folded into scale_l2 and out_scale.
 struct DecodeArgs {
   const void *q, *k, *v;
   void *o;          // final output (element type), used when pieces == 1
@@ -33,12 +36,23 @@ struct DecodeArgs {
   int32_t kv_div;
   int32_t bh, sq, sk;
   int32_t pieces, chunk; // pieces of `chunk` keys each (pieces == 1: chunk >= sk)
-  float scale_l2;
+  float scale_l2;   // scale * log2(e) (times the dequantisation factors of q and k)
+  float out_scale;  // 1 (the dequantisation factor of v)
   RowMap mq, mk, mv, mo;
 };
 
 constexpr int kDecodeWaves = 4;
-constexpr int kDecodeLoads = 8; // K (and V) loads a wave keeps in flight per block
+
+// A lane's eight elements of a row: one 16-byte load of 16-bit elements, one 8-byte load of e4m3 bytes; and how
+// many K (and V) loads a wave keeps in flight per block (the same bytes either way).
+template <typename TI> struct DecodeIn {
+  using Load = u32x4;
+  static constexpr int LOADS = 8;
+};
+template <> struct DecodeIn<uint8_t> {
+  using Load = u32x2;
+  static constexpr int LOADS = 16;
+};
 
 template <typename T> FMHA_DEV void unpack8(u32x4 w, float (&x)[8]) {
   if constexpr (__is_same(T, _Float16)) {
@@ -54,6 +68,17 @@ template <typename T> FMHA_DEV void unpack8(u32x4 w, float (&x)[8]) {
     }
   }
 }
+template <typename T> FMHA_DEV void unpack8(u32x2 w, float (&x)[8]) { // e4m3
+  static_assert(__is_same(T, uint8_t), "8-byte loads hold e4m3 bytes");
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
+    x[4 * i] = lo[0];
+    x[4 * i + 1] = lo[1];
+    x[4 * i + 2] = hi[0];
+    x[4 * i + 3] = hi[1];
+  }
+}
 
 // Sum over the LPR (8 or 16) neighbouring lanes that hold one row; every lane gets the total.
 template <int LPR> FMHA_DEV float row_sum(float x) {
@@ -65,11 +90,14 @@ template <int LPR> FMHA_DEV float row_sum(float x) {
   return x;
 }
 
-template <typename T, int D, int NQ, bool MASK>
+// TI: element type of q, k, v (fp16, bf16 or uint8_t = e4m3); TO: of o and the mask (= TI unless TI is e4m3).
+template <typename TI, typename TO, int D, int NQ, bool MASK>
 __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(const DecodeArgs a) {
+  using T = TI;
+  using Load = typename DecodeIn<TI>::Load;
   constexpr int LPR = D / 8;       // lanes per row
   constexpr int NG = 64 / LPR;     // lane groups per wave = rows per load instruction
-  constexpr int U = kDecodeLoads;
+  constexpr int U = DecodeIn<TI>::LOADS;
   constexpr int BLK = U * NG;      // keys per wave and block
   constexpr int NS = kDecodeWaves * NG; // softmax states per workgroup
   constexpr float NEG_INF = -__builtin_inff();
@@ -95,14 +123,14 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
   const T *Kb = (const T *)a.k + a.mk.head(head) + c8 * 8;
   const T *Vb = (const T *)a.v + a.mv.head(head) + c8 * 8;
   const size_t kss = (size_t)a.mk.ss, vss = (size_t)a.mv.ss;
-  const T *mrow = MASK ? (const T *)a.mask + (size_t)(head / a.mask_div) * (size_t)a.mask_sb : nullptr;
+  const TO *mrow = MASK ? (const TO *)a.mask + (size_t)(head / a.mask_div) * (size_t)a.mask_sb : nullptr;
 
   // the lane's 8 columns of every query row, times scale * log2(e)
   float qf[NQ][8];
 #pragma unroll
   for (int r = 0; r < NQ; ++r) {
     const int qr = r < a.sq ? r : a.sq - 1;
-    const u32x4 t = *(const u32x4 *)((const T *)a.q + a.mq.head(head) + (size_t)qr * (size_t)a.mq.ss + c8 * 8);
+    const Load t = *(const Load *)((const T *)a.q + a.mq.head(head) + (size_t)qr * (size_t)a.mq.ss + c8 * 8);
     unpack8<T>(t, qf[r]);
 #pragma unroll
     for (int e = 0; e < 8; ++e) qf[r][e] *= a.scale_l2;
@@ -122,7 +150,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
   // One set of registers per stream: the K loads of the wave's next block are issued as soon as this block's
   // scores are formed, its V loads as soon as this block's P.V is done, so that 8-16 loads per wave (and the other
   // waves of the SIMD) cover the trip to memory.
-  u32x4 kc[U], vc[U];
+  Load kc[U], vc[U];
   float mc[U];
   auto key_of = [&](int b, int j) {
     const int key = k0 + b * BLK + j * NG + g;
@@ -132,13 +160,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
 #pragma unroll
     for (int j = 0; j < U; ++j) {
       const int key = key_of(b, j);
-      kc[j] = *(const u32x4 *)(Kb + (size_t)key * kss);
+      kc[j] = *(const Load *)(Kb + (size_t)key * kss);
       if constexpr (MASK) mc[j] = (float)mrow[key];
     }
   };
   auto issue_v = [&](int b) {
 #pragma unroll
-    for (int j = 0; j < U; ++j) vc[j] = *(const u32x4 *)(Vb + (size_t)key_of(b, j) * vss);
+    for (int j = 0; j < U; ++j) vc[j] = *(const Load *)(Vb + (size_t)key_of(b, j) * vss);
   };
   if (w < nblk) {
     issue_k(w);
@@ -226,7 +254,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
       for (int e = 0; e < 8; ++e) out[e] = fmaf(s_acc[i][r][c8 * 8 + e], f, out[e]);
     }
   }
-  const float inv = tot > 0.f ? 1.f / tot : 0.f; // no visible key: O = 0, LSE = -inf
+  const float inv = tot > 0.f ? a.out_scale / tot : 0.f; // no visible key: O = 0, LSE = -inf
   const float lse = tot > 0.f ? (M + fast_log2(tot)) * FMHA_LN2 : NEG_INF;
   if (a.pieces > 1) {
     float *dst = a.o_part + ((size_t)blockIdx.x * a.sq + r) * D + c8 * 8;
@@ -239,15 +267,17 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
     Pack16 y;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      if constexpr (__is_same(T, _Float16)) y.h[e] = (_Float16)(out[e] * inv);
+      if constexpr (__is_same(TO, _Float16)) y.h[e] = (_Float16)(out[e] * inv);
       else y.b[e] = (__bf16)(out[e] * inv);
     }
-    *(u32x4 *)((T *)a.o + a.mo.head(head) + (size_t)r * (size_t)a.mo.ss + c8 * 8) = y.u;
+    *(u32x4 *)((TO *)a.o + a.mo.head(head) + (size_t)r * (size_t)a.mo.ss + c8 * 8) = y.u;
     if (a.lse && c8 == 0) a.lse[(size_t)head * a.sq + r] = lse;
   }
 }
 
 // Return 0 on success, 1 if the shape is not built, 2 if the launch failed.
 int fwd_decode_dispatch(const DecodeArgs &a, int d, bool bf16, hipStream_t s);
+// The same for e4m3 q, k, v (o and mask fp16 or bf16).
+int fwd_decode_fp8_dispatch(const DecodeArgs &a, int d, bool out_bf16, hipStream_t s);
 
 } // namespace fmha

@@ -35,8 +35,17 @@ CASES = [
     (2, 320, 320, 64, torch.float16, None, True),        # causal
     (2, 200, 333, 128, torch.bfloat16, "pad", False),
     (2, 257, 257, 128, torch.float16, "pad", True),
-    (2, 1, 1000, 64, torch.float16, None, False),        # decode step
+    (2, 1, 1000, 64, torch.float16, None, False),        # one query row (kept on this kernel: FMHA_FWD_DECODE=0)
 ]
+
+
+@pytest.fixture
+def matrix_pipe_only(monkeypatch):
+    """Keeps launches of one to four query rows off the decode kernel, whose probabilities stay fp32."""
+    monkeypatch.setenv("FMHA_FWD_DECODE", "0")
+    yield
+    monkeypatch.delenv("FMHA_FWD_DECODE")
+    capi.lib().fmha_reload_overrides()
 
 
 def _quantise(x, amax=448.0):
@@ -46,7 +55,7 @@ def _quantise(x, amax=448.0):
 
 
 @pytest.mark.parametrize("bh,sq,sk,d,odt,mask,causal", CASES)
-def test_fp8_forward_matches_the_oracle_with_the_same_rounding(bh, sq, sk, d, odt, mask, causal):
+def test_fp8_forward_matches_the_oracle_with_the_same_rounding(bh, sq, sk, d, odt, mask, causal, matrix_pipe_only):
     g = torch.Generator().manual_seed(bh + sk)
     std = 1.0 if d == 64 else 0.5
     q, k, v = (torch.randn(bh, s, d, generator=g) * std for s in (sq, sk, sk))
@@ -155,3 +164,63 @@ def test_fp8_operator_equals_the_c_abi_call():
     o, lse = ops.fmha_fwd_fp8(q8, k8, v8, 0.5, 2.0, 1.5, m, 0.0, False)
     o2, lse2 = capi.fwd_fp8(q8, k8, v8, 0.5, 2.0, 1.5, mask=m, want_lse=True)
     assert torch.equal(o, o2) and torch.equal(lse, lse2)
+
+
+DECODE_CASES = [
+    # bh, sq, sk, d, out dtype, mask, kv_len, forced pieces (None: the library's choice, 0: never)
+    (4, 1, 1000, 64, torch.float16, None, False, 0),
+    (2, 1, 4096, 128, torch.float16, None, False, None),     # cut by the library itself
+    (4, 2, 3000, 128, torch.bfloat16, "pad", True, 3),
+    (3, 4, 700, 64, torch.float16, None, True, 2),
+    (2, 3, 333, 128, torch.float16, "pad", False, 0),
+]
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,odt,mask,kvl,force", DECODE_CASES)
+def test_fp8_decode_steps_keep_fp32_probabilities(bh, sq, sk, d, odt, mask, kvl, force, monkeypatch):
+    """One to four query rows without a causal mask run on the streaming decode kernel: e4m3 rows are unpacked to
+    fp32 and nothing is rounded until O, so the result is the oracle's on the same e4m3 inputs WITHOUT any rounding
+    of the probabilities, to the rounding of O (plus 1e-4 of max|v| for the fp32 sums); valid key counts and the key
+    range in pieces as in the 16-bit forward."""
+    g = torch.Generator().manual_seed(bh * 100 + sk)
+    std = 1.0 if d == 64 else 0.5
+    q, k, v = (torch.randn(bh, s, d, generator=g) * std for s in (sq, sk, sk))
+    q8, dq = _quantise(q)
+    k8, dk = _quantise(k)
+    v8, dv = _quantise(v)
+    m = pad_mask(bh // 2 if bh % 2 == 0 else bh, sk, sk // 2, sk).to(odt) if mask == "pad" else None
+    lens = torch.randint(1, sk + 1, (bh,), generator=g, dtype=torch.int32) if kvl else None
+    if force is not None:
+        monkeypatch.setenv("FMHA_FWD_SPLIT", str(force))
+    try:
+        o, lse = capi.fwd_fp8(q8.cuda(), k8.cuda(), v8.cuda(), dq, dk, dv, mask=None if m is None else m.cuda(),
+                              out_dtype=odt, want_lse=True, kv_len=None if lens is None else lens.cuda())
+        o0, lse0 = capi.fwd_fp8(q8.cuda(), k8.cuda(), v8.cuda(), dq, dk, dv, mask=None if m is None else m.cuda(),
+                                out_dtype=odt, want_lse=True, kv_len=None if lens is None else lens.cuda(),
+                                workspace=False)
+        torch.cuda.synchronize()
+    finally:
+        monkeypatch.delenv("FMHA_FWD_SPLIT", raising=False)
+        capi.lib().fmha_reload_overrides()
+    full = np.zeros((bh, sq, sk), np.float32)
+    if m is not None:
+        full += np.repeat(f32(m).reshape(-1, 1, sk), bh // m.shape[0], 0)
+    if lens is not None:
+        for i, n in enumerate(lens.tolist()):
+            full[i, :, n:] = -np.inf
+    qf, kf, vf = (f32(t.float()) for t in (q8, k8, v8))
+    exact = oracle.attention(qf, kf, vf * np.float32(dv), mask=full, scale=d ** -0.5 * dq * dk, want=("o", "lse"))
+    top = np.abs(exact["o"]).max()
+    vmax = float(np.abs(vf).max()) * dv
+    out_round = 2.0 ** -11 if odt == torch.float16 else 2.0 ** -8
+    for got, gl in ((o, lse), (o0, lse0)):
+        assert np.abs(f32(got.cpu()) - exact["o"]).max() <= 1e-4 * vmax + out_round * top
+        assert np.abs(gl.cpu().numpy() - exact["lse"]).max() <= 1e-3
+
+
+def test_fp8_key_counts_need_the_decode_kernel():
+    """Launches the decode kernel does not serve (more than four rows, causal) refuse valid key counts."""
+    q8, k8, v8 = (torch.randn(2, s, 64).to(torch.float8_e4m3fn).cuda() for s in (8, 256, 256))
+    lens = torch.tensor([100, 200], dtype=torch.int32).cuda()
+    with pytest.raises(capi.FmhaError, match="-6"):
+        capi.fwd_fp8(q8, k8, v8, kv_len=lens)
