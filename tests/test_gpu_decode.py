@@ -233,3 +233,72 @@ def test_ragged_last_piece_reads_no_row_past_the_end(d, pieces):
     ref = oracle.attention(f32(q), f32(k), f32(v), want=("o", "lse"))
     assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
     assert np.abs(f32(o.cpu()) - ref["o"]).max() <= O_TOL["fp16"]
+
+
+def test_randomized_decode_steps_against_the_oracle(monkeypatch):
+    """150 seeded random decode problems: one to four query rows, head dim 64 / 128, fp16 / bf16 / e4m3 inputs,
+    ragged key ranges, per-key masks (batch- or head-wise, with holes and -inf), valid key counts, folded and
+    [B, S, H, D] layouts, whole key range or 2-7 pieces.  O within 2e-3 (fp16, e4m3 inputs) / 2e-2 (bf16) of the
+    oracle, LSE within 2e-3, -inf rows in the same places."""
+    import random
+    rng = random.Random(424242)
+    L = capi.lib()
+    try:
+        for it in range(150):
+            kind = rng.choice(["fp16", "fp16", "bf16", "e4m3"])
+            d = rng.choice([64, 128])
+            b, h = rng.choice([1, 2, 3]), rng.choice([1, 2, 4])
+            bh = b * h
+            sq = rng.choice([1, 1, 1, 2, 3, 4])
+            sk = rng.choice([1, 7, 33, 64, 100, 255, 256, 257, 500, 1000, 1777, 3000])
+            maskk = rng.choice(["none", "none", "pad", "head"])
+            use_len = rng.random() < 0.4
+            strided = kind != "e4m3" and rng.random() < 0.3
+            n = rng.choice([0, 0, 2, 3, 7])
+            g = torch.Generator().manual_seed(1000 + it)
+            std = 1.0 if d == 64 else 0.5
+            tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+            q, k, v = (torch.randn(bh, s, d, generator=g) * std for s in (sq, sk, sk))
+            m = None
+            if maskk == "pad":
+                m = torch.zeros(b, 1, 1, sk)
+                for i in range(b):
+                    m[i, ..., rng.randint(1, sk):] = -10000.0
+            elif maskk == "head":
+                m = torch.randn(bh, 1, sk, generator=g)
+                m[torch.rand(bh, 1, sk, generator=g) < 0.3] = float("-inf")
+            lens = torch.tensor([rng.randint(0, sk) for _ in range(b)], dtype=torch.int32) if use_len else None
+            monkeypatch.setenv("FMHA_FWD_SPLIT", str(n))
+            mc = None if m is None else m.to(tdt).cuda()
+            lc = None if lens is None else lens.cuda()
+            if kind == "e4m3":
+                q8, k8, v8 = (t.to(torch.float8_e4m3fn) for t in (q, k, v))
+                o, lse = capi.fwd_fp8(q8.cuda(), k8.cuda(), v8.cuda(), 0.5, 2.0, 0.25, mask=mc, out_dtype=tdt,
+                                      want_lse=True, kv_len=lc)
+                qf, kf, vf, scale = f32(q8.float()), f32(k8.float()), f32(v8.float()) * np.float32(0.25), d ** -0.5
+            else:
+                qc, kc, vc = (t.to(tdt).cuda() for t in (q, k, v))
+                if strided:
+                    lay = lambda x: x.view(b, h, x.shape[1], d).permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+                    qc, kc, vc = lay(qc), lay(kc), lay(vc)
+                o, lse, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, kv_len=lc)
+                qf, kf, vf, scale = f32(q.to(tdt)), f32(k.to(tdt)), f32(v.to(tdt)), d ** -0.5
+            torch.cuda.synchronize()
+            full = np.zeros((bh, sq, sk), np.float32)
+            if m is not None:
+                mm = f32(m.to(tdt)).reshape(-1, 1, sk)
+                full += np.repeat(mm, bh // mm.shape[0], 0)
+            if lens is not None:
+                for i, cnt in enumerate(lens.tolist()):
+                    full[i * h:(i + 1) * h, :, cnt:] = -np.inf
+            ref = oracle.attention(qf, kf, vf, mask=full, scale=scale, want=("o", "lse"))
+            what = f"case #{it}: {kind} d{d} b{b} h{h} sq{sq} sk{sk} mask {maskk} len {use_len} strided {strided} pieces {n}"
+            tol = (2e-2 if kind == "bf16" else 2e-3) * max(1.0, float(np.abs(ref["o"]).max()) / 2.0)
+            assert np.abs(f32(o.reshape(bh, sq, d).cpu()) - ref["o"]).max() <= tol, what
+            fin = np.isfinite(ref["lse"])
+            gl = lse.reshape(bh, sq).cpu().numpy()
+            assert np.array_equal(np.isfinite(gl), fin), what
+            assert not fin.any() or np.abs(gl[fin] - ref["lse"][fin]).max() <= 2e-3 + 2.0 ** -8 * (kind == "bf16"), what
+    finally:
+        monkeypatch.delenv("FMHA_FWD_SPLIT", raising=False)
+        L.fmha_reload_overrides()
