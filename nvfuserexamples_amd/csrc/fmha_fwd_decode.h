@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
   using Load = typename DecodeIn<TI>::Load;
   constexpr int LPR = D / 8;       // lanes per row
   constexpr int NG = 64 / LPR;     // lane groups per wave = rows per load instruction
-  constexpr int U = DecodeIn<TI>::LOADS;
+  constexpr int U = NQ >= 4 ? 8 : DecodeIn<TI>::LOADS; // (four query rows: fewer loads in flight, for the registers)
   constexpr int BLK = U * NG;      // keys per wave and block
   constexpr int NS = kDecodeWaves * NG; // softmax states per workgroup
   constexpr float NEG_INF = -__builtin_inff();
