@@ -609,6 +609,15 @@ def torch_sdpa_context(torch, steps, warmup):
         out["train_step_dropout_us"] = round(ms_t * 1e3, 1)
         out["train_step_tflops"] = round(14.0 * B * H * S * S * D / (ms_t * 1e-3) / 1e12, 1)
         out["torch"] = torch.__version__
+        # a decode step (the first shape of `decode_steps`: 2 x 16 heads, one query row, 32 768 keys, D 128)
+        del qg, kg, vg, do
+        qd = torch.randn((2, 16, 1, 128), dtype=torch.float16, device="cuda", generator=g)
+        kvs = [tuple(torch.randn((2, 16, 32768, 128), dtype=torch.float16, device="cuda", generator=g) for _ in range(2))
+               for _ in range(3)]
+        with torch.no_grad():
+            ms_d, _ = time_steps(torch, lambda i: F.scaled_dot_product_attention(qd, *kvs[i % 3]), max(10, steps // 2),
+                                 max(2, warmup // 2), blocks=9)
+        out["decode_BH32_Sk32768_D128_us"] = round(ms_d * 1e3, 1)
     except Exception as e:  # a context figure must never break the benchmark
         out["unavailable"] = repr(e)[:200]
     return out
