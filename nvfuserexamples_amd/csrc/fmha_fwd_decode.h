@@ -4,8 +4,9 @@
 // so this kernel is built around the loads, not around the matrix pipe: a wave reads whole rows with 16-byte
 // loads (D / 8 neighbouring lanes cover one row, so a load instruction fetches 64 / (D / 8) complete rows),
 // keeps eight K loads and eight V loads in flight (up to 16 KB per wave, 128 KB per compute unit),
-// and does the arithmetic on the vector pipe in fp32: dot products by multiply-add on the unpacked elements,
-// summed over the lanes of a row by four DPP additions, an online softmax per lane group, P.V by multiply-add.
+// and does the arithmetic on the vector pipe in fp32: dot products on v_dot2c_f32_f16 / _bf16 (exact products of
+// the packed elements, fp32 sums; multiply-adds on unpacked elements for e4m3 rows), summed over the lanes of a
+// row by three or four DPP additions, an online softmax per lane group, P.V by multiply-add.
 // Nothing is staged in LDS and nothing is rounded on the way (scores, probabilities and sums are fp32).
 //
 // Work split: a workgroup of four waves owns one (head, piece of the key range); its waves take the piece's
@@ -80,6 +81,17 @@ template <typename T> FMHA_DEV void unpack8(u32x2 w, float (&x)[8]) { // e4m3
   }
 }
 
+// c + a.x * b.x + a.y * b.y on a pair of 16-bit elements (fp32 products and sum).
+template <typename T> FMHA_DEV float dot2(uint32_t a, uint32_t b, float c) {
+  if constexpr (__is_same(T, _Float16)) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), c, false);
+  } else {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, a), __builtin_bit_cast(b2, b), c, false);
+  }
+}
+
 // Sum over the LPR (8 or 16) neighbouring lanes that hold one row; every lane gets the total.
 template <int LPR> FMHA_DEV float row_sum(float x) {
   x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
@@ -103,8 +115,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
   constexpr float NEG_INF = -__builtin_inff();
   static_assert(D == 64 || D == 128, "rows of 8 or 16 lanes");
 
-  __shared__ float s_m[NS][NQ], s_l[NS][NQ];
-  __shared__ float s_acc[NS][NQ][D];
+  constexpr int RG = NQ < 4 ? NQ : 4; // query rows that meet in LDS at a time
+  __shared__ float s_m[NS][RG], s_l[NS][RG];
+  __shared__ float s_acc[NS][RG][D];
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
   const int g = l / LPR, c8 = l % LPR; // the lane's group and its 8 columns
@@ -125,15 +138,22 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
   const size_t kss = (size_t)a.mk.ss, vss = (size_t)a.mv.ss;
   const TO *mrow = MASK ? (const TO *)a.mask + (size_t)(head / a.mask_div) * (size_t)a.mask_sb : nullptr;
 
-  // the lane's 8 columns of every query row, times scale * log2(e)
-  float qf[NQ][8];
+  // the lane's 8 columns of every query row: 16-bit rows stay packed (the dot products run on v_dot2c_f32_*, exact
+  // products summed in fp32, and the score is scaled afterwards); e4m3 rows are unpacked and scaled here
+  constexpr bool DOT2 = sizeof(TI) == 2;
+  Load qp[DOT2 ? NQ : 1];
+  float qf[DOT2 ? 1 : NQ][8];
 #pragma unroll
   for (int r = 0; r < NQ; ++r) {
     const int qr = r < a.sq ? r : a.sq - 1;
     const Load t = *(const Load *)((const T *)a.q + a.mq.head(head) + (size_t)qr * (size_t)a.mq.ss + c8 * 8);
-    unpack8<T>(t, qf[r]);
+    if constexpr (DOT2) {
+      qp[r] = t;
+    } else {
+      unpack8<T>(t, qf[r]);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) qf[r][e] *= a.scale_l2;
+      for (int e = 0; e < 8; ++e) qf[r][e] *= a.scale_l2;
+    }
   }
 
   float m_run[NQ], l_run[NQ], acc[NQ][8];
@@ -179,15 +199,21 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
     float s[NQ][U];
 #pragma unroll
     for (int j = 0; j < U; ++j) {
-      float x[8];
-      unpack8<T>(kc[j], x);
       const bool live = kb + j * NG + g < k1;
+      float x[8];
+      if constexpr (!DOT2) unpack8<T>(kc[j], x);
 #pragma unroll
       for (int r = 0; r < NQ; ++r) {
         float d = 0.f;
+        if constexpr (DOT2) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) d = fmaf(qf[r][e], x[e], d);
-        d = row_sum<LPR>(d);
+          for (int i = 0; i < 4; ++i) d = dot2<T>(qp[r][i], kc[j][i], d);
+          d = row_sum<LPR>(d) * a.scale_l2;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) d = fmaf(qf[r][e], x[e], d);
+          d = row_sum<LPR>(d);
+        }
         if constexpr (MASK) d += fmaf(mc[j], a.mask_a, a.mask_b);
         s[r][j] = live ? d : NEG_INF;
       }
@@ -226,52 +252,57 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void fmha_fwd_decode_kernel(cons
     if (more) issue_v(b + kDecodeWaves);
   }
 
-  // ---- the workgroup's NS partial softmaxes meet in LDS
+  // ---- the workgroup's NS partial softmaxes meet in LDS (up to four query rows at a time: RG)
   const int st = w * NG + g;
 #pragma unroll
-  for (int r = 0; r < NQ; ++r) {
-    if (c8 == 0) {
-      s_m[st][r] = m_run[r];
-      s_l[st][r] = l_run[r];
+  for (int r0 = 0; r0 < NQ; r0 += RG) {
+    if (r0 > 0) __syncthreads(); // the previous rows have been read
+#pragma unroll
+    for (int rr = 0; rr < RG; ++rr) {
+      if (c8 == 0) {
+        s_m[st][rr] = m_run[r0 + rr];
+        s_l[st][rr] = l_run[r0 + rr];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s_acc[st][rr][c8 * 8 + e] = acc[r0 + rr][e];
     }
+    __syncthreads();
+    // thread t: query row r0 + t / LPR, columns 8 * (t % LPR) .. +7
+    const int rr = tid / LPR, r = r0 + rr;
+    if (rr < RG && r < a.sq) {
+      float M = NEG_INF;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s_acc[st][r][c8 * 8 + e] = acc[r][e];
-  }
-  __syncthreads();
-  // thread t: query row t / LPR, columns 8 * (t % LPR) .. +7
-  const int r = tid / LPR;
-  if (r >= NQ || r >= a.sq) return;
-  float M = NEG_INF;
+      for (int i = 0; i < NS; ++i) M = fmaxf(M, s_m[i][rr]);
+      float tot = 0.f, out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (M != NEG_INF) {
 #pragma unroll
-  for (int i = 0; i < NS; ++i) M = fmaxf(M, s_m[i][r]);
-  float tot = 0.f, out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (M != NEG_INF) {
+        for (int i = 0; i < NS; ++i) {
+          const float f = fast_exp2(s_m[i][rr] - M); // (an empty state: 2^-inf = 0)
+          tot = fmaf(s_l[i][rr], f, tot);
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const float f = fast_exp2(s_m[i][r] - M); // (an empty state: 2^-inf = 0)
-      tot = fmaf(s_l[i][r], f, tot);
+          for (int e = 0; e < 8; ++e) out[e] = fmaf(s_acc[i][rr][c8 * 8 + e], f, out[e]);
+        }
+      }
+      const float inv = tot > 0.f ? a.out_scale / tot : 0.f; // no visible key: O = 0, LSE = -inf
+      const float lse = tot > 0.f ? (M + fast_log2(tot)) * FMHA_LN2 : NEG_INF;
+      if (a.pieces > 1) {
+        float *dst = a.o_part + ((size_t)blockIdx.x * a.sq + r) * D + c8 * 8;
+        f32x4 lo = {out[0] * inv, out[1] * inv, out[2] * inv, out[3] * inv};
+        f32x4 hi = {out[4] * inv, out[5] * inv, out[6] * inv, out[7] * inv};
+        *(f32x4 *)dst = lo;
+        *(f32x4 *)(dst + 4) = hi;
+        if (c8 == 0) a.lse_part[(size_t)blockIdx.x * a.sq + r] = lse;
+      } else {
+        Pack16 y;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) out[e] = fmaf(s_acc[i][r][c8 * 8 + e], f, out[e]);
+        for (int e = 0; e < 8; ++e) {
+          if constexpr (__is_same(TO, _Float16)) y.h[e] = (_Float16)(out[e] * inv);
+          else y.b[e] = (__bf16)(out[e] * inv);
+        }
+        *(u32x4 *)((TO *)a.o + a.mo.head(head) + (size_t)r * (size_t)a.mo.ss + c8 * 8) = y.u;
+        if (a.lse && c8 == 0) a.lse[(size_t)head * a.sq + r] = lse;
+      }
     }
-  }
-  const float inv = tot > 0.f ? a.out_scale / tot : 0.f; // no visible key: O = 0, LSE = -inf
-  const float lse = tot > 0.f ? (M + fast_log2(tot)) * FMHA_LN2 : NEG_INF;
-  if (a.pieces > 1) {
-    float *dst = a.o_part + ((size_t)blockIdx.x * a.sq + r) * D + c8 * 8;
-    f32x4 lo = {out[0] * inv, out[1] * inv, out[2] * inv, out[3] * inv};
-    f32x4 hi = {out[4] * inv, out[5] * inv, out[6] * inv, out[7] * inv};
-    *(f32x4 *)dst = lo;
-    *(f32x4 *)(dst + 4) = hi;
-    if (c8 == 0) a.lse_part[(size_t)blockIdx.x * a.sq + r] = lse;
-  } else {
-    Pack16 y;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      if constexpr (__is_same(TO, _Float16)) y.h[e] = (_Float16)(out[e] * inv);
-      else y.b[e] = (__bf16)(out[e] * inv);
-    }
-    *(u32x4 *)((TO *)a.o + a.mo.head(head) + (size_t)r * (size_t)a.mo.ss + c8 * 8) = y.u;
-    if (a.lse && c8 == 0) a.lse[(size_t)head * a.sq + r] = lse;
   }
 }
 

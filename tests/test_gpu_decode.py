@@ -69,6 +69,8 @@ CASES = [
     (5, 2, 777, 128, "bf16", 2, "perhead", True),      # two query rows
     (4, 4, 1234, 64, "fp16", 3, "pad", True),          # four
     (3, 3, 333, 128, "fp16", 2, None, False),          # three (run as four)
+    (3, 8, 900, 128, "bf16", 3, "perhead", True),      # eight rows: the matrix-pipe kernels on the pieces
+    (2, 6, 1100, 64, "fp16", 2, "pad", False),
 ]
 
 
@@ -236,7 +238,7 @@ def test_ragged_last_piece_reads_no_row_past_the_end(d, pieces):
 
 
 def test_randomized_decode_steps_against_the_oracle(monkeypatch):
-    """150 seeded random decode problems: one to four query rows, head dim 64 / 128, fp16 / bf16 / e4m3 inputs,
+    """150 seeded random problems of one to eight query rows (up to four: the decode kernel; e4m3 rows: up to four), head dim 64 / 128, fp16 / bf16 / e4m3 inputs,
     ragged key ranges, per-key masks (batch- or head-wise, with holes and -inf), valid key counts, folded and
     [B, S, H, D] layouts, whole key range or 2-7 pieces.  O within 2e-3 (fp16, e4m3 inputs) / 2e-2 (bf16) of the
     oracle, LSE within 2e-3, -inf rows in the same places."""
@@ -249,7 +251,7 @@ def test_randomized_decode_steps_against_the_oracle(monkeypatch):
             d = rng.choice([64, 128])
             b, h = rng.choice([1, 2, 3]), rng.choice([1, 2, 4])
             bh = b * h
-            sq = rng.choice([1, 1, 1, 2, 3, 4])
+            sq = rng.choice([1, 1, 1, 2, 3, 4]) if kind == "e4m3" else rng.choice([1, 1, 1, 2, 3, 4, 5, 8])
             sk = rng.choice([1, 7, 33, 64, 100, 255, 256, 257, 500, 1000, 1777, 3000])
             maskk = rng.choice(["none", "none", "pad", "head"])
             use_len = rng.random() < 0.4
