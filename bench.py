@@ -214,15 +214,17 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
 
     # the same two operators at the headline sequence length (S 512): 403 / 671 MB per call, two sets rotated
     s5 = 512
-    keep5, infer5, train5 = [], [], []
+    keep5, infer5, train5, save5 = [], [], [], []
     for _ in range(2):
         q, k, v = (torch.randn(bh, s5, d, generator=g).to(torch.float16).cuda() for _ in range(3))
         o = torch.empty_like(q)
         amask = (torch.rand(bh, s5, s5, generator=g) > 0.1).to(torch.float16).cuda()
         pad = (torch.rand(bh, s5, s5, generator=g) > 0.9).to(torch.float16).mul_(-1000.0).cuda()
         dm = (torch.rand(bh, s5, s5, generator=g) > 0.5).to(torch.float16).cuda()
-        keep5.append((q, k, v, o, amask, pad, dm))
-        for kind in ("infer", "train"):
+        sm, dr = (torch.empty(bh, s5, s5, dtype=torch.float16, device="cuda") for _ in range(2))
+        lse5 = torch.empty(bh, s5, dtype=torch.float32, device="cuda")
+        keep5.append((q, k, v, o, amask, pad, dm, sm, dr, lse5))
+        for kind in ("infer", "train", "save"):
             P = capi.FwdParams()
             P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
             P.bh, P.sq, P.sk, P.d = bh, s5, s5, d
@@ -234,11 +236,15 @@ def short_sequence_legs(torch, capi, L, stream, steps, warmup):
             else:
                 P.mask, P.mask_kind = pad.data_ptr(), capi.MASK_ADDITIVE
                 P.drop_kind, P.drop_mask, P.drop_scale = capi.DROP_TENSOR, dm.data_ptr(), 2.0
-                train5.append(P)
+                if kind == "save":  # (with an LSE buffer: the forward, then one streaming launch for both saved tensors)
+                    P.save_softmax, P.save_dropout, P.lse = sm.data_ptr(), dr.data_ptr(), lse5.data_ptr()
+                (save5 if kind == "save" else train5).append(P)
     run("fmha_nvfuser_BH512_S512_D64_full_mask", infer5, 4 * bh * s5 * d * 2 + bh * s5 * s5 * 2, "2 sets rotated")
     run("fmha_train_nvfuser_BH512_S512_D64_full_masks", train5, 4 * bh * s5 * d * 2 + 2 * bh * s5 * s5 * 2,
         "2 sets rotated")
-    del keep5, infer5, train5
+    run("fmha_train_saveim_nvfuser_BH512_S512_D64_full_masks", save5, 4 * bh * s5 * d * 2 + 4 * bh * s5 * s5 * 2,
+        "2 sets rotated")
+    del keep5, infer5, train5, save5
 
     # train step at the same short shape (the reference has no backward): [B,1,1,S] padding mask, Philox
     # dropout; forward with LSE, then the one-launch short-sequence backward
