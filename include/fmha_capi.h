@@ -312,10 +312,31 @@ float fmha_drop_scale(float p_drop);
 const char *fmha_strerror(int code);
 
 /* The FMHA_* environment variables -- tuning and test overrides of the variant selection: FMHA_MASK_TRIM,
- * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_BWD_SHORT, FMHA_BWD_PAIR,
+ * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_FWD_HEAD, FMHA_BWD_SHORT, FMHA_BWD_PAIR,
  * FMHA_BWD_FUSED -- are read once per process, on the first launch.  This reads them again; not to be
  * called while another thread is launching.  (No counterpart in the reference.) */
 void fmha_reload_overrides(void);
+
+/*
+ * Pipe-ceiling microbenchmarks of the compute units (no counterpart in the reference; diagnostic only).
+ * mode: 0 exponentials only; 1 matrix instructions (32x32x16 fp16) only, four independent accumulators;
+ * 2 both in one wave's instruction stream, nexp (2, 4 or 6) exponentials behind every matrix instruction;
+ * 3 matrix instructions on one accumulator (a dependent chain); 4 the two waves of a SIMD split the work,
+ * one matrix only, one exponentials only (waves_per_simd must be 2); 5 matrix instructions whose A operand
+ * is read from LDS every time; 6 those LDS reads alone; 7 as 2, but the exponentials read registers that the
+ * matrix instructions of the previous trip wrote; 8 as 2, but the B operand of every matrix instruction is packed
+ * from exponentials of the previous trip.  random_data: 0 all-zero operands, 1 pseudo-random
+ * ones in [-1, 1) -- the board's power management sets the core clock by what the data toggles.
+ * Runs `launches` launches (the second half timed with events) of `iters` loop trips -- 4 matrix
+ * instructions and / or 4 * nexp exponentials per trip and wave -- with waves_per_simd (1 or 2) waves on
+ * every SIMD of the current device and writes
+ *   result[0] microseconds per launch, result[1] mean core clock in MHz as the waves saw it,
+ *   result[2] matrix TFLOP/s (0 without matrix work), result[3] exponentials per nanosecond over the chip.
+ * Unlike the launch functions it allocates and frees buffers of its own and synchronises the device.
+ * Returns 0, or -1 on a bad argument or a HIP error.
+ */
+int fmha_pipe_probe(int mode, int nexp, int random_data, int waves_per_simd, int iters, int launches,
+                    double *result);
 
 /* Library version, "major.minor". */
 const char *fmha_version(void);

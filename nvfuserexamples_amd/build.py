@@ -38,7 +38,7 @@ HIP_FLAGS = [
 def _tus():
     """(source, object name, extra defines) for every translation unit of the library."""
     tus = [("fmha_capi.hip", "fmha_capi.o", []), ("fmha_fwd_fp8.hip", "fmha_fwd_fp8.o", []),
-           ("fmha_fwd_decode.hip", "fmha_fwd_decode.o", [])]
+           ("fmha_fwd_decode.hip", "fmha_fwd_decode.o", []), ("fmha_probe.hip", "fmha_probe.o", [])]
     for bf in (0, 1):
         for d in (64, 128, 256):
             for strided in (0, 1):  # folded contiguous tensors / row layouts given at run time

@@ -19,9 +19,9 @@ DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
            "fmha_drop_threshold", "fmha_strerror", "fmha_version", "fmha_reload_overrides",
            "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale", "fmha_fwd_fp8_launch",
-           "fmha_fwd_workspace_bytes", "fmha_fwd_fp8_workspace_bytes")
+           "fmha_fwd_workspace_bytes", "fmha_fwd_fp8_workspace_bytes", "fmha_pipe_probe")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
-_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT", "FMHA_FWD_DECODE",
+_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT", "FMHA_FWD_DECODE", "FMHA_FWD_HEAD",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
 _env_seen = None
 
@@ -143,6 +143,8 @@ def lib():
         L.fmha_strerror.argtypes = [C.c_int]
         L.fmha_strerror.restype = C.c_char_p
         L.fmha_version.restype = C.c_char_p
+        L.fmha_pipe_probe.argtypes = [C.c_int] * 6 + [C.POINTER(C.c_double)]
+        L.fmha_pipe_probe.restype = C.c_int
         L.fmha_reload_overrides.argtypes = []
         L.fmha_reload_overrides.restype = None
         _lib = L

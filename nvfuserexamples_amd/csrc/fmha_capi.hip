@@ -57,7 +57,7 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // FMHA_FWD_DECODE=0 keeps forwards of one to four query rows on the matrix-pipe kernels.
 // The environment is read once per process (on the first launch); fmha_reload_overrides() reads it again.
 struct Overrides {
-  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, fwd_decode, bwd_pair, bwd_short, bwd_fused;
+  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, fwd_decode, fwd_head, bwd_pair, bwd_short, bwd_fused;
 };
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
@@ -72,6 +72,7 @@ Overrides read_overrides() {
   o.fwd_qb = env_int("FMHA_FWD_QB", 0);
   o.fwd_split = env_int("FMHA_FWD_SPLIT", -1);
   o.fwd_decode = env_int("FMHA_FWD_DECODE", 1);
+  o.fwd_head = env_int("FMHA_FWD_HEAD", -1);
   o.bwd_pair = env_int("FMHA_BWD_PAIR", -1);
   o.bwd_short = env_int("FMHA_BWD_SHORT", 1);
   o.bwd_fused = env_int("FMHA_BWD_FUSED", 0);
@@ -426,7 +427,7 @@ static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const Sp
   v.mask = a.mask ? kMaskPerKey : kMaskNone;
   v.causal = false;
   v.drop = 0;
-  v.saving = v.save_split = v.stream = v.short_keys = false;
+  v.saving = v.save_split = v.stream = v.short_keys = v.head = false;
   const int rc = fwd_dispatch_strided(b, v, p->dtype, D, s);
   if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
   {
@@ -589,6 +590,19 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   const int force = overrides().fwd_qb; // tuning override: 1 or 2
   if (force == 1 || (force == 2 && p->d == 64 && !v.causal && v.drop == 0 && v.mask != kMaskFull)) v.qb = force;
   if (strided) v.qb = 1; // the two-block variant is built for the folded layout only
+  // Key ranges of 257 to 512 keys at head dim 64: a whole head's K and V fit in LDS, and one workgroup of
+  // eight waves per (head, 512 queries) runs without copies or barriers in its loop.  Taken when the
+  // 512-query items fill the compute units evenly (FMHA_FWD_HEAD=0 never, =1 wherever the kernel applies).
+  v.head = false;
+  if (!strided && p->d == 64 && p->sk <= 512 && !v.causal && v.drop != 2 && v.mask != kMaskFull && !v.saving &&
+      overrides().fwd_head != 0) {
+    const int cus = cu_count();
+    const int chunks = (p->sq + 511) / 512;
+    const long long items = (long long)p->bh * chunks;
+    const bool full = chunks * 512 - p->sq <= 128; // at most two of the eight waves of a head's last item idle
+    const bool even = cus > 0 && (items % cus == 0 || items >= 4LL * cus);
+    v.head = overrides().fwd_head == 1 || (p->sk > 256 && full && even);
+  }
 
   int rc;
   if (strided) rc = fwd_dispatch_strided(a, v, p->dtype, D, s);

@@ -10,6 +10,7 @@
 #include "fmha_fwd_short.h"
 #include "fmha_fwd_save.h"
 #include "fmha_fwd_stream.h"
+#include "fmha_fwd_head.h"
 #else
 #define FMHA_TU_SHORT 0
 #endif
@@ -129,6 +130,35 @@ template <bool DROPT> int launch_stream(FwdArgs &a, hipStream_t s) {
 }
 #endif
 
+#if FMHA_TU_SHORT
+// a whole head's K and V resident in LDS: one persistent workgroup per compute unit
+#ifndef FMHA_HEAD_QB
+#define FMHA_HEAD_QB 2
+#endif
+template <int MASK, int DROP> int launch_head(FwdArgs &a, hipStream_t s) {
+  using HC = HeadCfgT<FMHA_HEAD_QB>;
+  auto kern = fmha_fwd_head_kernel<FMHA_TU_T, FMHA_HEAD_QB, MASK, DROP>;
+  static const int resident = [&]() -> int {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            HC::LDS_BYTES) != hipSuccess)
+      return -1;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      return -1;
+    return cus;
+  }();
+  if (resident < 0) return 2;
+  if (a.sk > HC::MAXK) return 1;
+  a.nqt = (a.sq + HC::QT - 1) / HC::QT;
+  long long nblk = (long long)a.bh * a.nqt;
+  if (nblk > 0x7fffffffLL) return 2;
+  if (nblk > resident) nblk = resident;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(HC::NT), HC::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+#endif
+
 template <int QB, int MASK, bool CAUSAL> int by_drop(FwdArgs &a, int drop, hipStream_t s) {
   if (drop == 0) return launch<QB, MASK, CAUSAL, 0>(a, s);
   if (drop == 1) return launch<QB, MASK, CAUSAL, 1>(a, s);
@@ -170,7 +200,7 @@ template <int MASK, bool CAUSAL> int plain_by_drop(FwdArgs &a, int drop, hipStre
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
-  if (v.qb == 2 || v.short_keys || v.save_split || v.stream || (kStrided && v.drop == 2)) return 1;
+  if (v.qb == 2 || v.short_keys || v.save_split || v.stream || v.head || (kStrided && v.drop == 2)) return 1;
   if (v.mask == kMaskPerKey)
     return v.causal ? plain_by_drop<kMaskPerKey, true>(a, v.drop, s) : plain_by_drop<kMaskPerKey, false>(a, v.drop, s);
   if (v.mask == kMaskFull)
@@ -192,8 +222,13 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
     return rc ? rc : launch_save(a, s);
   }
   if (v.stream) return v.drop == 2 ? launch_stream<true>(a, s) : launch_stream<false>(a, s);
+  if (v.head) {
+    if (v.causal || v.drop == 2 || v.mask == kMaskFull) return 1;
+    if (v.mask == kMaskPerKey) return v.drop ? launch_head<kMaskPerKey, 1>(a, s) : launch_head<kMaskPerKey, 0>(a, s);
+    return v.drop ? launch_head<kMaskNone, 1>(a, s) : launch_head<kMaskNone, 0>(a, s);
+  }
 #else
-  if (v.short_keys || v.save_split || v.stream) return 1;
+  if (v.short_keys || v.save_split || v.stream || v.head) return 1;
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;

@@ -149,6 +149,24 @@ template <> FMHA_DEV float dot2_ones<__bf16>(bf16x8 v, int pair, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(x, one, acc, false);
 }
 
+// lo += v[2 pair], hi += v[2 pair + 1] in fp32: the row sums of the ROUNDED probabilities, so that the denominator
+// matches what the second product sums (a row with one visible key reproduces that key's value exactly).  Not the
+// packed dot product that would do both in one instruction: next to matrix instructions v_dot2c costs about twenty
+// cycles apiece on this chip (measured: one matrix instruction + 2 / 4 / 6 v_dot2c_f32_f16 55 / 63 / 71 cycles;
+// + 2 / 4 / 6 v_fma_mix_f32 35 / 36 / 40; + 2 / 4 / 6 v_add_f32 34 / 35 / 37), while these disappear in the matrix
+// instruction's shadow.
+template <typename T> FMHA_DEV void sum_pair(typename Elem<T>::v8 v, int pair, float &lo, float &hi);
+template <> FMHA_DEV void sum_pair<_Float16>(f16x8 v, int pair, float &lo, float &hi) {
+  const uint32_t u = as_u32x4(v)[pair];
+  asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel_hi:[1,0,0]" : "+v"(lo) : "v"(u));
+  asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(hi) : "v"(u));
+}
+template <> FMHA_DEV void sum_pair<__bf16>(bf16x8 v, int pair, float &lo, float &hi) {
+  const uint32_t u = as_u32x4(v)[pair];
+  lo += __uint_as_float(u << 16);
+  hi += __uint_as_float(u & 0xffff0000u);
+}
+
 template <typename T, int D, int QB, int NW, int MASK, bool CAUSAL, int DROP, bool STRIDED = false>
 __global__ __launch_bounds__(NW * 64) void fmha_fwd_kernel(const FwdArgs a) {
   using RW = Rows<STRIDED, D>; // (run-time row layouts are built at head dim 256 only, where this is the only forward)

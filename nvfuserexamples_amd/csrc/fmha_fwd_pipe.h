@@ -543,11 +543,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
     const char *ldsV = ldsVb + (tprev & 1) * TILEB;
     const char *ldsK = ldsKb + (tnext & 1) * TILEB;
     const char *ldsX = ldsXb + (tnext & 1) * BK * XROWB;
+    float rs2[QB]; // the row sum runs on two accumulators
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       bk[qb] = mref[qb];
       lim[qb] = lim_now[qb];
       rs[qb] = 0.f;
+      rs2[qb] = 0.f;
     }
     auto fetch = [&](int j) -> v8 {
       if (ops.kind[j] == 0) return readV(ldsV, ops.a0[j], ops.a2[j], ops.a1[j]);
@@ -560,7 +562,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       const int c = pr / 4, j = pr % 4;
       pc[qb][sb][c][2 * j] = (T)e0;
       pc[qb][sb][c][2 * j + 1] = (T)e1;
-      rs[qb] = dot2_ones<T>(pc[qb][sb][c], j, rs[qb]);
+      sum_pair<T>(pc[qb][sb][c], j, rs[qb], rs2[qb]); // (fp32 sums of the rounded pair, not a packed dot product)
     };
     v8 opnd[ops.n];
 #pragma unroll
@@ -589,6 +591,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
       for (; done < upto; ++done) slice(done);
       __builtin_amdgcn_sched_barrier(0);
     }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) rs[qb] += rs2[qb];
   };
 
   // per-element work that cannot go through the matrix pipe: a full mask tensor, the causal test
@@ -618,7 +622,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
 
   // P = exp2(x + shift) rounded to T, and the row sum of the rounded values
   auto exp_pack = [&](const f32x16 (&x)[NSB], float shift, v8 (&pk)[NSB][2]) -> float {
-    float rs = 0.f;
+    float rs = 0.f, rs2 = 0.f;
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb) {
       float p[16];
@@ -629,10 +633,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu((QB == 
 #pragma unroll
         for (int j = 0; j < 8; ++j) pk[sb][c][j] = (T)p[8 * c + j];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) rs = dot2_ones<T>(pk[sb][c], j, rs);
+        for (int j = 0; j < 4; ++j) sum_pair<T>(pk[sb][c], j, rs, rs2);
       }
     }
-    return rs;
+    return rs + rs2;
   };
   // move the reference of query block qb to this tile's maximum (x is relative to bk);
   // returns the shift that re-bases x onto the new reference

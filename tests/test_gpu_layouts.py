@@ -167,15 +167,21 @@ def test_operators_and_autograd_take_strided_tensors():
         assert torch.equal(gp[:, :, i].permute(0, 2, 1, 3).reshape(a3.shape), a3)
 
 
-def test_headline_shape_packed_projection_equals_folded_path():
+def test_headline_shape_packed_projection_equals_folded_path(monkeypatch):
     """B32 H16 S512 D64 with a padding mask, read from a packed [B,S,3,H,D] buffer: at this shape the
-    forward deals the mask rows to its workgroups by length, in both layouts alike.  Full size, so the
-    check is bit-equality with the folded path (itself held to the oracle elsewhere), train step included."""
+    pipelined forward deals the mask rows to its workgroups by length, in both layouts alike.  Full size, so the
+    check is bit-equality with the folded path on the same kernel (itself held to the oracle elsewhere), train
+    step included.  (By default the folded layout takes the whole-head kernel at this shape, which walks the keys
+    in tiles of 32 instead of 64: its output agrees to the rounding of the element type, not bit for bit.)"""
     b, h, s, d = 32, 16, 512, 64
     q, k, v, do = make_qkv(b * h, s, s, d, seed=21, with_dout=True)
     kw = dict(mask=pad_mask(b, s, s // 2, s).half().cuda(), drop_kind=capi.DROP_PHILOX, p_drop=0.1, seed=3, offset=9)
     qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    o_head, l_head, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    monkeypatch.setenv("FMHA_FWD_HEAD", "0")
     o3, l3, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    assert (o_head.float() - o3.float()).abs().max().item() <= 2e-3
+    assert (l_head - l3).abs().max().item() <= 1e-3
     g3 = capi.bwd(doc, qc, kc, vc, o3, l3, **kw)
     q4, k4, v4 = _packed(qc, kc, vc, b, h)
     o4, l4, _, _ = capi.fwd(q4, k4, v4, want_lse=True, **kw)
