@@ -325,7 +325,15 @@ void fmha_reload_overrides(void);
  * one matrix only, one exponentials only (waves_per_simd must be 2); 5 matrix instructions whose A operand
  * is read from LDS every time; 6 those LDS reads alone; 7 as 2, but the exponentials read registers that the
  * matrix instructions of the previous trip wrote; 8 as 2, but the B operand of every matrix instruction is packed
- * from exponentials of the previous trip.  random_data: 0 all-zero operands, 1 pseudo-random
+ * from exponentials of the previous trip; 9-11 the attention kernels' mix of two exponentials, a packing conversion,
+ * a packed dot product and an integer add behind every matrix instruction (on registers of their own / reading what
+ * the matrix instructions wrote / also feeding their B operand); 12-35 nexp instructions of ONE kind behind every
+ * matrix instruction: 12 v_dot2c_f32_f16, 13 v_cvt_f16_f32 + v_pack_b32_f16, 14 v_add_f32, 15 v_pk_add_f16,
+ * 16 v_cvt_pk_f16_f32, 17 v_exp_f32, 18 (nexp = 5) two exponentials + one packing conversion + two adds,
+ * 19 v_fma_mix_f32, 20 v_mad_u64_u32, 21 v_bitop3_b32, 22 v_mov_b32 with a DPP quad permutation, 23 v_pk_sub_i16,
+ * 24 v_perm_b32, 25 v_cndmask_b32, 26 v_mul_f32, 27 v_fma_f32, 28 v_pk_mul_f16, 29 v_max3_f32,
+ * 30 v_permlane32_swap_b32, 31 v_cvt_f32_f16, 32 v_dot2_f32_f16, 33 v_sub_f32, 34 v_and_b32, 35 v_pk_ashrrev_i16.
+ * random_data: 0 all-zero operands, 1 pseudo-random
  * ones in [-1, 1) -- the board's power management sets the core clock by what the data toggles.
  * Runs `launches` launches (the second half timed with events) of `iters` loop trips -- 4 matrix
  * instructions and / or 4 * nexp exponentials per trip and wave -- with waves_per_simd (1 or 2) waves on

@@ -539,14 +539,21 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
 
     FMHA_TL(); // 0: item start
     if (cold) {
-      // Every wave has left the previous item (its tiles and extra rows are about to be overwritten); tiles 0-3 of
-      // K and 0-1 of V go first, and the compiler's own wait for the Q rows requested behind them covers them.
+      // Every wave has left the previous item (its tiles and extra rows are about to be overwritten).  Tiles 0-3
+      // of K and 0-1 of V and the mask values go first, the Q rows behind them: the barrier below needs every
+      // wave's part of the former, but a wave's Q rows are its own business, so it comes BEFORE the wait for them
+      // and a wave starts computing as soon as its own rows are there.
       if (idx != (int)blockIdx.x) lds_barrier();
       dmaK(cur, 0);
       dmaV(cur, 0);
       if (UT == 2) dmaK(cur, 1);
-      loadQ(cur);
       xm = load_xm(cur);
+      loadQ(cur);
+      __builtin_amdgcn_sched_barrier(0);
+      storeX(xm, cur.kend, xb); // (the compiler's wait for the mask value leaves the QB * KS loads behind it in flight)
+      __builtin_amdgcn_sched_barrier(0);
+      vm_wait<QB * KS>();       // this wave's part of the first tiles is in LDS
+      lds_barrier();            // ... and everybody's, and the extra rows
     } else {
       // Requested before the previous item's output stores: wait for everything but those stores.
       switch (__builtin_amdgcn_readfirstlane(nst)) {
@@ -559,7 +566,7 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
     }
     __builtin_amdgcn_sched_barrier(0);
     const Item nxt = make_item(more ? nidx : idx);
-    FMHA_TL(); // 1: requests out (cold) / waited (warm)
+    FMHA_TL(); // 1: requests out and first tiles in (cold) / waited (warm)
     // Q' = Q * scale * log2(e), rounded once, as B-operand registers
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb)
@@ -570,10 +577,9 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
         for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
       }
     if (cold) {
-      storeX(xm, cur.kend, xb);
       __builtin_amdgcn_sched_barrier(0);
-      vm_wait<0>(); // (nothing new: the loads above have been consumed) this wave's part of the first tiles is in LDS
-      // the rest in the order of its use; hook 3 waits for the first kColdHook3 of these
+      // (the Q rows have been consumed: nothing of this wave's is in flight)  The rest of the item's rows in the
+      // order of their use; hook 3 waits for the first of them
       if (UT == 2) {
         dmaV(cur, 1);
         dmaK(cur, 2);
@@ -607,9 +613,8 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
         bx[qb][2] = (T)1.f;
       }
     }
-    FMHA_TL(); // 2: before the start barrier
-    if (cold) lds_barrier(); // the extra rows and everybody's part of the first tiles are in LDS
-    FMHA_TL(); // 3: start barrier passed
+    FMHA_TL(); // 2: Q converted, state cleared
+    FMHA_TL(); // 3
     const int nkt2 = tiles2(trimmed_keys(cur.kend, xb));
     const int np = units_of(cur), npn = units_of(nxt);
     // copies a cold item still has in flight at its hook 3 once those that iterations 3-6 read have landed

@@ -48,6 +48,10 @@ __global__ __launch_bounds__(512) void pipe_probe_kernel(unsigned long long *out
   typedef _Float16 h2p __attribute__((ext_vector_type(2)));
   h2p ppk[4] = {{a[0], a[1]}, {a[2], a[3]}, {b[0], b[1]}, {b[2], b[3]}};
   uint32_t cnt = (uint32_t)tid;
+  uint32_t iv[8];
+  unsigned long long lv[4] = {1ull, 2ull, 3ull, 4ull};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) iv[j] = (uint32_t)tid * 2654435761u + (uint32_t)j;
   const unsigned long long r0 = __builtin_amdgcn_s_memrealtime(), c0 = __builtin_readcyclecounter();
   for (int it = 0; it < iters; ++it) {
     if (MODE == 3) { // dependent chain: one accumulator
@@ -59,6 +63,34 @@ __global__ __launch_bounds__(512) void pipe_probe_kernel(unsigned long long *out
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < NEXP; ++j) v[(i * NEXP + j) & 7] = __builtin_amdgcn_exp2f(v[(i * NEXP + j) & 7] * 0.5f - 1.0f);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else if (MODE >= 20 && MODE <= 35) {
+      // NEXP instructions of one kind (inline assembly, registers of their own) behind every matrix instruction
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < NEXP; ++j) {
+          const int r = (i * NEXP + j) & 7;
+          uint32_t &x = iv[r], &y = iv[(r + 3) & 7];
+          if (MODE == 20) asm volatile("v_mad_u64_u32 %0, vcc, %1, %2, %0" : "+v"(lv[r & 3]) : "v"(x), "v"(y) : "vcc");
+          if (MODE == 21) asm volatile("v_bitop3_b32 %0, %0, %1, %2 bitop3:0x96" : "+v"(x) : "v"(y), "v"(iv[(r + 5) & 7]));
+          if (MODE == 22) asm volatile("v_mov_b32_dpp %0, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(x) : "v"(y));
+          if (MODE == 23) asm volatile("v_pk_sub_i16 %0, %0, %1" : "+v"(x) : "v"(y));
+          if (MODE == 24) asm volatile("v_perm_b32 %0, %0, %1, %2" : "+v"(x) : "v"(y), "v"(iv[(r + 5) & 7]));
+          if (MODE == 25) asm volatile("v_cndmask_b32 %0, %0, %1, vcc" : "+v"(x) : "v"(y) : "vcc");
+          if (MODE == 26) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(x) : "v"(y));
+          if (MODE == 27) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x) : "v"(y), "v"(iv[(r + 5) & 7]));
+          if (MODE == 28) asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(x) : "v"(y));
+          if (MODE == 29) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(x) : "v"(y), "v"(iv[(r + 5) & 7]));
+          if (MODE == 30) asm volatile("v_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y));
+          if (MODE == 31) asm volatile("v_cvt_f32_f16 %0, %1" : "=v"(x) : "v"(y));
+          if (MODE == 32) asm volatile("v_dot2_f32_f16 %0, %1, %2, %0" : "+v"(x) : "v"(y), "v"(iv[(r + 5) & 7]));
+          if (MODE == 33) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(x) : "v"(y));
+          if (MODE == 34) asm volatile("v_and_b32 %0, %0, %1" : "+v"(x) : "v"(y));
+          if (MODE == 35) asm volatile("v_pk_ashrrev_i16 %0, 15, %0" : "+v"(x));
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     } else if (MODE >= 12 && MODE <= 19) {
@@ -173,6 +205,9 @@ __global__ __launch_bounds__(512) void pipe_probe_kernel(unsigned long long *out
     for (int r = 0; r < 16; ++r) s += acc[i][r];
 #pragma unroll
   for (int j = 0; j < 8; ++j) s += v[j] + (float)bw[0][j] + (float)bw[1][j] + pe[j];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s += (float)iv[j];
+  s += (float)(lv[0] + lv[1] + lv[2] + lv[3]);
   s += rsum + (float)cnt + (float)ppk[0][0] + (float)ppk[1][0] + (float)ppk[2][0] + (float)ppk[3][0];
   if ((tid & 63) == 0 && (w == 0 || w == 4)) {
     unsigned long long *o = out + ((size_t)blockIdx.x * 2 + (w >> 2)) * 3;
@@ -206,6 +241,10 @@ template <int MODE, int NEXP> void launch_probe(int grid, int threads, unsigned 
 // 5 matrix instructions with the A operand read from LDS each time; 6 those LDS reads alone; 7 as 2, the
 // exponentials reading registers that the matrix instructions of the previous trip wrote; 8 as 2, the B operand of
 // the matrix instructions packed from the exponentials of the previous trip.
+// 20-35: nexp instructions of one kind behind every matrix instruction, on registers of their own: 20 v_mad_u64_u32,
+// 21 v_bitop3_b32, 22 v_mov_b32 with a DPP quad permutation, 23 v_pk_sub_i16, 24 v_perm_b32, 25 v_cndmask_b32,
+// 26 v_mul_f32, 27 v_fma_f32, 28 v_pk_mul_f16, 29 v_max3_f32, 30 v_permlane32_swap_b32, 31 v_cvt_f32_f16,
+// 32 v_dot2_f32_f16, 33 v_sub_f32, 34 v_and_b32, 35 v_pk_ashrrev_i16.
 // random_data: 0 all-zero operands, 1 pseudo-random in [-1, 1).  waves_per_simd: 1 or 2.
 // Runs `launches` launches of `iters` loop trips (4 matrix instructions and/or 4 * nexp exponentials per trip and
 // wave) on every compute unit, times the second half of them with events, and writes
@@ -216,7 +255,7 @@ template <int MODE, int NEXP> void launch_probe(int grid, int threads, unsigned 
 extern "C" int fmha_pipe_probe(int mode, int nexp, int random_data, int waves_per_simd, int iters, int launches,
                                double *result) {
   using namespace fmha;
-  if (!result || mode < 0 || mode > 19 || (waves_per_simd != 1 && waves_per_simd != 2) || iters <= 0 || launches < 2)
+  if (!result || mode < 0 || mode > 35 || (waves_per_simd != 1 && waves_per_simd != 2) || iters <= 0 || launches < 2)
     return -1;
   if (nexp != 2 && nexp != 4 && nexp != 6 && nexp != 5) return -1;
   if (mode == 4 && waves_per_simd != 2) return -1;
@@ -268,6 +307,22 @@ extern "C" int fmha_pipe_probe(int mode, int nexp, int random_data, int waves_pe
       FMHA_PROBE_CASE(17)
       FMHA_PROBE_CASE(18)
       FMHA_PROBE_CASE(19)
+      FMHA_PROBE_CASE(20)
+      FMHA_PROBE_CASE(21)
+      FMHA_PROBE_CASE(22)
+      FMHA_PROBE_CASE(23)
+      FMHA_PROBE_CASE(24)
+      FMHA_PROBE_CASE(25)
+      FMHA_PROBE_CASE(26)
+      FMHA_PROBE_CASE(27)
+      FMHA_PROBE_CASE(28)
+      FMHA_PROBE_CASE(29)
+      FMHA_PROBE_CASE(30)
+      FMHA_PROBE_CASE(31)
+      FMHA_PROBE_CASE(32)
+      FMHA_PROBE_CASE(33)
+      FMHA_PROBE_CASE(34)
+      FMHA_PROBE_CASE(35)
     }
 #undef FMHA_PROBE_CASE
   };
