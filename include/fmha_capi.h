@@ -332,14 +332,17 @@ void fmha_reload_overrides(void);
  * 16 v_cvt_pk_f16_f32, 17 v_exp_f32, 18 (nexp = 5) two exponentials + one packing conversion + two adds,
  * 19 v_fma_mix_f32, 20 v_mad_u64_u32, 21 v_bitop3_b32, 22 v_mov_b32 with a DPP quad permutation, 23 v_pk_sub_i16,
  * 24 v_perm_b32, 25 v_cndmask_b32, 26 v_mul_f32, 27 v_fma_f32, 28 v_pk_mul_f16, 29 v_max3_f32,
- * 30 v_permlane32_swap_b32, 31 v_cvt_f32_f16, 32 v_dot2_f32_f16, 33 v_sub_f32, 34 v_and_b32, 35 v_pk_ashrrev_i16.
+ * 30 v_permlane32_swap_b32, 31 v_cvt_f32_f16, 32 v_dot2_f32_f16, 33 v_sub_f32, 34 v_and_b32, 35 v_pk_ashrrev_i16;
+ * 36 nexp v_xor_b32 behind every matrix instruction and 37 the same v_xor_b32 alone (these two also take
+ * nexp = 8, 16 and 32: how much vector work a matrix instruction hides, and the plain vector issue rate).
  * random_data: 0 all-zero operands, 1 pseudo-random
  * ones in [-1, 1) -- the board's power management sets the core clock by what the data toggles.
  * Runs `launches` launches (the second half timed with events) of `iters` loop trips -- 4 matrix
  * instructions and / or 4 * nexp exponentials per trip and wave -- with waves_per_simd (1 or 2) waves on
  * every SIMD of the current device and writes
  *   result[0] microseconds per launch, result[1] mean core clock in MHz as the waves saw it,
- *   result[2] matrix TFLOP/s (0 without matrix work), result[3] exponentials per nanosecond over the chip.
+ *   result[2] matrix TFLOP/s (0 without matrix work), result[3] exponentials (modes 36, 37: v_xor_b32 lane results)
+ *   per nanosecond over the chip.
  * Unlike the launch functions it allocates and frees buffers of its own and synchronises the device.
  * Returns 0, or -1 on a bad argument or a HIP error.
  */

@@ -65,6 +65,18 @@ __global__ __launch_bounds__(512) void pipe_probe_kernel(unsigned long long *out
         for (int j = 0; j < NEXP; ++j) v[(i * NEXP + j) & 7] = __builtin_amdgcn_exp2f(v[(i * NEXP + j) & 7] * 0.5f - 1.0f);
         __builtin_amdgcn_sched_barrier(0);
       }
+    } else if (MODE == 36 || MODE == 37) {
+      // NEXP full-rate vector instructions (v_xor_b32) behind every matrix instruction (36) or alone (37)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (MODE == 36) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[i], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < NEXP; ++j) {
+          const int r = (i * NEXP + j) & 7;
+          asm volatile("v_xor_b32 %0, %0, %1" : "+v"(iv[r]) : "v"(iv[(r + 3) & 7]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     } else if (MODE >= 20 && MODE <= 35) {
       // NEXP instructions of one kind (inline assembly, registers of their own) behind every matrix instruction
 #pragma unroll
@@ -244,7 +256,8 @@ template <int MODE, int NEXP> void launch_probe(int grid, int threads, unsigned 
 // 20-35: nexp instructions of one kind behind every matrix instruction, on registers of their own: 20 v_mad_u64_u32,
 // 21 v_bitop3_b32, 22 v_mov_b32 with a DPP quad permutation, 23 v_pk_sub_i16, 24 v_perm_b32, 25 v_cndmask_b32,
 // 26 v_mul_f32, 27 v_fma_f32, 28 v_pk_mul_f16, 29 v_max3_f32, 30 v_permlane32_swap_b32, 31 v_cvt_f32_f16,
-// 32 v_dot2_f32_f16, 33 v_sub_f32, 34 v_and_b32, 35 v_pk_ashrrev_i16.
+// 32 v_dot2_f32_f16, 33 v_sub_f32, 34 v_and_b32, 35 v_pk_ashrrev_i16.  36: nexp v_xor_b32 behind every matrix
+// instruction; 37: those v_xor_b32 alone (both also with nexp = 8, 16, 32).
 // random_data: 0 all-zero operands, 1 pseudo-random in [-1, 1).  waves_per_simd: 1 or 2.
 // Runs `launches` launches of `iters` loop trips (4 matrix instructions and/or 4 * nexp exponentials per trip and
 // wave) on every compute unit, times the second half of them with events, and writes
@@ -255,9 +268,10 @@ template <int MODE, int NEXP> void launch_probe(int grid, int threads, unsigned 
 extern "C" int fmha_pipe_probe(int mode, int nexp, int random_data, int waves_per_simd, int iters, int launches,
                                double *result) {
   using namespace fmha;
-  if (!result || mode < 0 || mode > 35 || (waves_per_simd != 1 && waves_per_simd != 2) || iters <= 0 || launches < 2)
+  if (!result || mode < 0 || mode > 37 || (waves_per_simd != 1 && waves_per_simd != 2) || iters <= 0 || launches < 2)
     return -1;
-  if (nexp != 2 && nexp != 4 && nexp != 6 && nexp != 5) return -1;
+  const bool wide = mode >= 36; // these two modes also take 8, 16 and 32 instructions per group
+  if (nexp != 2 && nexp != 4 && nexp != 6 && nexp != 5 && !(wide && (nexp == 8 || nexp == 16 || nexp == 32))) return -1;
   if (mode == 4 && waves_per_simd != 2) return -1;
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
@@ -323,6 +337,19 @@ extern "C" int fmha_pipe_probe(int mode, int nexp, int random_data, int waves_pe
       FMHA_PROBE_CASE(33)
       FMHA_PROBE_CASE(34)
       FMHA_PROBE_CASE(35)
+#define FMHA_PROBE_WIDE(M)                                                                  \
+  case M:                                                                                   \
+    if (nexp == 2) launch_probe<M, 2>(grid, threads, out, src, iters, s);                   \
+    else if (nexp == 4) launch_probe<M, 4>(grid, threads, out, src, iters, s);              \
+    else if (nexp == 5) launch_probe<M, 5>(grid, threads, out, src, iters, s);              \
+    else if (nexp == 6) launch_probe<M, 6>(grid, threads, out, src, iters, s);              \
+    else if (nexp == 8) launch_probe<M, 8>(grid, threads, out, src, iters, s);              \
+    else if (nexp == 16) launch_probe<M, 16>(grid, threads, out, src, iters, s);            \
+    else launch_probe<M, 32>(grid, threads, out, src, iters, s);                            \
+    break;
+      FMHA_PROBE_WIDE(36)
+      FMHA_PROBE_WIDE(37)
+#undef FMHA_PROBE_WIDE
     }
 #undef FMHA_PROBE_CASE
   };
@@ -345,8 +372,8 @@ extern "C" int fmha_pipe_probe(int mode, int nexp, int random_data, int waves_pe
       tick += (double)host[3 * i + 1];
     }
     const double us = (double)ms * 1e3 / timed;
-    const bool has_mfma = mode != 0 && mode != 6;
-    const bool has_exp = mode == 0 || mode == 2 || mode == 4 || mode >= 7;
+    const bool has_mfma = mode != 0 && mode != 6 && mode != 37;
+    const bool has_exp = mode == 0 || mode == 2 || mode == 4 || mode >= 7; // (modes 36, 37: the v_xor_b32 count)
     const double mfma_waves = (double)grid * (mode == 4 ? 4 : 4 * waves_per_simd);
     const double exp_waves = (double)grid * (mode == 4 ? 4 : 4 * waves_per_simd);
     result[0] = us;
