@@ -40,11 +40,23 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA
 PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E
-# HBM bytes per launch of the headline forward kernel with every key tile visited, as counted by rocprofv3
-# (FETCH_SIZE 49 329.3 x 2.000 + WRITE_SIZE 32 768.0 x 1.000 KiB, the factors from 256 MiB copies in the same
-# runs: profiles/fmha_fwd_pipe_kernel_B32H16S512D64_f16.md).  A counter reading of the build as profiled,
-# not something this script can measure; the algorithmic figure is computed beside it.
-MEASURED_TRAFFIC_BYTES = int((98658.6 + 32768.0) * 1024)
+# HBM bytes per launch of the headline forward kernel (every key tile visited) as rocprofv3 counted them
+# (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy in the same run):
+# a counter reading of the build that was profiled, not something this script can measure.  It is read from
+# a tracked file that names the commit it was taken at, so that a stale figure shows as such.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+HEADLINE_KERNEL = "fmha_fwd_head_kernel<f16,QB2,per-key mask,no dropout>"
+
+
+def measured_traffic(key):
+    """(bytes per launch, commit the counters were read at) from profiles/traffic.json, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            e = json.load(f)[key]
+        return int(e["bytes_per_launch"]), e.get("commit")
+    except (OSError, KeyError, ValueError, TypeError):
+        return None, None
+
 
 B, H, S, D = 32, 16, 512, 64
 
@@ -336,6 +348,22 @@ def operator_legs(torch, steps, warmup):
         _, graph_ms = time_steps(torch, lambda i: graph.replay(), steps, warmup)
         legs[name] = {"eager_us_per_call": round(eager_ms * 1e3, 2), "graph_replay_us_per_call": round(graph_ms * 1e3, 2)}
         del graph, keep
+    # the reference's own protocol on the same operators and inputs (reference perf_measurement.py:29-50,
+    # perf_measurement_train.py:35-60): 10 warm-up calls, then 1000 calls under no_grad between two events
+    # on the current stream, one input set, outputs allocated per call
+    for name, fn in calls.items():
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.no_grad():
+            for _ in range(10):
+                fn()
+            start.record()
+            for _ in range(1000):
+                fn()
+            stop.record()
+        start.synchronize()
+        stop.synchronize()
+        legs[name]["reference_protocol_us_per_call"] = round(start.elapsed_time(stop), 2)  # ms / 1000 calls = us per call
+    legs["reference_protocol"] = "10 warm-up + 1000 timed calls of torch.ops.mha_manual.<op> under no_grad between two events"
     return legs
 
 
@@ -629,37 +657,37 @@ def torch_sdpa_context(torch, steps, warmup):
     return out
 
 
-def power_probe(torch, step, seconds=2.0):
-    """Socket power and graphics clocks as the board's management firmware reports them (amd-smi),
-    sampled while `step` runs back to back on a second thread.  The attention kernels are
-    power-limited on this part, so the figures belong beside the roofline fraction: the MFMA peak
-    is quoted at the maximum clock, which the board does not hold under this load.
-    Returns None where the tool is missing or its output has no such fields."""
+def smi_sample():
+    """One reading of socket power and graphics clocks from the board's management firmware (amd-smi), or None."""
     import re
     import shutil
     import subprocess
-    import threading
     exe = shutil.which("amd-smi") or "/opt/rocm/bin/amd-smi"
     if not os.path.exists(exe):
         return None
+    try:
+        r = subprocess.run([exe, "metric", "-g", "0", "-c", "-p"], stdout=subprocess.PIPE,
+                           stderr=subprocess.DEVNULL, text=True, timeout=20)
+    except Exception:
+        return None
+    pw = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", r.stdout)
+    clk = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", r.stdout)]
+    mx = re.search(r"MAX_CLK:\s*(\d+)\s*MHz", r.stdout)
+    if not pw or not clk:
+        return None
+    return {"socket_power_w": int(pw.group(1)), "gfx_clk_mhz_mean": round(sum(clk) / len(clk)),
+            "gfx_clk_mhz_min": min(clk), "gfx_max_clk_mhz": int(mx.group(1)) if mx else None}
 
-    def sample():
-        try:
-            r = subprocess.run([exe, "metric", "-g", "0", "-c", "-p"], stdout=subprocess.PIPE,
-                               stderr=subprocess.DEVNULL, text=True, timeout=20)
-        except Exception:
-            return None
-        pw = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", r.stdout)
-        clk = [int(m) for m in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", r.stdout)]
-        mx = re.search(r"MAX_CLK:\s*(\d+)\s*MHz", r.stdout)
-        if not pw or not clk:
-            return None
-        return {"socket_power_w": int(pw.group(1)), "gfx_clk_mhz_mean": round(sum(clk) / len(clk)),
-                "gfx_clk_mhz_min": min(clk), "gfx_max_clk_mhz": int(mx.group(1)) if mx else None}
 
+def power_probe(torch, step, idle, seconds=2.0):
+    """Socket power and graphics clocks as the board's management firmware reports them (amd-smi),
+    sampled while `step` runs back to back on a second thread; `idle` is a reading taken before the
+    process touched the GPU.  The firmware's clock is the frequency it has set (a target, read at one
+    instant per die); the clock the waves really saw is `effective_core_clock_mhz` (cycle counter over the
+    100 MHz counter inside the kernel).  Returns None where the tool is missing or its output has no such fields."""
+    import threading
+    sample = smi_sample
     torch.cuda.synchronize()
-    time.sleep(0.5)
-    idle = sample()
     stop = [False]
 
     def load():
@@ -684,26 +712,24 @@ def power_probe(torch, step, seconds=2.0):
     if not idle or not busy:
         return None
     top = max(busy, key=lambda b: b["socket_power_w"])
-    return {"tool": "amd-smi metric -c -p, sampled while the headline kernel runs back to back",
+    return {"tool": "amd-smi metric -c -p: idle before the process's first GPU work, busy while the headline kernel runs back to back",
             "idle_socket_power_w": idle["socket_power_w"], "busy_socket_power_w": top["socket_power_w"],
             "busy_gfx_clk_mhz_mean": top["gfx_clk_mhz_mean"], "busy_gfx_clk_mhz_min": top["gfx_clk_mhz_min"],
             "gfx_max_clk_mhz": top["gfx_max_clk_mhz"], "samples": len(busy)}
 
 
-def cpu_baseline(torch, budget_s=12.0):
+def _cpu_eager_leg(torch, b, h, s, d, lo, budget_s, min_iters):
     """The reference's eager composition (its ground truth, reference test.py:12-18: matmul, mask add, softmax,
-    matmul) on the host cores in fp32, on a bounded sample of the headline workload: 2 of its 32 sequences (32 of
-    the 512 heads, S 512, D 64, the same kind of padding mask), repeated for about 12 s."""
+    matmul) on the host cores in fp32: b sequences of h heads, padding mask with valid lengths U{lo..s}; 3 warm-up
+    calls, then calls until both `min_iters` and `budget_s` seconds are reached."""
     from oracle import eager
-    b, h, s, d = 2, H, S, D
     g = torch.Generator().manual_seed(0)
     q, k, v = (torch.randn(b * h, s, d, generator=g) for _ in range(3))
-    lens = torch.randint(s // 2, s + 1, (b,), generator=g)
+    lens = torch.randint(lo, s + 1, (b,), generator=g)
     keep = torch.zeros(b, 1, s)
     for i in range(b):
         keep[i, 0, :lens[i]] = 1.0
     keep = keep.repeat_interleave(h, 0)  # [bh,1,s] 0/1 mask as the inference op takes it
-    cores = torch.get_num_threads()
     for _ in range(3):
         eager.infer_mha(q, k, v, keep)
     n, t0 = 0, time.perf_counter()
@@ -711,13 +737,103 @@ def cpu_baseline(torch, budget_s=12.0):
         eager.infer_mha(q, k, v, keep)
         n += 1
         el = time.perf_counter() - t0
-        if el > budget_s or n >= 200000:
+        if (el > budget_s and n >= min_iters) or n >= 2000000:
             break
-    flops = 4.0 * b * h * s * s * d
+    return n, el, 4.0 * b * h * s * s * d
+
+
+def pipe_ceilings(torch, capi, L, stream, fwd_params_of, time_it):
+    """What the compute units sustain on loops of nothing but the instructions in question (fmha_pipe_probe of the
+    C ABI: two waves on every SIMD of the chip, four matrix instructions per loop trip and wave, 2000 trips), and the
+    headline kernel on all-zero operands.  Each entry: TFLOP/s of the 32x32x16 fp16 matrix instructions, the core
+    clock the waves saw, and for the mixes the share of the matrix-only rate at the same data.  Diagnostic, never
+    part of `value`."""
+    res = (C.c_double * 4)()
+
+    def probe(mode, n, rnd, wps=2, iters=2000):
+        if L.fmha_pipe_probe(mode, n, rnd, wps, iters, 6, res) != 0:
+            return None
+        return {"us": round(res[0], 1), "clock_mhz": round(res[1]), "mfma_tflops": round(res[2], 1)}
+    out = {"protocol": "fmha_pipe_probe(mode, n, random_data, waves_per_simd=2, iters=2000, launches=6), second half of "
+                       "the launches timed between events; MI355X dense fp16 peak 2500 TFLOP/s = one 32x32x16 matrix "
+                       "instruction per 32 cycles and SIMD at 2400 MHz"}
+    for rnd, tag in ((0, "zero_data"), (1, "random_data")):
+        base = probe(1, 2, rnd)
+        if base is None:
+            return {"unavailable": "fmha_pipe_probe failed"}
+        e = {"mfma_only": base, "mfma_only_one_wave_per_simd": probe(1, 2, rnd, wps=1),
+             "mfma_one_accumulator_chain": probe(3, 2, rnd)}
+        for name, mode, n in (("mfma_plus_2_exp", 2, 2), ("mfma_plus_4_exp", 2, 4), ("mfma_plus_6_exp", 2, 6),
+                              ("mfma_plus_softmax_mix_2exp_1cvt_2add", 18, 5),
+                              ("mfma_plus_4_v_dot2c_f32_f16", 12, 4), ("mfma_plus_4_v_fma_mix_f32", 19, 4),
+                              ("mfma_plus_4_v_xor", 36, 4), ("mfma_plus_8_v_xor", 36, 8),
+                              ("mfma_plus_16_v_xor", 36, 16), ("mfma_plus_32_v_xor", 36, 32),
+                              ("sibling_waves_one_mfma_one_exp", 4, 4)):
+            r = probe(mode, n, rnd)
+            if r:
+                r["share_of_mfma_only"] = round(r["mfma_tflops"] / base["mfma_tflops"], 3)
+                # core cycles per group of one matrix instruction and its n vector instructions, per SIMD
+                r["cycles_per_group"] = round(r["us"] * r["clock_mhz"] / (2 * 2000 * 4), 1)
+            e[name] = r
+        v = probe(37, 16, rnd)
+        if v:
+            v["cycles_per_vector_instruction_per_simd"] = round(v["us"] * v["clock_mhz"] / (2 * 2000 * 4 * 16), 2)
+            v.pop("mfma_tflops")
+        e["v_xor_only_16_per_group"] = v
+        v1 = probe(37, 16, rnd, wps=1)
+        if v1:
+            v1["cycles_per_vector_instruction_per_simd"] = round(v1["us"] * v1["clock_mhz"] / (2000 * 4 * 16), 2)
+            v1.pop("mfma_tflops")
+        e["v_xor_only_16_per_group_one_wave_per_simd"] = v1
+        out[tag] = e
+    # the headline kernel on all-zero q, k, v (same masks): same instruction stream, nothing toggles
+    g = torch.Generator().manual_seed(0)
+    zs = []
+    for _ in range(2):
+        z = {n: torch.zeros(B * H, S, D, dtype=torch.float16, device="cuda") for n in ("q", "k", "v")}
+        z["o"] = torch.empty_like(z["q"])
+        lens = torch.randint(S // 2, S + 1, (B,), generator=g)
+        m = torch.zeros(B, 1, 1, S)
+        for b in range(B):
+            m[b, 0, 0, lens[b]:] = -10000.0
+        z["mask"] = m.to(torch.float16).cuda()
+        zs.append(z)
+    zp = [fwd_params_of(z) for z in zs]
+    capi.check(L.fmha_fwd_launch(C.byref(zp[0]), stream))
+    ms0 = time_it(lambda i: L.fmha_fwd_launch(C.byref(zp[i % 2]), stream))
+    probe_buf = torch.zeros(4, dtype=torch.int64, device="cuda")
+    zp[0].clock_probe = probe_buf.data_ptr()
+    for i in range(61):
+        L.fmha_fwd_launch(C.byref(zp[(i + 1) % 2]), stream)   # ends on set 0
+    torch.cuda.synchronize()
+    zp[0].clock_probe = None
+    c0, t0, c1, t1 = probe_buf.tolist()
+    out["headline_kernel_zero_inputs"] = {"us": round(ms0 * 1e3, 2),
+                                          "tflops": round(4.0 * B * H * S * S * D / (ms0 * 1e-3) / 1e12, 1),
+                                          "effective_core_clock_mhz": round((c1 - c0) / ((t1 - t0) / 100.0), 1) if t1 > t0 else None}
+    return out
+
+
+def cpu_baseline(torch, budget_s=10.0):
+    """The CPU baseline on the configuration the reference can run on a CPU: BERT-base attention forward, batch 8,
+    heads 12, sequence 128, head dim 64, additive [8,1,1,128] padding mask (valid lengths U{64..128}), the eager
+    fp32 composition on the host cores: 3 warm-up calls, then at least 20 timed calls (about 10 s of them)."""
+    cores = torch.get_num_threads()
+    n, el, flops = _cpu_eager_leg(torch, 8, 12, 128, 64, 64, budget_s, 20)
     return {"value": round(flops * n / el / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"{n} iterations of the eager fp32 composition (matmul, mask add, softmax, matmul) over {b} of "
-                      f"the workload's {B} sequences (B{b} H{h} S{s} D{d}, padding mask) in {el:.1f} s, torch CPU with "
-                      f"{cores} threads",
+            "sample": f"B8 H12 S128 D64 fp32, [8,1,1,128] padding mask: 3 warm-up + {n} timed calls of the eager "
+                      f"composition (matmul, mask add, softmax, matmul) in {el:.1f} s, torch CPU with {cores} threads",
+            "ms_per_iter": round(el / n * 1e3, 4)}
+
+
+def cpu_headline_sample(torch, budget_s=6.0):
+    """The same composition on a bounded sample of the headline workload: 2 of its 32 sequences (32 of the 512
+    heads, S 512, D 64, the same kind of padding mask)."""
+    cores = torch.get_num_threads()
+    n, el, flops = _cpu_eager_leg(torch, 2, H, S, D, S // 2, budget_s, 5)
+    return {"value": round(flops * n / el / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{n} timed calls over 2 of the workload's {B} sequences (B2 H{H} S{S} D{D}, padding mask) in "
+                      f"{el:.1f} s, torch CPU with {cores} threads",
             "ms_per_iter": round(el / n * 1e3, 4)}
 
 
@@ -730,6 +846,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-bwd", action="store_true", help="skip the train-step (fwd+bwd) leg")
     ap.add_argument("--no-power", action="store_true", help="skip the socket power / clock telemetry leg")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the pipe-ceiling microbenchmarks")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 256 MiB device copy a few times: under `rocprofv3 --pmc FETCH_SIZE` "
                          "(or WRITE_SIZE) its known traffic calibrates the counter for the attention kernels")
@@ -744,6 +861,7 @@ def main():
               file=sys.stderr)
         return 2
 
+    idle_power = None if (args.no_power or args.profile) else smi_sample()  # before this process touches the GPU
     import torch
     from nvfuserexamples_amd import capi
     if not torch.cuda.is_available():
@@ -825,11 +943,11 @@ def main():
     # effective core clock while the headline kernel runs: counters of its first workgroup, read in the
     # middle of a back-to-back run (clock_probe of the C ABI)
     probe = torch.zeros(4, dtype=torch.int64, device="cuda")
-    fps[0].clock_probe = probe.data_ptr()
+    fps_dense[0].clock_probe = probe.data_ptr()
     for i in range(args.warmup + 60):
-        fwd_step(i + 1)  # ends on input set 0
+        fwd_dense(i + 1)  # ends on input set 0
     torch.cuda.synchronize()
-    fps[0].clock_probe = None
+    fps_dense[0].clock_probe = None
     c0, t0, c1, t1 = probe.tolist()
     eff_clock = round((c1 - c0) / ((t1 - t0) / 100.0), 1) if t1 > t0 else None
     # the same batches kept as a packed [B,S,3,H,D] projection output, read in place, with O written
@@ -861,12 +979,20 @@ def main():
         o4.permute(0, 2, 1, 3).contiguous()
     ms_perm, _ = time_steps(torch, permutes, max(10, args.steps // 4), 5)
     del pks, pps
-    power = None if args.no_power else power_probe(torch, fwd_step)
+    power = None if args.no_power else power_probe(torch, fwd_dense, idle_power)
+    ceilings = None
+    if not args.no_ceilings:
+        ceilings = pipe_ceilings(torch, capi, L, stream,
+                                 lambda t: fwd_params(capi, t, flags=capi.FLAG_NO_MASK_TRIM),
+                                 lambda step: time_steps(torch, step, args.steps, args.warmup)[0])
+        ceilings["headline_kernel_random_inputs"] = {"us": round(ms * 1e3, 2), "tflops": round(tflops, 1),
+                                                     "effective_core_clock_mhz": eff_clock}
     # share of the (query tile, 128-key tile pair) products the kernel really visits: it leaves out the tile
     # pairs that hold only hard-masked keys (their weights are exactly zero)
     visited = float(sum(((n.float() / 128).ceil() * 128 / S).mean().item() for n in lens) / len(lens))
     del sets, fps, fps_dense, lps, lens
 
+    traffic_bytes, traffic_commit = measured_traffic("fmha_fwd_head_kernel_B32H16S512D64_f16")
     out = {
         "metric": "MHA fwd TFLOP/s (B32,H16,S512,D64 fp16)", "value": round(tflops, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
@@ -881,11 +1007,11 @@ def main():
         "value_frac_of_mfma_peak": round(tflops / PEAK_MFMA_TFLOPS, 4),
         # achieved = algorithmic flops of one launch / launch duration (event pair per launch, median block);
         # traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what the
-        # counter reads for a 256 MiB copy (profiles/fmha_fwd_pipe_kernel_B32H16S512D64_f16.md)
+        # counter reads for a 256 MiB copy (profiles/traffic.json, profiles/fmha_fwd_head_kernel_B32H16S512D64_f16.md)
         "roofline": {"bound": "mfma", "achieved": round(tflops_launch, 2), "peak": PEAK_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tflops_launch / PEAK_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "fmha_fwd_pipe_kernel<f16,D64,per-key mask>", "flops_per_launch": flops,
+                     "traffic": traffic_bytes, "traffic_from_commit": traffic_commit,
+                     "kernel": HEADLINE_KERNEL, "flops_per_launch": flops,
                      "executed_frac": round(tflops_launch / PEAK_MFMA_TFLOPS, 4),   # every counted tile is visited
                      "visited_tile_share": 1.0,
                      "algorithmic_bytes_per_launch": bytes_,
@@ -922,6 +1048,7 @@ def main():
     out["fp8_e4m3_forward"] = fp8_leg(torch, capi, L, stream, args.steps, args.warmup)
     out["decode_steps"] = decode_leg(torch, capi, args.steps, args.warmup)
     out["power"] = power
+    out["pipe_ceilings"] = ceilings
     out["effective_core_clock_mhz"] = eff_clock  # MFMA peak is quoted at the maximum clock (2400 MHz)
 
     # ---- train step (forward with LSE + Philox dropout, then backward): every key tile visited, as the
@@ -1005,6 +1132,7 @@ def main():
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch)
+        out["cpu_baseline_headline_sample"] = cpu_headline_sample(torch)
     print(json.dumps(out))
     return 0
 

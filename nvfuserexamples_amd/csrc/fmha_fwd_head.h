@@ -228,10 +228,12 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
     return (const T *)a.q + ((size_t)it.bh * (size_t)a.sq + (size_t)q) * D + h * 8;
   };
   u32x4 qraw[QB][KS];
-  auto loadQ = [&](const Item &it) {
+  // (real = false: a request that must exist for the registers' sake but whose rows nobody will use -- every
+  // lane reads the tensor's first row, one cache line instead of the wave's 8 KB)
+  auto loadQ = [&](const Item &it, bool real = true) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      const T *row = q_row(it, qb);
+      const T *row = real ? q_row(it, qb) : (const T *)a.q + h * 8;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) qraw[qb][ks] = *(const u32x4 *)(row + ks * 16);
     }
@@ -694,8 +696,8 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
       hook(t);
       // The Q registers have had their last use: request the next item's rows.  (Unconditionally, so that the
       // raw rows are not a value that has to survive the whole item on the path that would not load them; an
-      // item that starts cold loads them again.)
-      loadQ(nxt);
+      // item that starts cold loads them again, and after the last item the request is for one row only.)
+      loadQ(nxt, more);
       FMHA_TL(); // last hook and Q request
       steady(t, std::integral_constant<int, 0>{}, Yes{}, xB, bkB, limB, xA, bkA, limA, pA, pB);
       FMHA_TL(); // last iteration
