@@ -768,7 +768,10 @@ def pipe_ceilings(torch, capi, L, stream, fwd_params_of, time_it):
                               ("mfma_plus_4_v_dot2c_f32_f16", 12, 4), ("mfma_plus_4_v_fma_mix_f32", 19, 4),
                               ("mfma_plus_4_v_xor", 36, 4), ("mfma_plus_8_v_xor", 36, 8),
                               ("mfma_plus_16_v_xor", 36, 16), ("mfma_plus_32_v_xor", 36, 32),
-                              ("sibling_waves_one_mfma_one_exp", 4, 4)):
+                              ("sibling_waves_one_mfma_one_exp", 4, 4),
+                              ("mfma_plus_4_v_cvt_pk_f16_f32", 16, 4), ("mfma_plus_4_v_mad_u64_u32", 20, 4),
+                              ("mfma_plus_4_v_bitop3_b32", 21, 4), ("mfma_plus_4_v_mov_b32_dpp", 22, 4),
+                              ("mfma_plus_4_v_cndmask_b32", 25, 4), ("mfma_plus_4_v_permlane32_swap", 30, 4)):
             r = probe(mode, n, rnd)
             if r:
                 r["share_of_mfma_only"] = round(r["mfma_tflops"] / base["mfma_tflops"], 3)
