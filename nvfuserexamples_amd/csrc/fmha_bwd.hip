@@ -11,7 +11,7 @@
 #else
 #define FMHA_TU_SHORT 0
 #endif
-#if FMHA_TU_D == 256
+#if FMHA_TU_D == 256 || defined(FMHA_BWD_FORCE_WIDE) // (the second: development builds, to measure the wave-pair kernel at narrower heads)
 #define FMHA_TU_WIDE 1
 #include "fmha_bwd_wide.h"
 #else
