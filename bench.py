@@ -555,7 +555,7 @@ def profile_leg(torch, capi, L, stream, args):
     leg = args.profile
     steps = []
     keep = []
-    if leg in ("fwd", "fwd_trim", "train", "train_one_pass"):
+    if leg in ("fwd", "fwd_trim", "train"):
         train = leg.startswith("train")
         sets = make_inputs(torch, capi, args.sets, seed=1 if train else 0, train=train)
         flags = 0 if leg == "fwd_trim" else capi.FLAG_NO_MASK_TRIM
@@ -564,12 +564,6 @@ def profile_leg(torch, capi, L, stream, args):
         keep += [sets, F]
         if train:
             Bp = [bwd_params(capi, t, flags=flags) for t in sets]
-            if leg == "train_one_pass":
-                need = int(L.fmha_bwd_workspace_bytes(B * H, S, S, D))
-                ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
-                for P in Bp:
-                    P.flags, P.workspace, P.workspace_bytes = flags | capi.FLAG_BWD_ONE_PASS, ws.data_ptr(), need
-                keep.append(ws)
             steps.append(lambda i: L.fmha_bwd_launch(C.byref(Bp[i % len(Bp)]), stream))
             keep.append(Bp)
     elif leg in ("c4", "c5", "d256"):
@@ -854,7 +848,7 @@ def main():
                     help="also run a plain 256 MiB device copy a few times: under `rocprofv3 --pmc FETCH_SIZE` "
                          "(or WRITE_SIZE) its known traffic calibrates the counter for the attention kernels")
     ap.add_argument("--profile", metavar="LEG", default=None,
-                    help="run only LEG's launches (fwd, fwd_trim, train, train_one_pass, c4, c5, d256, fp8, decode, "
+                    help="run only LEG's launches (fwd, fwd_trim, train, c4, c5, d256, fp8, decode, "
                          "decode_plain) and no "
                          "timing: for rocprofv3 runs in which every dispatch of a kernel is the same workload")
     args = ap.parse_args()
@@ -1101,16 +1095,6 @@ def main():
                                   mask_trim_tflops_dense_count=round(fl_t / (ms_tt * 1e-3) / 1e12, 2),
                                   mask_trim_visited_tile_share=round(vis_t, 4),
                                   mask_trim_tflops_executed=round(fl_t * vis_t / (ms_tt * 1e-3) / 1e12, 2))
-            # the one-pass backward (opt-in) on the same batches
-            need = int(L.fmha_bwd_workspace_bytes(B * H, S, S, D))
-            ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
-            for P in tb:
-                P.flags, P.workspace, P.workspace_bytes = capi.FLAG_BWD_ONE_PASS, ws.data_ptr(), need
-            if L.fmha_bwd_launch(C.byref(tb[0]), stream) == 0:
-                ms_b1, _ = time_steps(torch, bwd_step, args.steps, args.warmup)
-                out["fwd_bwd"]["one_pass_bwd_only_ms"] = round(ms_b1, 5)
-            for P in tb:
-                P.flags, P.workspace, P.workspace_bytes = 0, None, 0
             # the same train step with the valid lengths handed over as counts (kv_len) instead of the mask
             # tensor: same results, key tiles past a sequence's length skipped in all three kernels
             for P, n in zip(tf + tb, tlens + tlens):
@@ -1120,7 +1104,6 @@ def main():
                 ms_tl, _ = time_steps(torch, train_step, args.steps, args.warmup)
                 out["fwd_bwd"]["kv_len_ms_per_step"] = round(ms_tl, 5)
                 out["fwd_bwd"]["kv_len_speedup_vs_default_mask_path"] = round(ms_tt / ms_tl, 3)
-            del ws
         else:
             out["fwd_bwd"] = {"error": f"fwd rc={rc_f} bwd rc={rc_b}: " + L.fmha_strerror(rc_b or rc_f).decode()}
         del tsets

@@ -425,12 +425,6 @@ fmha_bwd(const at::Tensor &dout_, const at::Tensor &q_, const at::Tensor &k_, co
   set_mask_and_dropout(p, m, mask, q, k.s, p_drop, seed, offset);
   at::Tensor kv_keep;
   set_kv_len(p, kv_len, q.bh, kv_keep);
-  at::Tensor workspace;
-  if (const uint64_t need = fmha_bwd_workspace_bytes(p.bh, p.sq, p.sk, p.d)) {
-    workspace = at::empty({static_cast<int64_t>(need)}, q.t.options().dtype(at::kByte));
-    p.workspace = workspace.data_ptr();
-    p.workspace_bytes = need;
-  }
   const int rc = fmha_bwd_launch(&p, current_stream(q.t));
   TORCH_CHECK(rc == FMHA_OK, "mha_manual backward: ", fmha_strerror(rc));
   return std::make_tuple(dq, dk, dv);

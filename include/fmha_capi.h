@@ -55,12 +55,9 @@ enum {
  * exceeds every visible key's by more than 8800.  FMHA_FLAG_NO_MASK_TRIM makes them visit every tile
  * regardless. */
 enum {
-  FMHA_FLAG_NO_MASK_TRIM = 1,
-  /* backward only: take the one-pass kernel where it applies (head dim 64, up to 512 keys, no causal
-   * mask, no [.., sq, sk] mask tensor; beyond 256 keys only with `workspace`).  It forms scores,
-   * exponentials and dropout decisions once instead of once per kernel, and measures level with the
-   * default two-kernel path at best, so it is never chosen unasked. */
-  FMHA_FLAG_BWD_ONE_PASS = 2
+  FMHA_FLAG_NO_MASK_TRIM = 1
+  /* (value 2 asked for a one-pass backward kernel in earlier versions; it never beat the default and was
+   * removed: the bit is accepted and ignored) */
 };
 
 /* return codes */
@@ -254,7 +251,7 @@ typedef struct fmha_bwd_params {
   int32_t bh, sq, sk, d;
   int32_t dtype;
   float scale;
-  int32_t flags; /* 0 or FMHA_FLAG_NO_MASK_TRIM | FMHA_FLAG_BWD_ONE_PASS */
+  int32_t flags; /* 0 or FMHA_FLAG_NO_MASK_TRIM */
 
   const int32_t *kv_len; /* as in fmha_fwd_params; dk and dv rows at or past the count are zero */
   int32_t kv_len_bh_div;
@@ -264,10 +261,8 @@ typedef struct fmha_bwd_params {
   int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3], do_stride[3];
   int64_t dq_stride[3], dk_stride[3], dv_stride[3];
 
-  /* Optional scratch in device memory (16-byte aligned; contents before and after the call are
-   * meaningless), used with FMHA_FLAG_BWD_ONE_PASS only: with at least
-   * fmha_bwd_workspace_bytes(bh, sq, sk, d) bytes of it, heads of 257 to 512 keys can take the one-pass
-   * kernel, which keeps fp32 partial sums of dq there between the two halves of the key range. */
+  /* Reserved (earlier versions' one-pass backward kept partial sums there): no backward kernel uses a
+   * workspace; leave NULL / 0. */
   void *workspace;
   uint64_t workspace_bytes;
 } fmha_bwd_params;
@@ -277,7 +272,7 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);
 /*
  * The backward for callers that cannot allocate (no counterpart in the reference): code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  Same as fmha_bwd_launch, except that
- * `delta` and `workspace` of the struct are ignored: both come out of an array of
+ * `delta` of the struct is ignored: it comes out of an array of
  * 4 * fmha_bwd_noalloc_max_rows() bytes (8 MiB) that the library holds in the memory of every GPU it
  * runs on until the process ends.  bh * sq beyond fmha_bwd_noalloc_max_rows() is refused
  * (FMHA_E_SCRATCH).  The call allocates nothing and synchronises nothing.  All calls on one GPU share
@@ -288,7 +283,7 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);
 int fmha_bwd_launch_noalloc(const fmha_bwd_params *p, void *hip_stream);
 uint64_t fmha_bwd_noalloc_max_rows(void);
 
-/* Workspace the backward can make use of for these sizes (0: none). */
+/* Workspace the backward can make use of for these sizes: always 0 (kept for callers of earlier versions). */
 uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d);
 
 /*
@@ -312,8 +307,8 @@ float fmha_drop_scale(float p_drop);
 const char *fmha_strerror(int code);
 
 /* The FMHA_* environment variables -- tuning and test overrides of the variant selection: FMHA_MASK_TRIM,
- * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_FWD_HEAD, FMHA_BWD_SHORT, FMHA_BWD_PAIR,
- * FMHA_BWD_FUSED -- are read once per process, on the first launch.  This reads them again; not to be
+ * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_FWD_HEAD, FMHA_BWD_SHORT, FMHA_BWD_PAIR
+ * -- are read once per process, on the first launch.  This reads them again; not to be
  * called while another thread is launching.  (No counterpart in the reference.) */
 void fmha_reload_overrides(void);
 

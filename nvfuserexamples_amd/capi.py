@@ -13,7 +13,6 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfmha_hip.so")
 F16, BF16 = 0, 1
 MASK_NONE, MASK_ADDITIVE, MASK_KEEP01 = 0, 1, 2
 FLAG_NO_MASK_TRIM = 1  # fwd(flags=...): visit every key tile even where a per-key mask hard-masks the tail
-FLAG_BWD_ONE_PASS = 2  # bwd(flags=...): the one-pass backward kernel where it applies
 DROP_NONE, DROP_PHILOX, DROP_TENSOR = 0, 1, 2
 
 EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fmha_philox_keep_mask",
@@ -22,7 +21,7 @@ EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fm
            "fmha_fwd_workspace_bytes", "fmha_fwd_fp8_workspace_bytes", "fmha_pipe_probe")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
 _ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT", "FMHA_FWD_DECODE", "FMHA_FWD_HEAD",
-              "FMHA_BWD_PAIR", "FMHA_BWD_SHORT", "FMHA_BWD_FUSED")
+              "FMHA_BWD_PAIR", "FMHA_BWD_SHORT")
 _env_seen = None
 
 
@@ -314,9 +313,9 @@ def bwd(dout, q, k, v, o, lse, mask=None, mask_kind=MASK_ADDITIVE, mask_neg=-100
     """Launch the backward on the current stream.  Returns (dq, dk, dv).  kv_len and the tensor
     layouts as in fwd(); each gradient comes back in its input's dimension order.
 
-    workspace: True allocates the scratch that fmha_bwd_workspace_bytes() asks for (if any), a uint8
+    workspace: True allocates the scratch that fmha_bwd_workspace_bytes() asks for (none: no backward kernel uses one), a uint8
     device tensor is passed on as it is, None / False passes none (the two-kernel path beyond 256 keys).
-    noalloc: call fmha_bwd_launch_noalloc (delta and workspace out of the library's own scratch memory)."""
+    noalloc: call fmha_bwd_launch_noalloc (delta out of the library's own scratch memory)."""
     import torch
     bh, sq, d, heads, qs = _rows(q, "q")
     _, sk, _, hk, ks = _rows(k, "k")

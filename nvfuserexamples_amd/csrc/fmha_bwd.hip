@@ -7,7 +7,6 @@
 #if FMHA_TU_D == 64
 #define FMHA_TU_SHORT 1
 #include "fmha_bwd_short.h"
-#include "fmha_bwd_fused.h"
 #else
 #define FMHA_TU_SHORT 0
 #endif
@@ -104,21 +103,6 @@ template <int DROP, int SMAX, bool CAUSAL> int launch_short(BwdArgs &a, hipStrea
 }
 #endif
 
-#if FMHA_TU_SHORT
-// up to 512 keys: one workgroup per head computes dQ, dK and dV from one evaluation of the scores
-template <int MASK, int DROP> int launch_fused(BwdArgs &a, hipStream_t s) {
-  static_assert(BwdFusedCfg::MAX_KEYS == kBwdFusedMaxKeys && BwdFusedCfg::BQ == kBwdFusedTileRows &&
-                    BwdFusedCfg::WS_TILE_BYTES == kBwdFusedTileWsBytes,
-                "the C ABI sizes the workspace with these");
-  auto kern = fmha_bwd_fused_kernel<FMHA_TU_T, MASK, DROP, kStrided>;
-  constexpr int kLds = BwdFusedCfg::LDS_BYTES;
-  static const int attr = set_lds(kern, kLds);
-  if (attr) return 2;
-  hipLaunchKernelGGL(kern, dim3((unsigned)a.bh), dim3(BwdFusedCfg::NT), kLds, s, a);
-  return hipGetLastError() == hipSuccess ? 0 : 2;
-}
-#endif
-
 template <int MASK, bool CAUSAL> int by_drop(BwdArgs &a, const BwdVariant &v, hipStream_t s) {
   if (v.drop == 0) return launch<MASK, CAUSAL, 0>(a, v.pair, s);
   if (v.drop == 1) return launch<MASK, CAUSAL, 1>(a, v.pair, s);
@@ -138,13 +122,8 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(BwdArgs &a, const BwdVariant &v, hipStre
     if (small) return v.drop == 1 ? launch_short<1, 128, false>(a, s) : launch_short<0, 128, false>(a, s);
     return v.drop == 1 ? launch_short<1, 256, false>(a, s) : launch_short<0, 256, false>(a, s);
   }
-  if (v.fused) {
-    if (v.causal || v.mask == kMaskFull || a.sk > BwdFusedCfg::MAX_KEYS) return 1;
-    if (v.mask == kMaskPerKey) return v.drop == 1 ? launch_fused<kMaskPerKey, 1>(a, s) : launch_fused<kMaskPerKey, 0>(a, s);
-    return v.drop == 1 ? launch_fused<kMaskNone, 1>(a, s) : launch_fused<kMaskNone, 0>(a, s);
-  }
 #else
-  if (v.short_seq || v.fused) return 1;
+  if (v.short_seq) return 1;
 #endif
   if (v.mask == kMaskPerKey)
     return v.causal ? by_drop<kMaskPerKey, true>(a, v, s) : by_drop<kMaskPerKey, false>(a, v, s);

@@ -53,7 +53,7 @@ struct BwdArgs {
   const int32_t *kv_len; // optional valid key count per group of kv_div heads
   int32_t kv_div;
   RowMap mq, mk, mv, mo, mdo, mdq, mdk, mdv; // row layouts (mk.ss == mv.ss)
-  float *ws; // one-pass kernel only: fp32 partial dQ sums between key chunks
+  float *ws; // the caller's workspace pointer: no kernel of a release build reads it (development builds: cycle stamps)
   int32_t dcols; // elements per row that exist (<= the kernel's head dim; run-time layouts only)
 };
 

@@ -54,10 +54,11 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
 // that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call), FMHA_FWD_SPLIT=0 never cuts a
 // forward's key range into pieces, FMHA_FWD_SPLIT=n (2..64) cuts it into about n wherever pieces are possible,
-// FMHA_FWD_DECODE=0 keeps forwards of one to four query rows on the matrix-pipe kernels.
+// FMHA_FWD_DECODE=0 keeps forwards of one to four query rows on the matrix-pipe kernels, FMHA_FWD_HEAD=0|1 keeps
+// forwards off / puts them on the whole-head kernel wherever it applies.
 // The environment is read once per process (on the first launch); fmha_reload_overrides() reads it again.
 struct Overrides {
-  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, fwd_decode, fwd_head, bwd_pair, bwd_short, bwd_fused;
+  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, fwd_decode, fwd_head, bwd_pair, bwd_short;
 };
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
@@ -75,7 +76,6 @@ Overrides read_overrides() {
   o.fwd_head = env_int("FMHA_FWD_HEAD", -1);
   o.bwd_pair = env_int("FMHA_BWD_PAIR", -1);
   o.bwd_short = env_int("FMHA_BWD_SHORT", 1);
-  o.bwd_fused = env_int("FMHA_BWD_FUSED", 0);
   return o;
 }
 Overrides &overrides() {
@@ -613,16 +613,12 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   return rc == 0 ? FMHA_OK : (rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH);
 }
 
-uint64_t fmha_bwd_workspace_bytes(int32_t bh, int32_t sq, int32_t sk, int32_t d) {
-  if (bh <= 0 || sq <= 0 || sk <= kBwdFusedMaxKeys / 2 || sk > kBwdFusedMaxKeys || d != 64) return 0;
-  return (uint64_t)bwd_fused_workspace_need(bh, sq);
-}
+uint64_t fmha_bwd_workspace_bytes(int32_t, int32_t, int32_t, int32_t) { return 0; } // no backward kernel uses one
 
 } // extern "C"
 
-// The library's own scratch memory, for fmha_bwd_launch_noalloc: delta (bh*sq floats) first, what is left
-// serves as the one-pass kernel's workspace where that fits.  Every GPU holds its own copy of the array; its
-// device address is looked up once per device (the array's name is only a host-side handle).
+// The library's own scratch memory, for fmha_bwd_launch_noalloc: delta (bh*sq floats).  Every GPU holds its own
+// copy of the array; its device address is looked up once per device (the array's name is only a host-side handle).
 namespace {
 constexpr size_t kScratchBytes = 8u << 20;
 } // namespace
@@ -762,19 +758,14 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   std::memset(&local, 0, sizeof local);
   std::memcpy(&local, caller, caller->struct_bytes < sizeof local ? (size_t)caller->struct_bytes : sizeof local);
   if (own_scratch) {
-    // delta and the workspace come out of the library's array; what the caller put there is not looked at
+    // delta comes out of the library's array; what the caller put there is not looked at
     local.delta = nullptr;
-    local.workspace = nullptr;
-    local.workspace_bytes = 0;
     if (local.bh <= 0 || local.sq <= 0) return FMHA_E_SHAPE;
     const uint64_t rows = (uint64_t)local.bh * (uint64_t)local.sq;
     if (rows * sizeof(float) > kScratchBytes) return FMHA_E_SCRATCH;
     unsigned char *base = (unsigned char *)scratch_on_current_device();
     if (!base) return FMHA_E_LAUNCH;
     local.delta = (float *)base;
-    const size_t used = (size_t)((rows * sizeof(float) + 255u) & ~(uint64_t)255u);
-    local.workspace = base + used;
-    local.workspace_bytes = kScratchBytes - used;
   }
   const fmha_bwd_params *p = &local;
   if (!p->q || !p->k || !p->v || !p->o || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk || !p->dv)
@@ -856,18 +847,7 @@ int bwd_launch_impl(const fmha_bwd_params *caller, void *hip_stream, bool own_sc
   if (short_rows == 1) short_rows = 256;
   v.short_seq = p->d == 64 && p->sq <= short_rows && p->sk <= short_rows && p->sq <= 256 && p->sk <= 256 &&
                 v.mask != kMaskFull;
-  // The one-pass kernel (one workgroup per head of up to 512 keys, no causal mask, no full mask tensor; beyond 256
-  // keys it needs the caller's workspace) runs only where the caller asks for it: it measures level with the
-  // two-kernel path at best.
-  a.ws = (float *)p->workspace;
-  {
-    const bool asked = (p->flags & FMHA_FLAG_BWD_ONE_PASS) != 0 || overrides().bwd_fused == 1;
-    const bool can = p->d == 64 && !v.short_seq && !v.causal && v.mask != kMaskFull && p->sk <= kBwdFusedMaxKeys &&
-                     (p->sk <= kBwdFusedMaxKeys / 2 ||
-                      (p->workspace && ((uintptr_t)p->workspace & 15u) == 0 &&
-                       p->workspace_bytes >= bwd_fused_workspace_need(p->bh, p->sq)));
-    v.fused = asked && can;
-  }
+  a.ws = (float *)p->workspace; // no kernel of a release build reads it (development builds: cycle stamps)
   hipStream_t s = (hipStream_t)hip_stream;
   int rc;
   if (strided) {

@@ -42,15 +42,7 @@ struct BwdVariant {
   int drop; // 0 none, 1 Philox
   int pair; // causal tile pairing: -1 decide from the amount of work, 0 off, 1 on
   bool short_seq; // sq, sk <= 256 without a full mask tensor: the one-launch kernel (head dim 64)
-  bool fused;     // up to 512 keys, no causal mask, no full mask tensor: the one-pass kernel (head dim 64)
 };
-
-// Bytes of caller-provided workspace the one-pass backward needs for these sizes (fp32 partial dQ
-// sums of heads with more than 256 live keys).
-constexpr int kBwdFusedMaxKeys = 512, kBwdFusedTileRows = 64, kBwdFusedTileWsBytes = 16384;
-inline size_t bwd_fused_workspace_need(int bh, int sq) {
-  return (size_t)bh * (size_t)((sq + kBwdFusedTileRows - 1) / kBwdFusedTileRows) * kBwdFusedTileWsBytes;
-}
 
 int bwd_dispatch_f16_d64(BwdArgs &a, const BwdVariant &v, hipStream_t s);
 int bwd_dispatch_f16_d128(BwdArgs &a, const BwdVariant &v, hipStream_t s);

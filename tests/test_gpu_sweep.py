@@ -42,7 +42,8 @@ def _case(it, rng, forced=None):
         sk=rng.choice([1, 5, 8, 31, 32, 33, 40, 64, 65, 96, 127, 128, 129, 192, 200, 250, 256, 257, 300, 333, 512, 700]),
         causal=rng.random() < 0.3, p=rng.choice([0.0, 0.0, 0.1, 0.3]),
         mask=rng.choice(["none", "pad", "pad", "pad", "full", "keyinf", "padinf", "padholes"]),
-        want_len=rng.random() < 0.3, want_strided=rng.random() < 0.25, one_pass=rng.random() < 0.3)
+        want_len=rng.random() < 0.3, want_strided=rng.random() < 0.25,
+        spare=rng.random())  # (a draw an earlier option used: kept so that the sequence of cases stays the same)
     c.setdefault("lens", None)
     c["use_len"] = c["mask"] == "none" and c.get("want_len", False)
     c["strided"] = c.get("want_strided", False) and c["mask"] != "full"
@@ -89,7 +90,7 @@ def _run_case(it, c, rng):
             return x.view(b, h, x.shape[1], d).permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
         qc, kc, vc, dc = f(qc), f(kc), f(vc), f(dc)
     mc = None if m is None else m.cuda()
-    bflags = capi.FLAG_BWD_ONE_PASS if c.get("one_pass") else 0
+    bflags = 0
     o, lse, _, _ = capi.fwd(qc, kc, vc, mask=mc, want_lse=True, **kw)
     dq, dk, dv = capi.bwd(dc, qc, kc, vc, o, lse, mask=mc, flags=bflags, **kw)
     torch.cuda.synchronize()
@@ -154,7 +155,7 @@ ZERO_GRADIENT = [
     dict(d=128, dtype="fp16", b=1, h=4, sq=257, sk=8, causal=False, p=0.1, mask="padinf", lens=[1], want_strided=True),
     dict(d=64, dtype="fp16", b=2, h=2, sq=300, sk=1, causal=False, p=0.3, mask="full"),
     dict(d=64, dtype="fp16", b=1, h=1, sq=1, sk=200, causal=True, p=0.1, mask="none"),
-    dict(d=64, dtype="bf16", b=2, h=2, sq=300, sk=300, causal=False, p=0.1, mask="pad", lens=[1, 1], one_pass=True),
+    dict(d=64, dtype="bf16", b=2, h=2, sq=300, sk=300, causal=False, p=0.1, mask="pad", lens=[1, 1]),
 ]
 
 
