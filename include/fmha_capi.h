@@ -278,7 +278,9 @@ int fmha_bwd_launch(const fmha_bwd_params *p, void *hip_stream);
  * (FMHA_E_SCRATCH).  The call allocates nothing and synchronises nothing.  All calls on one GPU share
  * that GPU's array: calls that may overlap there (different streams or threads) race on it; serialise
  * them or use fmha_bwd_launch with buffers of the caller's own.  Results are bit-identical to
- * fmha_bwd_launch's.
+ * fmha_bwd_launch's.  Under stream capture: the FIRST call on a device (it looks up the array's address) and the
+ * first launch of each kernel variant in the process (it sets the kernel's LDS size) are not stream operations
+ * and must have happened before the capture begins -- make one eager call with the same shape class first.
  */
 int fmha_bwd_launch_noalloc(const fmha_bwd_params *p, void *hip_stream);
 uint64_t fmha_bwd_noalloc_max_rows(void);

@@ -336,6 +336,7 @@ static int fwd_dispatch_strided(FwdArgs &a, const FwdVariant &v, int dtype, int 
 // The merge of `pieces` partial results (fp32 from the decode kernel, element type otherwise) into o and lse.
 template <bool F32> static int merge_launch(int dtype, void *o, float *lse, int bh, int sq, int d, const void *o_part,
                                             const float *lse_part, const RowMap &mo, int pieces, hipStream_t s) {
+  if ((long long)bh * sq > 0x7fffffffLL) return 2; // one workgroup per output row
   const dim3 grid((unsigned)((long long)bh * sq)), block(kMergeThreads);
   if (dtype == FMHA_DTYPE_F16) {
     using TP = std::conditional_t<F32, float, _Float16>;
@@ -392,9 +393,11 @@ static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const Sp
   float *lse_part = (float *)(ws + pl.off_lse);
   uint16_t *mask_part = a.mask ? (uint16_t *)(ws + pl.off_mask) : nullptr;
   const long long vh = (long long)p->bh * pl.pieces;
+  if (vh > 0x7fffffffLL) return FMHA_E_SHAPE; // the kernels see bh * pieces heads
   if (a.mask) {
     const long long threads = vh * (pl.chunk / 8);
     const int nt = 256;
+    if ((threads + nt - 1) / nt > 0x7fffffffLL) return FMHA_E_SHAPE;
     hipLaunchKernelGGL(split_mask_kernel, dim3((unsigned)((threads + nt - 1) / nt)), dim3(nt), 0, s, mask_part,
                        (const uint16_t *)a.mask, a.mask_sb, a.mask_div, p->bh, p->sk, pl.pieces, pl.chunk);
     if (hipGetLastError() != hipSuccess) return FMHA_E_LAUNCH;

@@ -273,7 +273,10 @@ __global__ __launch_bounds__(Fp8Cfg<D>::NT) void fmha_fwd_fp8_kernel(const Fp8Ar
     // from a saturated conversion must take this path although the build tells the compiler that NaNs do not
     // occur).  The scores are recomputed from the operands (the fast path has
     // overwritten them), the reference becomes ceil(max), everything is rescaled by the exact power of two.
-    if (__builtin_amdgcn_ballot_w64(!seen || __float_as_uint(tsum) > __float_as_uint(SUM_LIMIT))) {
+    // Only the rows that need it change their reference (and take the recomputed probabilities): a row's result
+    // depends on that row alone, whatever rows share its wave.
+    const bool need = !seen || __float_as_uint(tsum) > __float_as_uint(SUM_LIMIT);
+    if (__builtin_amdgcn_ballot_w64(need)) {
       f32x16 y[2];
       float mx = NEG_INF;
 #pragma unroll
@@ -300,21 +303,25 @@ __global__ __launch_bounds__(Fp8Cfg<D>::NT) void fmha_fwd_fp8_kernel(const Fp8Ar
       mx = xhalf_max(mx);
       const bool live = mx > -1e20f; // this tile shows the row a key that is not masked out
       float Mn = M;
-      if (live) Mn = seen ? fmaxf(M, __builtin_ceilf(mx)) : __builtin_ceilf(mx);
-      const float alpha = seen ? fast_exp2(M - Mn) : 1.f; // (nothing has been accumulated before the first live tile)
-      psum = 0.f;
+      if (need && live) Mn = seen ? fmaxf(M, __builtin_ceilf(mx)) : __builtin_ceilf(mx);
+      const float alpha = seen ? fast_exp2(M - Mn) : 1.f; // (nothing has been accumulated before the first live tile; 1 where the reference stays)
+      float psum_new = 0.f;
 #pragma unroll
       for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float p = live ? fast_exp2(y[sb][r] - Mn) : 0.f;
           y[sb][r] = p;
-          psum += p;
+          psum_new += p;
         }
+      psum = need ? psum_new : psum;
 #pragma unroll
       for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) pb[sb * 4 + g] = pack4_e4m3(y[sb][4 * g], y[sb][4 * g + 1], y[sb][4 * g + 2], y[sb][4 * g + 3]);
+        for (int g = 0; g < 4; ++g) {
+          const int pn = pack4_e4m3(y[sb][4 * g], y[sb][4 * g + 1], y[sb][4 * g + 2], y[sb][4 * g + 3]);
+          pb[sb * 4 + g] = need ? pn : pb[sb * 4 + g]; // (both half-waves of a row decide alike: the sums they test are the row's)
+        }
       tsum = mfma_fp8_k64(ones, pb, zero)[0];
       l_run *= alpha;
       l_true *= alpha;
@@ -323,7 +330,7 @@ __global__ __launch_bounds__(Fp8Cfg<D>::NT) void fmha_fwd_fp8_kernel(const Fp8Ar
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
       M = Mn;
-      seen = seen || live;
+      seen = seen || (need && live);
       set_bx();
     }
     l_run += tsum;

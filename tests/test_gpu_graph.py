@@ -106,3 +106,53 @@ def test_decode_step_in_pieces_replays_from_a_graph():
         torch.cuda.synchronize()
         for a, b_ in zip(got, want):
             assert torch.equal(a, b_), r
+
+
+def test_noalloc_backward_replays_from_a_graph():
+    """fmha_bwd_launch_noalloc is meant for callers under capture.  Its first call on a device looks up the
+    address of the library's scratch array and sets kernel attributes, neither of which is a stream operation:
+    that call happens eagerly (the warm-up inside _capture), then the launch is captured and replayed twice on
+    new values, bit for bit equal to fmha_bwd_launch with a delta buffer of the caller's."""
+    import ctypes as C
+    from nvfuserexamples_amd import capi
+    L = capi.lib()
+    bh, s, d = 8, 320, 64
+    q, k, v, do = (t.cuda() for t in make_qkv(bh, s, s, d, seed=2, with_dout=True))
+    m = pad_mask(bh // 2, s, s // 2, s).half().cuda()
+    o = torch.empty_like(q)
+    lse = torch.empty(bh, s, dtype=torch.float32, device="cuda")
+    got = [torch.empty_like(q) for _ in range(3)]
+    ref = [torch.empty_like(q) for _ in range(3)]
+    delta = torch.empty(bh, s, dtype=torch.float32, device="cuda")
+
+    def params(grads, dl):
+        P = capi.BwdParams()
+        P.q, P.k, P.v, P.o, P.dout, P.lse = (t.data_ptr() for t in (q, k, v, o, do, lse))
+        P.delta = dl.data_ptr() if dl is not None else None
+        P.dq, P.dk, P.dv = (t.data_ptr() for t in grads)
+        P.bh, P.sq, P.sk, P.d, P.dtype, P.scale = bh, s, s, d, capi.F16, d ** -0.5
+        P.mask, P.mask_kind = m.data_ptr(), capi.MASK_ADDITIVE
+        P.mask_bh_div, P.mask_stride_b, P.mask_stride_q = 2, s, 0
+        P.drop_kind, P.p_drop, P.drop_scale, P.seed, P.offset = capi.DROP_PHILOX, 0.1, 0.0, 5, 7
+        return P
+    Pn, Pr = params(got, None), params(ref, delta)
+
+    def forward():
+        lse.copy_(capi.fwd(q, k, v, mask=m, want_lse=True, out=o, drop_kind=capi.DROP_PHILOX, p_drop=0.1, seed=5, offset=7)[1])
+
+    def step():
+        capi.check(L.fmha_bwd_launch_noalloc(C.byref(Pn), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+    forward()
+    g, _ = _capture(step)
+    for r in range(2):
+        for dst, src in zip((q, k, v, do), make_qkv(bh, s, s, d, seed=20 + r, with_dout=True)):
+            dst.copy_(src.cuda())
+        forward()
+        for t in got:
+            t.fill_(float("nan"))
+        g.replay()
+        capi.check(L.fmha_bwd_launch(C.byref(Pr), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        for a, b_ in zip(got, ref):
+            assert torch.equal(a, b_), r
