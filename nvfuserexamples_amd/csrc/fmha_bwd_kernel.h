@@ -794,8 +794,8 @@ __global__ __launch_bounds__(NW * 64)
       const int key = k0w + kb * 32 + kl;
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb) {
-        uint32_t wd[4][4];
-        if (DROP == 1) drop_words_k(a.drop, (uint32_t)bh, (uint32_t)(q0 + sb * 32), (uint32_t)key, h, l, wd);
+        uint32_t rb[4]; // rb[t], byte gq: the random byte of (query 8 gq + 4h + t of the block, this lane's key)
+        if (DROP == 1) drop_bytes_k(a.drop, (uint32_t)bh, (uint32_t)(q0 + sb * 32), (uint32_t)key, h, l, rb);
         float pz[16], ds[16];
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
@@ -811,7 +811,7 @@ __global__ __launch_bounds__(NW * 64)
             float gv = g[kb][sb][4 * gq + t];
             float pzv = p;
             if (DROP == 1) {
-              const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
+              const bool keep = drop_keep_byte(rb[t], gq, a.drop.thr);
               gv = keep ? gv : -Dl[t];
               pzv = keep ? p : 0.f; // (drop_scale multiplies dV once, on store)
               // keep the selection in fp32: left alone the compiler converts first and selects halves, which costs

@@ -213,8 +213,8 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
           x = E::mfma(panel_read_rows<T, BT>(tQ, pl, qb & 1, ks), kreg[ks], x);
           g = E::mfma(panel_read_rows<T, BT>(tDO, pl, qb & 1, ks), vreg[ks], g);
         }
-        uint32_t wd[4][4];
-        if (DROP == 1) drop_words_k(a.drop, (uint32_t)bh, (uint32_t)(qb * 32), (uint32_t)key, h, l, wd);
+        uint32_t rb[4]; // rb[t], byte gq: the random byte of (query 8 gq + 4h + t of the block, this lane's key)
+        if (DROP == 1) drop_bytes_k(a.drop, (uint32_t)bh, (uint32_t)(qb * 32), (uint32_t)key, h, l, rb);
         v8 pfrag[2], dsfrag[2];
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
@@ -228,7 +228,7 @@ void fmha_bwd_short_kernel(const BwdArgs a) {
             float gv = g[4 * gq + t] - Dl[t];
             float pz = p;
             if (DROP == 1) {
-              const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
+              const bool keep = drop_keep_byte(rb[t], gq, a.drop.thr);
               gv = keep ? fmaf(g[4 * gq + t], a.drop_scale, -Dl[t]) : -Dl[t];
               pz = keep ? p : 0.f; // (drop_scale multiplies dV once, on store)
             }

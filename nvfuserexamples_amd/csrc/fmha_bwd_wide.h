@@ -275,8 +275,8 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
         const bool diag = CAUSAL && (k0w + 31 > q0);
 #pragma unroll
         for (int sb = 0; sb < NSB; ++sb) {
-          uint32_t wd[4][4];
-          if (DROP == 1) drop_words_k(a.drop, (uint32_t)bh, (uint32_t)(q0 + sb * 32), (uint32_t)key, h, l, wd);
+          uint32_t rb[4]; // rb[t], byte gq: the random byte of (query 8 gq + 4h + t of the block, this lane's key)
+          if (DROP == 1) drop_bytes_k(a.drop, (uint32_t)bh, (uint32_t)(q0 + sb * 32), (uint32_t)key, h, l, rb);
           v8 send[2];
 #pragma unroll
           for (int gq = 0; gq < 4; ++gq)
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(bwd_wide_threads<D>()) __attribute__((amdgpu_waves_
               const float p = fast_exp2(xv);
               const int r = 4 * gq + t;
               if (DROP == 1) {
-                const bool keep = drop_keep_byte(wd[gq][t], key & 3, a.drop.thr);
+                const bool keep = drop_keep_byte(rb[t], gq, a.drop.thr);
                 frag[sb][r >> 3][r & 7] = (T)(keep ? p : 0.f); // (drop_scale multiplies dV once, on store)
                 send[r >> 3][r & 7] = (T)(keep ? p : -p);
               } else {

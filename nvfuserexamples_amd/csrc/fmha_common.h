@@ -469,21 +469,25 @@ FMHA_DEV void drop_words_q(const DropCtx &c, uint32_t bh, uint32_t q, uint32_t k
   quad_transpose4(w, lane);                                        // w[g] = word of row q in block g
 }
 
-// Lane = key layout.  The lane owns key k and, in one 32-query block starting at qb32, the
-// queries 4h + 8g + t.  Returns in w[g][t] the word of query row (qb32 + 4h + 8g + t) in the
-// block containing key k (the lane's byte is k % 4).  Lanes of a quad share k/4: lane i
-// evaluates the block of g = i and broadcasts its four words.
-FMHA_DEV void drop_words_k(const DropCtx &c, uint32_t bh, uint32_t qb32, uint32_t k, int h, int lane,
-                           uint32_t w[4][4]) {
+// Lane = key layout.  The lane owns key k and, in one 32-query block starting at qb32, the queries 4h + 8g + t
+// (g, t = 0..3).  Lanes of a quad share k / 4: lane i evaluates the block of g = i.  Of every word (row t of block
+// g) a lane uses one byte only, byte k % 4 = lane % 4, so for each t the quad transposes a 4 x 4 matrix of BYTES
+// (row = the lane that evaluated block g, column = the byte) instead of broadcasting whole words.  Returns r[t]
+// whose byte g is the random byte of (query qb32 + 4h + 8g + t, key k): a compare with a static byte selector per
+// element, no extraction.  Two butterfly stages per word, each a quad-permuted move and a v_perm_b32 with a
+// selector that depends on the lane's position in the quad only (16 instructions per block; broadcasting the
+// sixteen words and extracting the lane's byte of each took 32).
+FMHA_DEV void drop_bytes_k(const DropCtx &c, uint32_t bh, uint32_t qb32, uint32_t k, int h, int lane, uint32_t r[4]) {
   const uint32_t g = (uint32_t)lane & 3u;
   uint32_t o[4];
   drop_block(c, bh, (qb32 >> 2) + (uint32_t)h + 2u * g, k >> 2, o);
+  // v_perm_b32(hi, lo, sel): selector values 0-3 take bytes of lo (own), 4-7 bytes of hi (partner)
+  const uint32_t sel1 = (lane & 1) ? 0x03070105u : 0x06020400u; // with lane ^ 1: (own0, partner0, own2, partner2) / (partner1, own1, partner3, own3)
+  const uint32_t sel2 = (lane & 2) ? 0x03020706u : 0x05040100u; // with lane ^ 2: (own0, own1, partner0, partner1) / (partner2, partner3, own2, own3)
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    w[0][t] = quad_perm<0x00>(o[t]);
-    w[1][t] = quad_perm<0x55>(o[t]);
-    w[2][t] = quad_perm<0xAA>(o[t]);
-    w[3][t] = quad_perm<0xFF>(o[t]);
+    const uint32_t a1 = __builtin_amdgcn_perm(quad_perm<0xB1>(o[t]), o[t], sel1);
+    r[t] = __builtin_amdgcn_perm(quad_perm<0x4E>(a1), a1, sel2);
   }
 }
 
