@@ -418,10 +418,12 @@ def config_leg(torch, capi, L, stream, steps, warmup, b, h, s, d, dtype, causal,
     capi.check(L.fmha_bwd_launch(C.byref(sets[0][2]), stream))
 
     def fwd(i):
-        L.fmha_fwd_launch(C.byref(sets[i % nsets][1]), stream)
+        if L.fmha_fwd_launch(C.byref(sets[i % nsets][1]), stream):
+            raise RuntimeError("forward launch refused inside a timed region")
 
     def bwd(i):
-        L.fmha_bwd_launch(C.byref(sets[i % nsets][2]), stream)
+        if L.fmha_bwd_launch(C.byref(sets[i % nsets][2]), stream):
+            raise RuntimeError("backward launch refused inside a timed region")
 
     def both(i):
         fwd(i)
@@ -887,10 +889,12 @@ def main():
     capi.check(L.fmha_fwd_launch(C.byref(fps_dense[0]), stream))
 
     def fwd_step(i):
-        L.fmha_fwd_launch(C.byref(fps[i % len(fps)]), stream)
+        if L.fmha_fwd_launch(C.byref(fps[i % len(fps)]), stream):
+            raise RuntimeError("forward launch refused inside a timed region")
 
     def fwd_dense(i):
-        L.fmha_fwd_launch(C.byref(fps_dense[i % len(fps_dense)]), stream)
+        if L.fmha_fwd_launch(C.byref(fps_dense[i % len(fps_dense)]), stream):
+            raise RuntimeError("forward launch refused inside a timed region")
 
     spread = {}
     ms, wall_ms = time_steps(torch, fwd_dense, args.steps, args.warmup, stats=spread)
@@ -1062,11 +1066,12 @@ def main():
                 L.fmha_fwd_launch(C.byref(F), stream)   # O and LSE of every set, for the backward timed alone
 
             def train_step(i):
-                L.fmha_fwd_launch(C.byref(tf[i % len(tf)]), stream)
-                L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream)
+                if L.fmha_fwd_launch(C.byref(tf[i % len(tf)]), stream) or L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream):
+                    raise RuntimeError("train-step launch refused inside a timed region")
 
             def bwd_step(i):
-                L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream)
+                if L.fmha_bwd_launch(C.byref(tb[i % len(tb)]), stream):
+                    raise RuntimeError("backward launch refused inside a timed region")
 
             def fwd_t(i):
                 L.fmha_fwd_launch(C.byref(tf[i % len(tf)]), stream)
