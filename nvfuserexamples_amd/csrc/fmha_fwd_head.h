@@ -524,9 +524,22 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
   // walks on into it as soon as its own Q rows are there.  Otherwise (first item of a workgroup, or a very short
   // predecessor) the item starts cold: barrier, first tiles, barrier, and its rows arrive while it computes -- its
   // hook 3 waits only for those that iterations 3-6 read (tiles 4-7 of K, 2-5 of V).
+  // Q' = Q * scale * log2(e), rounded once, as B-operand registers.  The conversion must happen where this is called:
+  // left alone the compiler sinks it towards the first use of Q' -- below copies issued in between, and its wait for
+  // the raw rows, counted without those copies, then waits for all of them.
+  auto convertQ = [&]() {
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const v8 raw = as_v8<T>(qraw[qb][ks]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
+        asm volatile("" : "+v"(qreg[qb][ks]));
+      }
+  };
   int pf = 0;        // pairs of the current item's K and V that its predecessor requested
   bool xready = false; // ... and whether it wrote the item's extra-step rows
-  int nst = 0;       // output stores of the previous item that this wave may still have in flight
   int xb = 0;        // the extra-row buffer of the current item
   T xm = (T)0.f;     // a mask value on its way from memory to an extra-step row
   Item cur = make_item(blockIdx.x);
@@ -556,28 +569,14 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
       __builtin_amdgcn_sched_barrier(0);
       vm_wait<QB * KS>();       // this wave's part of the first tiles is in LDS
       lds_barrier();            // ... and everybody's, and the extra rows
-    } else {
-      // Requested before the previous item's output stores: wait for everything but those stores.
-      switch (__builtin_amdgcn_readfirstlane(nst)) {
-      case 10: vm_wait<10>(); break;
-      case 8: vm_wait<8>(); break;
-      case 5: vm_wait<5>(); break;
-      case 4: vm_wait<4>(); break;
-      default: vm_wait<0>(); break;
-      }
     }
+    // (A warm item has nothing to wait for: its Q rows were converted at the end of the previous item, before that
+    // item's output stores went out -- a wait for them here would also wait for those stores -- and its first tiles
+    // were confirmed by the previous item's hooks.)
     __builtin_amdgcn_sched_barrier(0);
     const Item nxt = make_item(more ? nidx : idx);
-    FMHA_TL(); // 1: requests out and first tiles in (cold) / waited (warm)
-    // Q' = Q * scale * log2(e), rounded once, as B-operand registers
-#pragma unroll
-    for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const v8 raw = as_v8<T>(qraw[qb][ks]);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) qreg[qb][ks][j] = (T)((float)raw[j] * a.scale_l2);
-      }
+    FMHA_TL(); // 1: requests out and first tiles in (cold)
+    if (cold) convertQ();
     if (cold) {
       __builtin_amdgcn_sched_barrier(0);
       // (the Q rows have been consumed: nothing of this wave's is in flight)  The rest of the item's rows in the
@@ -718,21 +717,21 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
     }
 
     // ---- item epilogue
+    // The next item's Q rows (requested at the last hook) become Q' before this item's outputs are stored: the
+    // wait for them covers only older requests, and the next item starts without a wait.
+    if (more) convertQ();
     T *Ob = (T *)a.o + (size_t)bh * (size_t)a.sq * D;
-    int stores = 0;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const int q = q0w + qb * 32 + ql;
       const float lt = xhalf_sum(lsum[qb]);
       const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
-      if (q0w + qb * 32 < a.sq) stores += a.lse ? 5 : 4;
       if (q < a.sq) {
 #pragma unroll
         for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * D + db * 32, o[qb][db], inv, h);
         if (a.lse && h == 0) a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
       }
     }
-    nst = stores;
     FMHA_TL(); // stores issued
     if (!more) break;
     idx = nidx;
