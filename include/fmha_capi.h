@@ -309,7 +309,7 @@ float fmha_drop_scale(float p_drop);
 const char *fmha_strerror(int code);
 
 /* The FMHA_* environment variables -- tuning and test overrides of the variant selection: FMHA_MASK_TRIM,
- * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_FWD_HEAD, FMHA_BWD_SHORT, FMHA_BWD_PAIR
+ * FMHA_FWD_QB, FMHA_FWD_SHORT, FMHA_FWD_STREAM, FMHA_FWD_SAVE_ONCE, FMHA_FWD_SAVE_SPLIT, FMHA_FWD_SPLIT, FMHA_FWD_DECODE, FMHA_FWD_HEAD, FMHA_BWD_SHORT, FMHA_BWD_PAIR
  * -- are read once per process, on the first launch.  This reads them again; not to be
  * called while another thread is launching.  (No counterpart in the reference.) */
 void fmha_reload_overrides(void);

@@ -20,7 +20,7 @@ EXPORTS = ("fmha_fwd_launch", "fmha_bwd_launch", "fmha_bwd_workspace_bytes", "fm
            "fmha_bwd_launch_noalloc", "fmha_bwd_noalloc_max_rows", "fmha_drop_scale", "fmha_fwd_fp8_launch",
            "fmha_fwd_workspace_bytes", "fmha_fwd_fp8_workspace_bytes", "fmha_pipe_probe")
 # environment overrides the library reads once; the wrappers below make it read them again when they change
-_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT", "FMHA_FWD_DECODE", "FMHA_FWD_HEAD",
+_ENV_NAMES = ("FMHA_MASK_TRIM", "FMHA_FWD_SHORT", "FMHA_FWD_SAVE_SPLIT", "FMHA_FWD_SAVE_ONCE", "FMHA_FWD_STREAM", "FMHA_FWD_QB", "FMHA_FWD_SPLIT", "FMHA_FWD_DECODE", "FMHA_FWD_HEAD",
               "FMHA_BWD_PAIR", "FMHA_BWD_SHORT")
 _env_seen = None
 

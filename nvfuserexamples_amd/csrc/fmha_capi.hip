@@ -48,7 +48,9 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 }
 
 // Tuning overrides for experiments and tests: FMHA_FWD_QB=1|2 forces the query blocks per wave of
-// the forward, FMHA_FWD_STREAM=0 keeps full-mask forwards on the pipelined kernel,
+// the forward, FMHA_FWD_STREAM=0 keeps full-mask forwards on the pipelined kernel, FMHA_FWD_SAVE_ONCE=0 /
+// FMHA_FWD_SAVE_SPLIT=0 keep the save-intermediates operator beyond 128 keys off its one-launch kernel / off the
+// forward-then-save pair of launches,
 // FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
 // one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
 // pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
@@ -58,7 +60,7 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // forwards off / puts them on the whole-head kernel wherever it applies.
 // The environment is read once per process (on the first launch); fmha_reload_overrides() reads it again.
 struct Overrides {
-  int mask_trim, fwd_short, fwd_save_split, fwd_stream, fwd_qb, fwd_split, fwd_decode, fwd_head, bwd_pair, bwd_short;
+  int mask_trim, fwd_short, fwd_save_split, fwd_save_once, fwd_stream, fwd_qb, fwd_split, fwd_decode, fwd_head, bwd_pair, bwd_short;
 };
 int env_int(const char *name, int dflt) {
   const char *e = std::getenv(name);
@@ -69,6 +71,7 @@ Overrides read_overrides() {
   o.mask_trim = env_int("FMHA_MASK_TRIM", 1);
   o.fwd_short = env_int("FMHA_FWD_SHORT", 1);
   o.fwd_save_split = env_int("FMHA_FWD_SAVE_SPLIT", 1);
+  o.fwd_save_once = env_int("FMHA_FWD_SAVE_ONCE", 1);
   o.fwd_stream = env_int("FMHA_FWD_STREAM", 1);
   o.fwd_qb = env_int("FMHA_FWD_QB", 0);
   o.fwd_split = env_int("FMHA_FWD_SPLIT", -1);
@@ -430,7 +433,7 @@ static int fwd_split_launch(const fmha_fwd_params *p, const FwdArgs &a, const Sp
   v.mask = a.mask ? kMaskPerKey : kMaskNone;
   v.causal = false;
   v.drop = 0;
-  v.saving = v.save_split = v.stream = v.short_keys = v.head = false;
+  v.saving = v.save_split = v.save_once = v.stream = v.short_keys = v.head = false;
   const int rc = fwd_dispatch_strided(b, v, p->dtype, D, s);
   if (rc != 0) return rc == 1 ? FMHA_E_UNSUPPORTED : FMHA_E_LAUNCH;
   {
@@ -569,7 +572,15 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  v.mask == kMaskFull && !v.causal && a.drop_mask && aligned16(a.mask) && (a.mask_sb % 8) == 0 &&
                  (a.mask_sq % 8) == 0 && aligned16(a.drop_mask) && (!a.save_softmax || aligned16(a.save_softmax)) &&
                  (!a.save_dropout || aligned16(a.save_dropout)) && overrides().fwd_save_split != 0;
-  if (v.save_split) v.saving = false; // the forward launch itself saves nothing
+  // Up to 512 keys one launch does it all: a wave keeps its probabilities and dropout rows in registers until the
+  // row's log-sum-exp is known, so the mask and the dropout tensor are read once (no LSE buffer needed).
+  v.save_once = saving && !v.short_keys && !strided && p->d == 64 && p->sk <= 512 && (p->sk % 8) == 0 &&
+                v.mask == kMaskFull && !v.causal && !p->kv_len && a.drop_mask && aligned16(a.mask) &&
+                (a.mask_sb % 8) == 0 && (a.mask_sq % 8) == 0 && aligned16(a.drop_mask) &&
+                (!a.save_softmax || aligned16(a.save_softmax)) && (!a.save_dropout || aligned16(a.save_dropout)) &&
+                overrides().fwd_save_once != 0 && overrides().fwd_stream != 0; // (it is the streaming forward's arithmetic)
+  if (v.save_once) v.save_split = false;
+  if (v.save_split || v.save_once) v.saving = false; // (save_split: the forward launch itself saves nothing)
   // Other forwards under an aligned full mask tensor (with or without a dropout tensor) are memory time at
   // head dim 64: the streaming kernel.
   v.stream = !v.short_keys && !v.saving && !strided && p->d == 64 && (p->sk % 8) == 0 && v.mask == kMaskFull &&

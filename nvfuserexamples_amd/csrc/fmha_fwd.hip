@@ -10,6 +10,7 @@
 #include "fmha_fwd_short.h"
 #include "fmha_fwd_save.h"
 #include "fmha_fwd_stream.h"
+#include "fmha_fwd_stream_save.h"
 #include "fmha_fwd_head.h"
 #else
 #define FMHA_TU_SHORT 0
@@ -131,6 +132,19 @@ template <bool DROPT> int launch_stream(FwdArgs &a, hipStream_t s) {
 #endif
 
 #if FMHA_TU_SHORT
+// the save-intermediates operator for 129 to 512 keys in one launch (one wave per SIMD: the whole register file)
+int launch_stream_save(FwdArgs &a, hipStream_t s) {
+  auto kern = fmha_fwd_stream_save_kernel<FMHA_TU_T>;
+  if (a.sk > StreamSaveCfg::SKMAX) return 1;
+  a.nqt = (a.sq + StreamSaveCfg::QT - 1) / StreamSaveCfg::QT;
+  const long long nblk = (long long)a.bh * a.nqt;
+  if (nblk > 0x7fffffffLL) return 2;
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(StreamSaveCfg::NW * 64), StreamSaveCfg::LDS_BYTES, s, a);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+#endif
+
+#if FMHA_TU_SHORT
 // a whole head's K and V resident in LDS: one persistent workgroup per compute unit
 #ifndef FMHA_HEAD_QB
 #define FMHA_HEAD_QB 2
@@ -200,7 +214,7 @@ template <int MASK, bool CAUSAL> int plain_by_drop(FwdArgs &a, int drop, hipStre
 } // namespace
 
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
-  if (v.qb == 2 || v.short_keys || v.save_split || v.stream || v.head || (kStrided && v.drop == 2)) return 1;
+  if (v.qb == 2 || v.short_keys || v.save_split || v.save_once || v.stream || v.head || (kStrided && v.drop == 2)) return 1;
   if (v.mask == kMaskPerKey)
     return v.causal ? plain_by_drop<kMaskPerKey, true>(a, v.drop, s) : plain_by_drop<kMaskPerKey, false>(a, v.drop, s);
   if (v.mask == kMaskFull)
@@ -217,6 +231,7 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
     if (v.saving) return launch_short<true, true>(a, s);
     return v.drop == 2 ? launch_short<true, false>(a, s) : launch_short<false, false>(a, s);
   }
+  if (v.save_once) return launch_stream_save(a, s);
   if (v.save_split) { // forward with LSE, then the saved outputs from that LSE
     const int rc = v.stream ? launch_stream<true>(a, s) : launch<1, kMaskFull, false, 2, true>(a, s);
     return rc ? rc : launch_save(a, s);
@@ -228,7 +243,7 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
     return v.drop ? launch_head<kMaskNone, 1>(a, s) : launch_head<kMaskNone, 0>(a, s);
   }
 #else
-  if (v.short_keys || v.save_split || v.stream || v.head) return 1;
+  if (v.short_keys || v.save_split || v.save_once || v.stream || v.head) return 1;
 #endif
   if (v.drop == 2) { // tensor dropout / save-intermediates: the legacy ops' shape class
     if (v.causal) return 1;

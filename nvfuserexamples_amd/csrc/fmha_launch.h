@@ -17,6 +17,7 @@ struct FwdVariant {
   int drop;     // 0 none, 1 Philox, 2 tensor / save-intermediates
   bool saving;  // drop == 2: the save-intermediates pass is wanted (plain kernel only)
   bool save_split; // saving beyond the one-pass kernel's range with a caller-provided LSE buffer: forward, then a save kernel
+  bool save_once;  // saving for 129 to 512 keys: one launch that keeps a wave's probabilities in registers (head dim 64, folded layout)
   bool stream;     // full mask tensor on aligned rows beyond the one-pass range: the streaming forward (head dim 64, folded layout)
   bool head;       // up to 512 keys, no / per-key mask, no causal mask: the whole-head kernel (head dim 64, folded layout)
   bool short_keys; // sk <= 128 under an aligned full mask tensor: the one-pass kernel (head dim 64, folded layout)

@@ -227,9 +227,11 @@ def test_short_key_ranges_under_full_masks(bh, sq, sk, dtype, mode, short, monke
         assert torch.equal(o2, o)  # saving does not disturb O
 
 
-# Beyond 128 keys the saved outputs come from a streaming kernel that follows the forward launch and
-# derives them from its row log-sum-exp (FMHA_FWD_SAVE_SPLIT=0: from a second sweep inside a plain forward
-# kernel, which is also what serves rows that do not start on 16-byte boundaries and head dim 128).
+# Beyond 128 keys the saved outputs come, up to 512 keys, from one launch that keeps a wave's probabilities in
+# registers until the row's log-sum-exp is known; FMHA_FWD_SAVE_ONCE=0 (and any longer key range): from a streaming
+# kernel that follows the forward launch and derives them from its row log-sum-exp; FMHA_FWD_SAVE_SPLIT=0 as well:
+# from a second sweep inside a plain forward kernel, which is also what serves rows that do not start on 16-byte
+# boundaries and head dim 128.
 SAVE_LONG = [
     # bh, sq, sk, d, dtype
     (6, 200, 264, 64, "fp16"),     # ragged query tiles, a partly filled last key tile
@@ -241,9 +243,11 @@ SAVE_LONG = [
 ]
 
 
-@pytest.mark.parametrize("split", ["1", "0"])
+@pytest.mark.parametrize("route", ["once", "split", "plain"])
 @pytest.mark.parametrize("bh,sq,sk,d,dtype", SAVE_LONG)
-def test_saved_intermediates_beyond_128_keys(bh, sq, sk, d, dtype, split, monkeypatch):
+def test_saved_intermediates_beyond_128_keys(bh, sq, sk, d, dtype, route, monkeypatch):
+    split = "0" if route == "plain" else "1"
+    monkeypatch.setenv("FMHA_FWD_SAVE_ONCE", "1" if route == "once" else "0")
     monkeypatch.setenv("FMHA_FWD_SAVE_SPLIT", split)
     # without the split the saving forward is the plain kernel, whose O is bit-identical to the pipelined
     # kernel's, not to the streaming kernel's: keep the non-saving call on the same family
@@ -264,6 +268,41 @@ def test_saved_intermediates_beyond_128_keys(bh, sq, sk, d, dtype, split, monkey
     assert np.array_equal((f32(dr.cpu()) == 0)[live], (f32(dm) == 0)[live])
     o2, _, _, _ = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=2.0)
     assert torch.equal(o2, o)  # saving does not disturb O
+
+
+@pytest.mark.parametrize("route", ["once", "split"])
+def test_saved_intermediates_of_rows_that_meet_their_first_key_late_or_never(route, monkeypatch):
+    """The one-launch kernel rescales a tile's kept probabilities by exp2(m_t - L): rows that see no key at all
+    (L = -inf), rows whose first tiles are entirely -inf (m_t = -inf there), and rows whose early keys carry a
+    finite -10000 while later ones carry 0 (m_t far below L: the factor underflows to zero, as the true value does)."""
+    monkeypatch.setenv("FMHA_FWD_SAVE_ONCE", "1" if route == "once" else "0")
+    bh, sq, sk = 3, 160, 448
+    q, k, v = make_qkv(bh, sq, sk, 64, seed=77)
+    g = torch.Generator().manual_seed(78)
+    pm = torch.randn(bh, sq, sk, generator=g)
+    pm[:, 5, :] = float("-inf")                 # never a key
+    pm[:, 9, :200] = float("-inf")              # three whole tiles and part of the fourth before the first key
+    pm[:, 17, :320] = -10000.0                  # finite but hopeless early keys
+    pm[:, 33, 64:] = float("-inf")              # only the first tile counts
+    pm[1, :, 128:192] = float("-inf")           # a whole tile dead for every row of a head
+    pm = pm.half()
+    dm = torch.empty(bh, sq, sk).random_(2, generator=g).half()
+    o, lse, sm, dr = _run(q, k, v, mask=pm.cuda(), drop_kind=capi.DROP_TENSOR, drop_mask=dm.cuda(), drop_scale=1.25,
+                          save=True, want_lse=True)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(pm), drop_mask=f32(dm), drop_scale=1.25,
+                           want=("o", "lse", "softmax", "dropout"))
+    tol = TOL["fp16"]
+    got_sm, got_dr = f32(sm.cpu()), f32(dr.cpu())
+    assert np.isfinite(got_sm).all() and np.isfinite(got_dr).all() and np.isfinite(f32(o.cpu())).all()
+    assert np.abs(f32(o.cpu()) - ref["o"]).max() <= 2 * tol
+    assert np.abs(got_sm - ref["softmax"]).max() <= tol / 2
+    assert np.abs(got_dr - ref["dropout"]).max() <= tol
+    assert (got_sm[:, 5] == 0).all() and (got_dr[:, 5] == 0).all() and (f32(o.cpu())[:, 5] == 0).all()
+    assert (got_sm[:, 9, :200] == 0).all() and (got_sm[:, 17, :320] == 0).all() and (got_sm[1, :, 128:192] == 0).all()
+    gl = lse.cpu().numpy()
+    dead = np.isneginf(ref["lse"])
+    assert dead.any() and np.array_equal(np.isneginf(gl), dead)
+    assert np.abs(gl[~dead] - ref["lse"][~dead]).max() <= LSE_TOL["fp16"]
 
 
 @pytest.mark.parametrize("bh,sq,sk,d,dtype,mask", [
