@@ -146,13 +146,19 @@ void fmha_fwd_save_kernel(const FwdArgs a) {
       for (int g = 0; g < 4; ++g) {
         const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int kk = k0 + sb * 32 + 8 * g + 4 * h + i;
-          const float s = fmaf(x[sb][4 * g + i], a.scale_l2, fmaf((float)mv[i], a.mask_a, a.mask_b)) - lq;
-          x[sb][4 * g + i] = kk < a.sk ? fast_exp2(s) : 0.f;
-        }
+        for (int i = 0; i < 4; ++i)
+          x[sb][4 * g + i] = fast_exp2(fmaf(x[sb][4 * g + i], a.scale_l2, fmaf((float)mv[i], a.mask_a, a.mask_b)) - lq);
       }
     scr.turn();
+    if (k0 + BK > a.sk) { // only a partly filled last tile has keys to switch off (workgroup-uniform)
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kk = k0 + sb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+          x[sb][r] = kk < a.sk ? x[sb][r] : 0.f;
+        }
+    }
 
     // ---- softmax out
     if (a.save_softmax) {

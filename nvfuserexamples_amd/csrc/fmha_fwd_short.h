@@ -136,22 +136,30 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   // ---- scale and mask (log2 units); keys past the end drop out
   scr.rows_in(mreg);
   scr.turn();
-  float mx = NEG_INF;
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int kk = sb * 32 + 8 * g + 4 * h + t;
-        float xv = fmaf(x[sb][4 * g + t], a.scale_l2, fmaf((float)mv[t], a.mask_a, a.mask_b));
-        xv = kk < a.sk ? xv : NEG_INF;
-        x[sb][4 * g + t] = xv;
-        mx = fmaxf(mx, xv);
-      }
+      for (int t = 0; t < 4; ++t)
+        x[sb][4 * g + t] = fmaf(x[sb][4 * g + t], a.scale_l2, fmaf((float)mv[t], a.mask_a, a.mask_b));
     }
   scr.turn();
+  if (a.sk < C::SKMAX) { // (workgroup-uniform: the reference's own 128 keys skip it)
+#pragma unroll
+    for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kk = sb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+        x[sb][r] = kk < a.sk ? x[sb][r] : NEG_INF;
+      }
+  }
+  float mx = NEG_INF;
+#pragma unroll
+  for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) mx = max3(mx, x[sb][r], x[sb][r + 1]);
   mx = xhalf_max(mx);
   const float mref = mx == NEG_INF ? 0.f : mx;
 
@@ -185,19 +193,24 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
     scr.rows_in(dreg);
     scr.turn();
   }
+  // (With a dropout tensor the products are formed as (x / sum) * (d * scale) whether the outputs are saved or
+  // not -- the saving and the plain operator then give the same O bit for bit; without one, 1 / sum and the scale
+  // are one factor per row.)
   v8 pfrag[NSB][2];
+  const float inv_scaled = inv * a.drop_scale;
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      float keep[4] = {a.drop_scale, a.drop_scale, a.drop_scale, a.drop_scale};
       if (DROPT) {
         const v4 dm = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
-        for (int t = 0; t < 4; ++t) keep[t] = (float)dm[t] * a.drop_scale;
-      }
+        for (int t = 0; t < 4; ++t)
+          pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)((x[sb][4 * g + t] * inv) * ((float)dm[t] * a.drop_scale));
+      } else {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)((x[sb][4 * g + t] * inv) * keep[t]);
+        for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)(x[sb][4 * g + t] * inv_scaled);
+      }
     }
   scr.turn();
 

@@ -150,22 +150,30 @@ void fmha_fwd_stream_save_kernel(const FwdArgs a) {
       }
       scr.rows_in(cur.m);
       scr.turn();
-      float tmax = NEG_INF;
 #pragma unroll
       for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int kk = k0 + sb * 32 + 8 * g + 4 * h + i;
-            float s = fmaf(x[sb][4 * g + i], a.scale_l2, fmaf((float)mv[i], a.mask_a, a.mask_b));
-            s = kk < a.sk ? s : NEG_INF;
-            x[sb][4 * g + i] = s;
-            tmax = fmaxf(tmax, s);
-          }
+          for (int i = 0; i < 4; ++i)
+            x[sb][4 * g + i] = fmaf(x[sb][4 * g + i], a.scale_l2, fmaf((float)mv[i], a.mask_a, a.mask_b));
         }
       scr.turn();
+      if (k0 + BK > a.sk) { // only a partly filled last tile has keys to switch off (workgroup-uniform)
+#pragma unroll
+        for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kk = k0 + sb * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            x[sb][r] = kk < a.sk ? x[sb][r] : NEG_INF;
+          }
+      }
+      float tmax = NEG_INF;
+#pragma unroll
+      for (int sb = 0; sb < NSB; ++sb)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) tmax = max3(tmax, x[sb][r], x[sb][r + 1]);
 
       // ---- online softmax
       tmax = xhalf_max(tmax);
@@ -184,10 +192,12 @@ void fmha_fwd_stream_save_kernel(const FwdArgs a) {
           rs += p;
         }
       lsum = fmaf(lsum, alpha, rs);
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) { // (exactly one wherever the maximum stayed)
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+          for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+      }
 
       // ---- dropped probabilities in the element type (B operand of the second product); undropped ones kept
       scr.rows_in(cur.d);
