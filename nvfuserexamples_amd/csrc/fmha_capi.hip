@@ -564,6 +564,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  v.drop != 1 && !p->kv_len && aligned16(a.mask) && (a.mask_sb % 8) == 0 && (a.mask_sq % 8) == 0 &&
                  (!a.drop_mask || aligned16(a.drop_mask)) && (!a.save_softmax || aligned16(a.save_softmax)) &&
                  (!a.save_dropout || aligned16(a.save_dropout)) && (!saving || a.drop_mask) &&
+                 (long long)p->sq * a.mask_sq < (1LL << 30) && // (the kernel forms 32-bit byte offsets within a head)
                  overrides().fwd_short != 0;
   // Longer key ranges: where the caller provides an LSE buffer, the save-intermediates operator is the forward
   // launch followed by a streaming kernel that derives both saved outputs from that LSE (instead of a second

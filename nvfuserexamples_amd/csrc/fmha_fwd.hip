@@ -93,8 +93,8 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
 
 #if FMHA_TU_SHORT
 // short key ranges under a full mask tensor (the reference's operators at their own shape)
-template <bool DROPT, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
-  auto kern = fmha_fwd_short_kernel<FMHA_TU_T, DROPT, SAVE>;
+template <bool DROPT, bool SAVE, bool FULL> int launch_short_as(FwdArgs &a, hipStream_t s) {
+  auto kern = fmha_fwd_short_kernel<FMHA_TU_T, DROPT, SAVE, FULL>;
   static const bool ready = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
                                                 ShortCfg::LDS_BYTES) == hipSuccess;
@@ -104,6 +104,10 @@ template <bool DROPT, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
   if (nblk > 0x7fffffffLL) return 2;
   hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(ShortCfg::NW * 64), ShortCfg::LDS_BYTES, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+// (more than 96 keys: every 32-key block exists, and the kernel is built without the conditions around them)
+template <bool DROPT, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
+  return a.sk > ShortCfg::SKMAX - 32 ? launch_short_as<DROPT, SAVE, true>(a, s) : launch_short_as<DROPT, SAVE, false>(a, s);
 }
 #endif
 

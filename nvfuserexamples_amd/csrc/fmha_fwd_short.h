@@ -35,7 +35,10 @@ struct ShortCfg {
   static constexpr int LDS_BYTES = 4 * TILEB + NW * Scratch::BYTES; // K, V (two tiles each) + one scratch per wave
 };
 
-template <typename T, bool DROPT, bool SAVE>
+// FULL: more than 96 keys, so all four 32-key blocks and both 64-row tiles exist (the reference's 128 keys).  The
+// products then run without conditions around their blocks: under a condition every block's accumulators are
+// merged with their "block skipped" values afterwards, 32 register copies per block of the second product.
+template <typename T, bool DROPT, bool SAVE, bool FULL>
 __global__ __launch_bounds__(ShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void fmha_fwd_short_kernel(const FwdArgs a) {
   using E = Elem<T>;
@@ -58,8 +61,9 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   int bid = blockIdx.x;
   const int nb = gridDim.x;
   if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);
-  const int bh = bid / a.nqt;
-  const int qt = bid - bh * a.nqt;
+  // (a.nqt = 1 at the reference's own 128 queries: no division there; the same for masks that are not shared)
+  const int bh = a.nqt == 1 ? bid : bid / a.nqt;
+  const int qt = a.nqt == 1 ? 0 : bid - bh * a.nqt;
   const int q0w = qt * C::QT + w * 32;
 
   const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
@@ -70,7 +74,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   TileCopy<T, D, C::BT, NT> tcopy;
   tcopy.init(tid, D);
   const uint32_t lds0 = lds_address(lds);
-  const bool two_tiles = a.sk > C::BT;
+  const bool two_tiles = FULL || a.sk > C::BT;
   tcopy.issue(Kb, 0, a.sk, lds0, tid);
   if (two_tiles) tcopy.issue(Kb, C::BT, a.sk, lds0 + TILEB, tid);
   tcopy.issue(Vb, 0, a.sk, lds0 + 2 * TILEB, tid);
@@ -78,10 +82,14 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 
   v8 qreg[KS];
   {
+    // Row addresses are a per-head base (uniform) plus a 32-bit byte offset: one multiply per row instead of
+    // 64-bit arithmetic ahead of every request (the host keeps sq * row pitch below 2^30 elements on this path).
     int q = q0w + ql;
     q = q < a.sq ? q : a.sq - 1;
+    const char *qb8 = (const char *)Qb;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qreg[ks] = as_v8<T>(*(const u32x4 *)(Qb + (size_t)q * D + ks * 16 + h * 8));
+    for (int ks = 0; ks < KS; ++ks)
+      qreg[ks] = as_v8<T>(*(const u32x4 *)(qb8 + (uint32_t)(q * D + ks * 16 + h * 8) * 2u));
   }
 
   // [.., sq, sk] rows as the wave reads and writes them: instruction i covers rows 4i .. 4i+3 of the
@@ -96,8 +104,9 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
     // scores are forced to -inf).  Unconditional loads matter: a load under a lane condition is merged
     // with its "else" value right behind it, which makes the compiler wait for it on the spot.
     const int ch8 = cvalid ? chunk * 8 : 0;
-    const T *mb = (const T *)a.mask + (size_t)(bh / a.mask_div) * a.mask_sb + ch8;
-    const T *db_ = DROPT ? (const T *)a.drop_mask + (size_t)bh * a.sq * a.sk + ch8 : nullptr;
+    const int mhead = a.mask_div == 1 ? bh : bh / a.mask_div;
+    const char *mb = (const char *)((const T *)a.mask + (size_t)mhead * a.mask_sb);
+    const char *db_ = DROPT ? (const char *)((const T *)a.drop_mask + (size_t)bh * a.sq * a.sk) : nullptr;
     int qrow[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -105,10 +114,10 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
       qrow[i] = q < a.sq ? q : a.sq - 1;
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) mreg[i] = *(const u32x4 *)(mb + (size_t)qrow[i] * a.mask_sq);
+    for (int i = 0; i < 8; ++i) mreg[i] = *(const u32x4 *)(mb + (uint32_t)(qrow[i] * (int)a.mask_sq + ch8) * 2u);
     if (DROPT) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dreg[i] = *(const u32x4 *)(db_ + (size_t)qrow[i] * a.sk);
+      for (int i = 0; i < 8; ++i) dreg[i] = *(const u32x4 *)(db_ + (uint32_t)(qrow[i] * a.sk + ch8) * 2u);
     }
   }
   // Loads complete in the order they were requested.  The K and V copies went out first: once at most
@@ -126,7 +135,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   for (int sb = 0; sb < NSB; ++sb) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) x[sb][r] = 0.f;
-    if (sb * 32 < a.sk) {
+    if (FULL || sb * 32 < a.sk) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
         x[sb] = E::mfma(panel_read_rows<T, C::BT>(lds + (sb >> 1) * TILEB, pl, sb & 1, ks), qreg[ks], x[sb]);
@@ -178,12 +187,12 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 
   // rows of the scratch leave as whole rows of a [.., sq, sk] output
   auto store_rows = [&](void *out) {
-    T *ob = (T *)out + (size_t)bh * a.sq * a.sk + chunk * 8;
+    char *ob = (char *)((T *)out + (size_t)bh * a.sq * a.sk);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int q = q0w + 4 * i + rsub;
       const u32x4 t = scr.row_out(i);
-      if (cvalid && q < a.sq) *(u32x4 *)(ob + (size_t)q * a.sk) = t;
+      if (cvalid && q < a.sq) *(u32x4 *)(ob + (uint32_t)(q * a.sk + chunk * 8) * 2u) = t;
     }
   };
   // ---- dropped, normalised probabilities in the element type: second operand and saved output.
@@ -195,7 +204,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   }
   // (With a dropout tensor the products are formed as (x / sum) * (d * scale) whether the outputs are saved or
   // not -- the saving and the plain operator then give the same O bit for bit; without one, 1 / sum and the scale
-  // are one factor per row.)
+  // are one factor per row, applied to the 64 values of O instead of the 128 of P.)
   v8 pfrag[NSB][2];
   const float inv_scaled = inv * a.drop_scale;
 #pragma unroll
@@ -207,9 +216,9 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
           pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)((x[sb][4 * g + t] * inv) * ((float)dm[t] * a.drop_scale));
-      } else {
+      } else { // unnormalised (values in (0, 1]); O takes the factor on its way out
 #pragma unroll
-        for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)(x[sb][4 * g + t] * inv_scaled);
+        for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)x[sb][4 * g + t];
       }
     }
   scr.turn();
@@ -250,7 +259,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb) {
-    if (sb * 32 < a.sk) {
+    if (FULL || sb * 32 < a.sk) {
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
@@ -264,7 +273,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   if (q < a.sq) {
     T *Ob = (T *)a.o + ((size_t)bh * a.sq + q) * D;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + db * 32, o[db], 1.f, h);
+    for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + db * 32, o[db], DROPT ? 1.f : inv_scaled, h);
     if (a.lse && h == 0) a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
   }
 }
