@@ -173,3 +173,77 @@ def test_randomized_sweep_against_the_oracle():
             _run_case(it, c, rng)
         except AssertionError as e:
             raise AssertionError(f"case #{it} {c}: {e}") from e
+
+
+# ---- the reference's three operators (full [bh,sq,sk] mask tensor; dropout tensor; saved outputs) over sizes that
+# reach every kernel they can run on: the one-pass kernel up to 128 keys (and its build for 97 to 128), the streaming
+# forward, the one-launch save kernel up to 512 keys, forward + save kernel beyond, and the plain / pipelined kernels
+# for key counts that are not multiples of 8.
+def _operator_case(it, rng):
+    dtype = rng.choice(["fp16", "fp16", "bf16"])
+    mode = rng.choice(["infer", "train", "save", "save"])
+    bh = rng.choice([1, 2, 5])
+    sq = rng.choice([1, 7, 32, 33, 100, 127, 128, 129, 200, 256, 300])
+    sk = rng.choice([8, 40, 64, 96, 104, 120, 128, 136, 192, 200, 256, 264, 320, 448, 512, 520, 576, 640, 77, 333])
+    maskk = rng.choice(["01", "01", "normal", "infcols"])
+    scale = rng.choice([2.0, 1.25, 1.0 / 0.9])
+    return dict(dtype=dtype, mode=mode, bh=bh, sq=sq, sk=sk, mask=maskk, drop_scale=scale)
+
+
+def _run_operator_case(it, c):
+    dtype, mode, bh, sq, sk = c["dtype"], c["mode"], c["bh"], c["sq"], c["sk"]
+    q, k, v = make_qkv(bh, sq, sk, 64, seed=1000 + it, dtype=dtype)
+    g = torch.Generator().manual_seed(2000 + it)
+    tol = 2e-3 if dtype == "fp16" else 2e-2
+    if mode == "infer":
+        m = torch.empty(bh, sq, sk).random_(2, generator=g).to(TDT[dtype])
+        o, lse, _, _ = capi.fwd(q.cuda(), k.cuda(), v.cuda(), mask=m.cuda(), mask_kind=capi.MASK_KEEP01, want_lse=True)
+        torch.cuda.synchronize()
+        ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m), mask_kind="keep01", want=("o", "lse"))
+        assert np.abs(f32(o.cpu()) - ref["o"]).max() <= tol, "o"
+        assert np.abs(lse.cpu().numpy() - ref["lse"]).max() <= (1e-3 if dtype == "fp16" else 5e-3), "lse"
+        return
+    if c["mask"] == "01":
+        pm = torch.empty(bh, sq, sk).random_(2, generator=g) * -1000
+    else:
+        pm = torch.randn(bh, sq, sk, generator=g) * 2
+        if c["mask"] == "infcols":
+            pm[:, :, 3::5] = float("-inf")
+            pm[:, sq // 2, :] = float("-inf")          # a row that sees no key
+            pm[:, 0, : max(1, sk - 3)] = float("-inf")  # a row whose keys are all in the last tile
+    pm = pm.to(TDT[dtype])
+    dm = torch.empty(bh, sq, sk).random_(2, generator=g).to(TDT[dtype])
+    save = mode == "save"
+    o, lse, sm, dr = capi.fwd(q.cuda(), k.cuda(), v.cuda(), mask=pm.cuda(), drop_kind=capi.DROP_TENSOR,
+                              drop_mask=dm.cuda(), drop_scale=c["drop_scale"], save=save, want_lse=True)
+    torch.cuda.synchronize()
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(pm), drop_mask=f32(dm), drop_scale=c["drop_scale"],
+                           want=("o", "lse", "softmax", "dropout"))
+    got_o = f32(o.cpu())
+    assert np.isfinite(got_o).all(), "o not finite"
+    assert np.abs(got_o - ref["o"]).max() <= 2 * tol * max(1.0, float(np.abs(ref["o"]).max()) / 2.0), "o"
+    dead = np.isneginf(ref["lse"])
+    gl = lse.cpu().numpy()
+    assert np.array_equal(np.isneginf(gl), dead), "lse: -inf rows differ"
+    if (~dead).any():
+        assert np.abs(gl[~dead] - ref["lse"][~dead]).max() <= (1e-3 if dtype == "fp16" else 5e-3) * \
+            max(1.0, float(np.abs(ref["lse"][~dead]).max()) / 8.0), "lse"
+    if save:
+        got_sm, got_dr = f32(sm.cpu()), f32(dr.cpu())
+        assert np.isfinite(got_sm).all() and np.isfinite(got_dr).all(), "saved outputs not finite"
+        assert np.abs(got_sm - ref["softmax"]).max() <= tol / 2, "softmax"
+        assert np.abs(got_dr - ref["dropout"]).max() <= tol * max(1.0, c["drop_scale"] / 2.0), "dropout"
+        o2, _, _, _ = capi.fwd(q.cuda(), k.cuda(), v.cuda(), mask=pm.cuda(), drop_kind=capi.DROP_TENSOR,
+                               drop_mask=dm.cuda(), drop_scale=c["drop_scale"])
+        torch.cuda.synchronize()
+        assert torch.equal(o2, o), "saving changed O"
+
+
+def test_randomized_sweep_of_the_reference_operators():
+    rng = random.Random(20241126)
+    for it in range(160):
+        c = _operator_case(it, rng)
+        try:
+            _run_operator_case(it, c)
+        except AssertionError as e:
+            raise AssertionError(f"operator case #{it} {c}: {e}") from e
