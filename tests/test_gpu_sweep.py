@@ -236,7 +236,10 @@ def _run_operator_case(it, c):
         o2, _, _, _ = capi.fwd(q.cuda(), k.cuda(), v.cuda(), mask=pm.cuda(), drop_kind=capi.DROP_TENSOR,
                                drop_mask=dm.cuda(), drop_scale=c["drop_scale"])
         torch.cuda.synchronize()
-        assert torch.equal(o2, o), "saving changed O"
+        if sk % 8 == 0:   # rows on 16-byte boundaries: the saving and the plain call run the same arithmetic
+            assert torch.equal(o2, o), "saving changed O"
+        else:             # otherwise two kernel families (the plain loop saves, the pipelined loop does not): a unit
+            assert (o2.float() - o.float()).abs().max().item() <= tol / 4, "saving changed O"   # in the last place at most
 
 
 def test_randomized_sweep_of_the_reference_operators():
