@@ -52,7 +52,7 @@ DropCtx make_drop_ctx(uint64_t seed, uint64_t offset, float p, int sq, int sk) {
 // FMHA_FWD_SAVE_SPLIT=0 keep the save-intermediates operator beyond 128 keys off its one-launch kernel / off the
 // forward-then-save pair of launches,
 // FMHA_FWD_SHORT=0 / FMHA_BWD_SHORT=0 keep short key ranges / short sequences off their
-// one-pass kernels (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
+// one-pass kernels (FMHA_FWD_SHORT=2: only the forwards without a full mask tensor) (FMHA_BWD_SHORT=128 limits the backward one to 128 rows), FMHA_BWD_PAIR=0|1 sets the
 // pairing of causal tiles in the backward, FMHA_MASK_TRIM=0 makes forward and backward visit the key tiles
 // that a per-key mask hard-masks (as FMHA_FLAG_NO_MASK_TRIM does per call), FMHA_FWD_SPLIT=0 never cuts a
 // forward's key range into pieces, FMHA_FWD_SPLIT=n (2..64) cuts it into about n wherever pieces are possible,
@@ -566,6 +566,18 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  (!a.save_dropout || aligned16(a.save_dropout)) && (!saving || a.drop_mask) &&
                  (long long)p->sq * a.mask_sq < (1LL << 30) && // (the kernel forms 32-bit byte offsets within a head)
                  overrides().fwd_short != 0;
+  // The same one-pass kernel without a full mask tensor: no mask, a per-key mask or valid key counts, no dropout or
+  // the Philox rule (FMHA_FWD_SHORT=2 keeps these on the pipelined kernel while the operators' shape stays here).
+  // Measured against the pipelined kernel at S 128 with a padding mask: BH 96 4.4-4.7 against 6.6-6.7 us, BH 512 8.7
+  // against 10.2 (10.2-10.5 against 11.9 with Philox dropout), BH 1 024 13.7 against 16.1 (16.7 against 18.4), level
+  // from BH 2 048 on -- and 5 % behind there with Philox dropout, which therefore stays on the persistent kernel
+  // once the launch has more than six items per compute unit.
+  if (!v.short_keys) {
+    const long long items = (long long)p->bh * ((p->sq + 127) / 128);
+    v.short_keys = !strided && p->d == 64 && p->sk <= 128 && v.mask != kMaskFull && !v.causal && v.drop != 2 && !saving &&
+                   (long long)p->sq * 64 < (1LL << 30) && (v.drop != 1 || items <= 6LL * cu_count()) &&
+                   overrides().fwd_short == 1 && overrides().fwd_head != 1;
+  }
   // Longer key ranges: where the caller provides an LSE buffer, the save-intermediates operator is the forward
   // launch followed by a streaming kernel that derives both saved outputs from that LSE (instead of a second
   // sweep inside a slower forward).  Same alignment needs as above.

@@ -92,22 +92,27 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
 }
 
 #if FMHA_TU_SHORT
-// short key ranges under a full mask tensor (the reference's operators at their own shape)
-template <bool DROPT, bool SAVE, bool FULL> int launch_short_as(FwdArgs &a, hipStream_t s) {
-  auto kern = fmha_fwd_short_kernel<FMHA_TU_T, DROPT, SAVE, FULL>;
+// short key ranges in one pass: under a full mask tensor (the reference's operators at their own shape), and under
+// no mask / a per-key mask / valid key counts, without dropout or with the Philox rule
+template <int MASK, int DROP, bool SAVE, bool FULL> int launch_short_as(FwdArgs &a, hipStream_t s) {
+  auto kern = [] {
+    if constexpr (MASK == kMaskFull) return fmha_fwd_short_kernel<FMHA_TU_T, DROP, SAVE, FULL>;
+    else return fmha_fwd_short_kernel_keymask<FMHA_TU_T, MASK, DROP, FULL>;
+  }();
+  constexpr int kLds = MASK == kMaskFull ? ShortCfg::LDS_BYTES : ShortCfg::LDS_BYTES_KEYMASK;
   static const bool ready = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                ShortCfg::LDS_BYTES) == hipSuccess;
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, kLds) == hipSuccess;
   if (!ready) return 2;
   a.nqt = (a.sq + ShortCfg::QT - 1) / ShortCfg::QT;
   const long long nblk = (long long)a.bh * a.nqt;
   if (nblk > 0x7fffffffLL) return 2;
-  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(ShortCfg::NW * 64), ShortCfg::LDS_BYTES, s, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(ShortCfg::NW * 64), kLds, s, a);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 // (more than 96 keys: every 32-key block exists, and the kernel is built without the conditions around them)
-template <bool DROPT, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
-  return a.sk > ShortCfg::SKMAX - 32 ? launch_short_as<DROPT, SAVE, true>(a, s) : launch_short_as<DROPT, SAVE, false>(a, s);
+template <int MASK, int DROP, bool SAVE> int launch_short(FwdArgs &a, hipStream_t s) {
+  return a.sk > ShortCfg::SKMAX - 32 ? launch_short_as<MASK, DROP, SAVE, true>(a, s)
+                                     : launch_short_as<MASK, DROP, SAVE, false>(a, s);
 }
 #endif
 
@@ -232,8 +237,16 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
 #endif
 #if FMHA_TU_SHORT
   if (v.short_keys) {
-    if (v.saving) return launch_short<true, true>(a, s);
-    return v.drop == 2 ? launch_short<true, false>(a, s) : launch_short<false, false>(a, s);
+    if (v.causal) return 1;
+    if (v.mask == kMaskFull) {
+      if (v.drop == 1) return 1;
+      if (v.saving) return launch_short<kMaskFull, 2, true>(a, s);
+      return v.drop == 2 ? launch_short<kMaskFull, 2, false>(a, s) : launch_short<kMaskFull, 0, false>(a, s);
+    }
+    if (v.drop == 2 || v.saving) return 1;
+    if (v.mask == kMaskPerKey)
+      return v.drop == 1 ? launch_short<kMaskPerKey, 1, false>(a, s) : launch_short<kMaskPerKey, 0, false>(a, s);
+    return v.drop == 1 ? launch_short<kMaskNone, 1, false>(a, s) : launch_short<kMaskNone, 0, false>(a, s);
   }
   if (v.save_once) return launch_stream_save(a, s);
   if (v.save_split) { // forward with LSE, then the saved outputs from that LSE

@@ -16,6 +16,10 @@
 //     (16 bytes per lane, 16 lanes per row).  The MFMA accumulator layout wants the opposite
 //     (lane = query row, 8-byte pieces), which as a global access pattern touches 32 different
 //     cache lines per instruction; a wave-private LDS scratch turns one layout into the other.
+// The same one-pass organisation serves short key ranges WITHOUT a full mask tensor (no mask, a per-key
+// [B,1,1,S] mask, valid key counts; no dropout or the Philox rule): MASK / DROP below.  The mask term of
+// every key then sits in a 128-float LDS row that the workgroup fills once, nothing passes through the
+// row scratch, and P goes into the second product unnormalised.
 // The second product takes the dropped, normalised probabilities -- the very values of the
 // saved "dropout" output -- as its operand, as the reference does (fmha/fmha_manual.cpp:478-490).
 #pragma once
@@ -33,14 +37,18 @@ struct ShortCfg {
   static constexpr int TILEB = BT * D * 2;
   using Scratch = RowScratch<SKMAX>;              // wave-private: rows of a [.., sq, sk] tensor <-> accumulator layout
   static constexpr int LDS_BYTES = 4 * TILEB + NW * Scratch::BYTES; // K, V (two tiles each) + one scratch per wave
+  static constexpr int LDS_BYTES_KEYMASK = 4 * TILEB + SKMAX * 4;   // K, V + the per-key mask terms (no scratch)
 };
 
 // FULL: more than 96 keys, so all four 32-key blocks and both 64-row tiles exist (the reference's 128 keys).  The
 // products then run without conditions around their blocks: under a condition every block's accumulators are
 // merged with their "block skipped" values afterwards, 32 register copies per block of the second product.
-template <typename T, bool DROPT, bool SAVE, bool FULL>
-__global__ __launch_bounds__(ShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void fmha_fwd_short_kernel(const FwdArgs a) {
+// MASK: kMaskFull (the operators' [.., sq, sk] tensor), kMaskPerKey or kMaskNone.  DROP: 0 none, 1 the Philox
+// rule, 2 a [.., sq, sk] dropout tensor (kMaskFull only).  SAVE: kMaskFull with a dropout tensor only.
+template <typename T, int MASK, int DROP, bool SAVE, bool FULL> FMHA_DEV void fwd_short_body(const FwdArgs &a) {
+  constexpr bool DROPT = DROP == 2;
+  constexpr bool ROWS = MASK == kMaskFull; // [.., sq, sk] tensors move through the row scratch
+  static_assert(ROWS || (!DROPT && !SAVE), "dropout tensors and saved outputs come with the full mask tensor");
   using E = Elem<T>;
   using v8 = typename E::v8;
   using v4 = typename E::v4;
@@ -71,6 +79,14 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
 
   // ---- every request of this workgroup, up front
+  // (per-key mask: one value per thread, requested ahead of the copies so that the wait for the copies covers it)
+  float *fM = (float *)(lds + 4 * TILEB); // !ROWS: mask term of key k in log2 units, -inf from the first invisible key on
+  const int kend = ROWS ? a.sk : visible_keys<false>(a, bh, 0);
+  T mraw = (T)0.f;
+  if (MASK == kMaskPerKey && tid < C::SKMAX) {
+    const int mhead = a.mask_div == 1 ? bh : bh / a.mask_div;
+    mraw = ((const T *)a.mask + (size_t)mhead * a.mask_sb)[tid < a.sk ? tid : a.sk - 1];
+  }
   TileCopy<T, D, C::BT, NT> tcopy;
   tcopy.init(tid, D);
   const uint32_t lds0 = lds_address(lds);
@@ -99,7 +115,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   const int rsub = scr.rsub, chunk = scr.chunk;
   const bool cvalid = chunk * 8 < a.sk;
   u32x4 mreg[8], dreg[8];
-  {
+  if (ROWS) {
     // Lanes whose chunk lies past sk read chunk 0 instead (their values are never used: those keys'
     // scores are forced to -inf).  Unconditional loads matter: a load under a lane condition is merged
     // with its "else" value right behind it, which makes the compiler wait for it on the spot.
@@ -124,7 +140,12 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   // the 4 Q, 8 mask and 8 dropout-row loads requested after them are outstanding, they have landed;
   // the first product then runs while the [.., sq, sk] rows are still on their way.  (A test compiles
   // this kernel to assembly and checks that count.)
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + 8 + (DROPT ? 8 : 0)) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 + (ROWS ? 8 : 0) + (DROPT ? 8 : 0)) : "memory");
+  if (!ROWS && tid < C::SKMAX) {
+    float mt = 0.f;
+    if (MASK == kMaskPerKey) mt = fmaf((float)mraw, a.mask_a, a.mask_b);
+    fM[tid] = tid < kend ? mt : NEG_INF;
+  }
   __syncthreads();
 
   PanelLane pl;
@@ -143,19 +164,27 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   }
 
   // ---- scale and mask (log2 units); keys past the end drop out
-  scr.rows_in(mreg);
-  scr.turn();
+  if (ROWS) {
+    scr.rows_in(mreg);
+    scr.turn();
+  }
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const v4 mv = as_v4<T>(scr.piece(sb, g));
+      if (ROWS) {
+        const v4 mv = as_v4<T>(scr.piece(sb, g));
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
-        x[sb][4 * g + t] = fmaf(x[sb][4 * g + t], a.scale_l2, fmaf((float)mv[t], a.mask_a, a.mask_b));
+        for (int t = 0; t < 4; ++t)
+          x[sb][4 * g + t] = fmaf(x[sb][4 * g + t], a.scale_l2, fmaf((float)mv[t], a.mask_a, a.mask_b));
+      } else {
+        const f32x4 mk = *(const f32x4 *)(fM + sb * 32 + 8 * g + 4 * h);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) x[sb][4 * g + t] = fmaf(x[sb][4 * g + t], a.scale_l2, mk[t]);
+      }
     }
-  scr.turn();
-  if (a.sk < C::SKMAX) { // (workgroup-uniform: the reference's own 128 keys skip it)
+  if (ROWS) scr.turn();
+  if (ROWS && a.sk < C::SKMAX) { // (workgroup-uniform: the reference's own 128 keys skip it; !ROWS: fM holds -inf there)
 #pragma unroll
     for (int sb = 0; sb < NSB; ++sb)
 #pragma unroll
@@ -206,6 +235,7 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
   // not -- the saving and the plain operator then give the same O bit for bit; without one, 1 / sum and the scale
   // are one factor per row, applied to the 64 values of O instead of the 128 of P.)
   v8 pfrag[NSB][2];
+  uint32_t wd[4] = {0u, 0u, 0u, 0u};
   const float inv_scaled = inv * a.drop_scale;
 #pragma unroll
   for (int sb = 0; sb < NSB; ++sb)
@@ -216,12 +246,27 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
           pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)((x[sb][4 * g + t] * inv) * ((float)dm[t] * a.drop_scale));
+      } else if (DROP == 1) { // Philox rule: unnormalised, dropped elements zero; O takes scale / sum on its way out
+        if (g == 0) drop_words_q(a.drop, (uint32_t)bh, (uint32_t)(q0w + ql), (uint32_t)(sb * 32), h, l, wd);
+        v4 s4;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) s4[t] = (T)x[sb][4 * g + t];
+        Pack8 pk;
+        if constexpr (__is_same(T, _Float16)) pk.h = s4;
+        else pk.b = s4;
+        uint32_t r0 = pk.u.x, r1 = pk.u.y;
+        drop_apply_pk4(wd[g], ((a.drop.thr - 1u) & 0xffffu) * 0x00010001u, r0, r1); // (thr = 0 gives -1: everything kept)
+        pk.u = u32x2{r0, r1};
+        if constexpr (__is_same(T, _Float16)) s4 = pk.h;
+        else s4 = pk.b;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = s4[t];
       } else { // unnormalised (values in (0, 1]); O takes the factor on its way out
 #pragma unroll
         for (int t = 0; t < 4; ++t) pfrag[sb][g >> 1][4 * (g & 1) + t] = (T)x[sb][4 * g + t];
       }
     }
-  scr.turn();
+  if (ROWS) scr.turn();
 
   if (SAVE && a.save_softmax) {
 #pragma unroll
@@ -276,6 +321,21 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
     for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + db * 32, o[db], DROPT ? 1.f : inv_scaled, h);
     if (a.lse && h == 0) a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
   }
+}
+
+// Under a full mask tensor: two workgroups per compute unit (the row scratch and up to 185 registers).
+template <typename T, int DROP, bool SAVE, bool FULL>
+__global__ __launch_bounds__(ShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void fmha_fwd_short_kernel(const FwdArgs a) {
+  fwd_short_body<T, kMaskFull, DROP, SAVE, FULL>(a);
+}
+// Without one: four workgroups per compute unit (33 KB of LDS, at most 128 registers), which is what keeps launches
+// of more heads than the device holds at once level with the persistent pipelined kernel.
+template <typename T, int MASK, int DROP, bool FULL>
+__global__ __launch_bounds__(ShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void fmha_fwd_short_kernel_keymask(const FwdArgs a) {
+  static_assert(MASK != kMaskFull, "the build for full mask tensors is fmha_fwd_short_kernel");
+  fwd_short_body<T, MASK, DROP, false, FULL>(a);
 }
 
 } // namespace fmha

@@ -28,7 +28,9 @@ def test_short_kernel_waits_for_exactly_the_loads_behind_its_copies():
                         "-S", "--cuda-device-only", SRC, "-o", out], check=True, capture_output=True)
         lines = open(out).read().split("\n")
     starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\S*fmha_fwd_short_kernel\S*:", l)]
-    assert len(starts) == 6  # inference, dropout tensor, dropout tensor + saved outputs; each for any key count and for 97 to 128 keys
+    # full mask tensor: inference, dropout tensor, dropout tensor + saved outputs; no / per-key mask: without dropout
+    # and with the Philox rule; each for any key count and for 97 to 128 keys
+    assert len(starts) == 14
     for start in starts:
         end = next(i for i in range(start, len(lines)) if lines[i].startswith(".Lfunc_end"))
         body = lines[start:end]
@@ -38,6 +40,6 @@ def test_short_kernel_waits_for_exactly_the_loads_behind_its_copies():
         first = waits[0]
         n = int(re.search(r"vmcnt\((\d+)\)", body[first]).group(1))
         behind = [l for l in body[copies[-1] + 1:first] if VM_OP.match(l)]
-        assert n in (12, 20) and len(behind) == n, (lines[start], n, len(behind))
+        assert n in (4, 12, 20) and len(behind) == n, (lines[start], n, len(behind))   # Q rows (+ mask rows (+ dropout rows))
         # and nothing that reads LDS comes before that wait
         assert not any(re.match(r"\s+ds_read", l) for l in body[:first]), lines[start]
