@@ -574,8 +574,9 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   // once the launch has more than six items per compute unit.
   if (!v.short_keys) {
     const long long items = (long long)p->bh * ((p->sq + 127) / 128);
-    v.short_keys = !strided && p->d == 64 && p->sk <= 128 && v.mask != kMaskFull && !v.causal && v.drop != 2 && !saving &&
-                   (long long)p->sq * 64 < (1LL << 30) && (v.drop != 1 || items <= 6LL * cu_count()) &&
+    const long long qpitch = strided ? (a.mq.ss > a.mo.ss ? a.mq.ss : a.mo.ss) : 64; // (folded or run-time row layouts)
+    v.short_keys = p->d == 64 && p->sk <= 128 && v.mask != kMaskFull && !v.causal && v.drop != 2 && !saving &&
+                   (long long)p->sq * qpitch < (1LL << 30) && (v.drop != 1 || items <= 6LL * cu_count()) &&
                    overrides().fwd_short == 1 && overrides().fwd_head != 1;
   }
   // Longer key ranges: where the caller provides an LSE buffer, the save-intermediates operator is the forward

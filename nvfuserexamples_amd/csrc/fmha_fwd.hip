@@ -14,6 +14,9 @@
 #include "fmha_fwd_head.h"
 #else
 #define FMHA_TU_SHORT 0
+#if FMHA_TU_D == 64
+#include "fmha_fwd_short.h" // run-time row layouts: its builds without a full mask tensor
+#endif
 #endif
 
 #if FMHA_TU_BF16
@@ -91,13 +94,14 @@ template <int QB, int MASK, bool CAUSAL, int DROP, bool kPipe = (DROP != 2)> int
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
-#if FMHA_TU_SHORT
+#if FMHA_TU_D == 64
 // short key ranges in one pass: under a full mask tensor (the reference's operators at their own shape), and under
 // no mask / a per-key mask / valid key counts, without dropout or with the Philox rule
 template <int MASK, int DROP, bool SAVE, bool FULL> int launch_short_as(FwdArgs &a, hipStream_t s) {
+  static_assert(MASK != kMaskFull || !kStrided, "full mask tensors: folded layout only");
   auto kern = [] {
     if constexpr (MASK == kMaskFull) return fmha_fwd_short_kernel<FMHA_TU_T, DROP, SAVE, FULL>;
-    else return fmha_fwd_short_kernel_keymask<FMHA_TU_T, MASK, DROP, FULL>;
+    else return fmha_fwd_short_kernel_keymask<FMHA_TU_T, MASK, DROP, FULL, kStrided>;
   }();
   constexpr int kLds = MASK == kMaskFull ? ShortCfg::LDS_BYTES : ShortCfg::LDS_BYTES_KEYMASK;
   static const bool ready = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -234,6 +238,14 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
 int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStream_t s) {
 #if defined(FMHA_DEV_MINIMAL) || FMHA_TU_STRIDED
   if (v.drop == 2 || v.qb == 2) return 1; // folded layout only
+#endif
+#if FMHA_TU_D == 64 && FMHA_TU_STRIDED
+  if (v.short_keys) { // run-time row layouts: the one-pass kernel's builds without a full mask tensor
+    if (v.causal || v.mask == kMaskFull || v.drop == 2 || v.saving) return 1;
+    if (v.mask == kMaskPerKey)
+      return v.drop == 1 ? launch_short<kMaskPerKey, 1, false>(a, s) : launch_short<kMaskPerKey, 0, false>(a, s);
+    return v.drop == 1 ? launch_short<kMaskNone, 1, false>(a, s) : launch_short<kMaskNone, 0, false>(a, s);
+  }
 #endif
 #if FMHA_TU_SHORT
   if (v.short_keys) {

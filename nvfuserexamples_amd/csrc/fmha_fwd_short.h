@@ -19,7 +19,7 @@
 // The same one-pass organisation serves short key ranges WITHOUT a full mask tensor (no mask, a per-key
 // [B,1,1,S] mask, valid key counts; no dropout or the Philox rule): MASK / DROP below.  The mask term of
 // every key then sits in a 128-float LDS row that the workgroup fills once, nothing passes through the
-// row scratch, and P goes into the second product unnormalised.
+// row scratch, and P goes into the second product unnormalised.  These builds also exist for run-time row layouts.
 // The second product takes the dropped, normalised probabilities -- the very values of the
 // saved "dropout" output -- as its operand, as the reference does (fmha/fmha_manual.cpp:478-490).
 #pragma once
@@ -45,8 +45,9 @@ struct ShortCfg {
 // merged with their "block skipped" values afterwards, 32 register copies per block of the second product.
 // MASK: kMaskFull (the operators' [.., sq, sk] tensor), kMaskPerKey or kMaskNone.  DROP: 0 none, 1 the Philox
 // rule, 2 a [.., sq, sk] dropout tensor (kMaskFull only).  SAVE: kMaskFull with a dropout tensor only.
-template <typename T, int MASK, int DROP, bool SAVE, bool FULL> FMHA_DEV void fwd_short_body(const FwdArgs &a) {
+template <typename T, int MASK, int DROP, bool SAVE, bool FULL, bool STRIDED = false> FMHA_DEV void fwd_short_body(const FwdArgs &a) {
   constexpr bool DROPT = DROP == 2;
+  static_assert(!STRIDED || MASK != kMaskFull, "run-time row layouts: the builds without a full mask tensor only");
   constexpr bool ROWS = MASK == kMaskFull; // [.., sq, sk] tensors move through the row scratch
   static_assert(ROWS || (!DROPT && !SAVE), "dropout tensors and saved outputs come with the full mask tensor");
   using E = Elem<T>;
@@ -74,21 +75,22 @@ template <typename T, int MASK, int DROP, bool SAVE, bool FULL> FMHA_DEV void fw
   const int qt = a.nqt == 1 ? 0 : bid - bh * a.nqt;
   const int q0w = qt * C::QT + w * 32;
 
-  const T *Qb = (const T *)a.q + (size_t)bh * a.sq * D;
-  const T *Kb = (const T *)a.k + (size_t)bh * a.sk * D;
-  const T *Vb = (const T *)a.v + (size_t)bh * a.sk * D;
+  using RW = Rows<STRIDED, D>; // folded [bh, s, 64] tensors, or the row maps of the argument block
+  const T *Qb = (const T *)a.q + RW::head(a.mq, bh, a.sq);
+  const T *Kb = (const T *)a.k + RW::head(a.mk, bh, a.sk);
+  const T *Vb = (const T *)a.v + RW::head(a.mv, bh, a.sk);
 
   // ---- every request of this workgroup, up front
   // (per-key mask: one value per thread, requested ahead of the copies so that the wait for the copies covers it)
   float *fM = (float *)(lds + 4 * TILEB); // !ROWS: mask term of key k in log2 units, -inf from the first invisible key on
-  const int kend = ROWS ? a.sk : visible_keys<false>(a, bh, 0);
+  const int kend = ROWS ? a.sk : visible_keys<STRIDED>(a, bh, 0);
   T mraw = (T)0.f;
   if (MASK == kMaskPerKey && tid < C::SKMAX) {
     const int mhead = a.mask_div == 1 ? bh : bh / a.mask_div;
     mraw = ((const T *)a.mask + (size_t)mhead * a.mask_sb)[tid < a.sk ? tid : a.sk - 1];
   }
   TileCopy<T, D, C::BT, NT> tcopy;
-  tcopy.init(tid, D);
+  tcopy.init(tid, RW::ss(a.mk));
   const uint32_t lds0 = lds_address(lds);
   const bool two_tiles = FULL || a.sk > C::BT;
   tcopy.issue(Kb, 0, a.sk, lds0, tid);
@@ -105,7 +107,7 @@ template <typename T, int MASK, int DROP, bool SAVE, bool FULL> FMHA_DEV void fw
     const char *qb8 = (const char *)Qb;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      qreg[ks] = as_v8<T>(*(const u32x4 *)(qb8 + (uint32_t)(q * D + ks * 16 + h * 8) * 2u));
+      qreg[ks] = as_v8<T>(*(const u32x4 *)(qb8 + ((uint32_t)q * RW::ss(a.mq) + (uint32_t)(ks * 16 + h * 8)) * 2u));
   }
 
   // [.., sq, sk] rows as the wave reads and writes them: instruction i covers rows 4i .. 4i+3 of the
@@ -316,7 +318,7 @@ template <typename T, int MASK, int DROP, bool SAVE, bool FULL> FMHA_DEV void fw
 
   const int q = q0w + ql;
   if (q < a.sq) {
-    T *Ob = (T *)a.o + ((size_t)bh * a.sq + q) * D;
+    T *Ob = (T *)a.o + RW::head(a.mo, bh, a.sq) + (size_t)q * RW::ss(a.mo);
 #pragma unroll
     for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + db * 32, o[db], DROPT ? 1.f : inv_scaled, h);
     if (a.lse && h == 0) a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
@@ -331,11 +333,11 @@ void fmha_fwd_short_kernel(const FwdArgs a) {
 }
 // Without one: four workgroups per compute unit (33 KB of LDS, at most 128 registers), which is what keeps launches
 // of more heads than the device holds at once level with the persistent pipelined kernel.
-template <typename T, int MASK, int DROP, bool FULL>
+template <typename T, int MASK, int DROP, bool FULL, bool STRIDED>
 __global__ __launch_bounds__(ShortCfg::NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void fmha_fwd_short_kernel_keymask(const FwdArgs a) {
   static_assert(MASK != kMaskFull, "the build for full mask tensors is fmha_fwd_short_kernel");
-  fwd_short_body<T, MASK, DROP, false, FULL>(a);
+  fwd_short_body<T, MASK, DROP, false, FULL, STRIDED>(a);
 }
 
 } // namespace fmha
