@@ -622,7 +622,9 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
   // eight waves per (head, 512 queries) runs without copies or barriers in its loop.  Taken when the
   // 512-query items fill the compute units evenly (FMHA_FWD_HEAD=0 never, =1 wherever the kernel applies).
   v.head = false;
-  if (!strided && p->d == 64 && p->sk <= 512 && !v.causal && v.drop != 2 && v.mask != kMaskFull && !v.saving &&
+  // (run-time row layouts too, where a head's rows stay within 32-bit byte offsets of its first one)
+  const bool head_rows_ok = !strided || ((long long)p->sk * a.mk.ss < (1LL << 30) && (long long)p->sq * a.mq.ss < (1LL << 40));
+  if (head_rows_ok && p->d == 64 && p->sk <= 512 && !v.causal && v.drop != 2 && v.mask != kMaskFull && !v.saving &&
       overrides().fwd_head != 0) {
     const int cus = cu_count();
     const int chunks = (p->sq + 511) / 512;

@@ -16,6 +16,7 @@
 #define FMHA_TU_SHORT 0
 #if FMHA_TU_D == 64
 #include "fmha_fwd_short.h" // run-time row layouts: its builds without a full mask tensor
+#include "fmha_fwd_head.h"  // and the whole-head kernel
 #endif
 #endif
 
@@ -157,14 +158,14 @@ int launch_stream_save(FwdArgs &a, hipStream_t s) {
 }
 #endif
 
-#if FMHA_TU_SHORT
+#if FMHA_TU_D == 64
 // a whole head's K and V resident in LDS: one persistent workgroup per compute unit
 #ifndef FMHA_HEAD_QB
 #define FMHA_HEAD_QB 2
 #endif
 template <int MASK, int DROP> int launch_head(FwdArgs &a, hipStream_t s) {
   using HC = HeadCfgT<FMHA_HEAD_QB>;
-  auto kern = fmha_fwd_head_kernel<FMHA_TU_T, FMHA_HEAD_QB, MASK, DROP>;
+  auto kern = fmha_fwd_head_kernel<FMHA_TU_T, FMHA_HEAD_QB, MASK, DROP, kStrided>;
   static const int resident = [&]() -> int {
     if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             HC::LDS_BYTES) != hipSuccess)
@@ -240,6 +241,11 @@ int FMHA_NAME(FMHA_TU_TNAME, FMHA_TU_D)(FwdArgs &a, const FwdVariant &v, hipStre
   if (v.drop == 2 || v.qb == 2) return 1; // folded layout only
 #endif
 #if FMHA_TU_D == 64 && FMHA_TU_STRIDED
+  if (v.head && !v.short_keys) { // run-time row layouts: the whole-head kernel
+    if (v.causal || v.drop == 2 || v.mask == kMaskFull) return 1;
+    if (v.mask == kMaskPerKey) return v.drop ? launch_head<kMaskPerKey, 1>(a, s) : launch_head<kMaskPerKey, 0>(a, s);
+    return v.drop ? launch_head<kMaskNone, 1>(a, s) : launch_head<kMaskNone, 0>(a, s);
+  }
   if (v.short_keys) { // run-time row layouts: the one-pass kernel's builds without a full mask tensor
     if (v.causal || v.mask == kMaskFull || v.drop == 2 || v.saving) return 1;
     if (v.mask == kMaskPerKey)

@@ -97,7 +97,9 @@ template <bool HAS_PV, bool HAS_S> constexpr HeadOperandList head_operand_list()
 FMHA_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 template <int N> FMHA_DEV void vm_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-template <typename T, int QBW, int MASK, int DROP>
+// STRIDED: the rows of q, k, v and o lie where the argument block's row maps say ([B,S,H,D] views, packed
+// projections) instead of in folded [bh, s, 64] tensors.
+template <typename T, int QBW, int MASK, int DROP, bool STRIDED = false>
 __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_eu(4 / QBW, 4 / QBW))) void fmha_fwd_head_kernel(const FwdArgs a) {
   using E = Elem<T>;
   using v8 = typename E::v8;
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
     Item it;
     it.bh = a.nqt == 1 ? idx : idx / a.nqt; // (one chunk per head: no division on the way to the first requests)
     it.qc = idx - it.bh * a.nqt;
-    it.kend = visible_keys<false>(a, it.bh, 0);
+    it.kend = visible_keys<STRIDED>(a, it.bh, 0);
     return it;
   };
   // tiles an item of n keys visits: an even number, so that the x / P buffers keep fixed roles
@@ -174,7 +176,12 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
     int r = u * (UT * BK) + crow;
     const int last = it.kend > 0 ? it.kend - 1 : 0;
     r = r < last ? r : last;
-    dma_global_to_lds_b128((const T *)tensor + (size_t)it.bh * (size_t)a.sk * D, (uint32_t)r * (D * 2) + ccolb, dst);
+    if constexpr (!STRIDED) {
+      dma_global_to_lds_b128((const T *)tensor + (size_t)it.bh * (size_t)a.sk * D, (uint32_t)r * (D * 2) + ccolb, dst);
+    } else {
+      const RowMap &map = area == (uint32_t)C::LDS_K ? a.mk : a.mv;
+      dma_global_to_lds_b128((const T *)tensor + map.head(it.bh), (uint32_t)r * ((uint32_t)map.ss * 2u) + ccolb, dst);
+    }
   };
   auto dmaK = [&](const Item &it, int u) { dma_unit(a.k, it, u, (uint32_t)C::LDS_K); };
   auto dmaV = [&](const Item &it, int u) { dma_unit(a.v, it, u, (uint32_t)C::LDS_V); };
@@ -225,7 +232,8 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
   auto q_row = [&](const Item &it, int qb) {
     int q = it.qc * QT + w * (QB * 32) + qb * 32 + ql;
     q = q < a.sq ? q : a.sq - 1; // rows past the end repeat the last valid row and are never stored
-    return (const T *)a.q + ((size_t)it.bh * (size_t)a.sq + (size_t)q) * D + h * 8;
+    if constexpr (!STRIDED) return (const T *)a.q + ((size_t)it.bh * (size_t)a.sq + (size_t)q) * D + h * 8;
+    else return (const T *)a.q + a.mq.head(it.bh) + (size_t)q * (size_t)a.mq.ss + h * 8;
   };
   u32x4 qraw[QB][KS];
   // (real = false: a request that must exist for the registers' sake but whose rows nobody will use -- every
@@ -720,7 +728,8 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
     // The next item's Q rows (requested at the last hook) become Q' before this item's outputs are stored: the
     // wait for them covers only older requests, and the next item starts without a wait.
     if (more) convertQ();
-    T *Ob = (T *)a.o + (size_t)bh * (size_t)a.sq * D;
+    T *Ob = (T *)a.o + (STRIDED ? a.mo.head(bh) : (size_t)bh * (size_t)a.sq * D);
+    const size_t o_pitch = STRIDED ? (size_t)a.mo.ss : (size_t)D;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const int q = q0w + qb * 32 + ql;
@@ -728,7 +737,7 @@ __global__ __launch_bounds__(HeadCfgT<QBW>::NT) __attribute__((amdgpu_waves_per_
       const float inv = lt > 0.f ? a.drop_scale / lt : 0.f;
       if (q < a.sq) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * D + db * 32, o[qb][db], inv, h);
+        for (int db = 0; db < DB; ++db) store_acc_block_row<T>(Ob + (size_t)q * o_pitch + db * 32, o[qb][db], inv, h);
         if (a.lse && h == 0) a.lse[(size_t)bh * a.sq + q] = lt > 0.f ? (mref[qb] + fast_log2(lt)) * FMHA_LN2 : NEG_INF;
       }
     }

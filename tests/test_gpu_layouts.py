@@ -194,3 +194,46 @@ def test_headline_shape_packed_projection_equals_folded_path(monkeypatch):
     # and without the dealing and the trimming
     o0 = capi.fwd(q4, k4, v4, flags=capi.FLAG_NO_MASK_TRIM, **kw)[0]
     assert torch.equal(o0, o4)
+    # the whole-head kernel reads the packed buffer in place too, and gives the bits it gives on folded tensors
+    monkeypatch.delenv("FMHA_FWD_HEAD")
+    o5, l5, _, _ = capi.fwd(q4, k4, v4, want_lse=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(o5.reshape(b * h, s, d), o_head)
+    assert torch.equal(l5.reshape(b * h, s), l_head)
+
+
+@pytest.mark.parametrize("b,h,sq,sk,p,masked,packed", [
+    (2, 3, 200, 333, 0.1, True, False),    # ragged query chunk, partly filled last key tile, dropout, padding mask
+    (3, 2, 512, 264, 0.0, False, True),    # packed projection, no mask
+    (1, 4, 1030, 512, 0.3, True, True),    # three 512-query items per head, the last one nearly empty
+])
+def test_whole_head_kernel_on_strided_layouts(b, h, sq, sk, p, masked, packed, monkeypatch):
+    """FMHA_FWD_HEAD=1 puts every eligible forward on the whole-head kernel: [B,H,S,D] views of [B,S,H,D] memory and
+    slices of a packed projection against the folded tensors (same bits) and the oracle."""
+    monkeypatch.setenv("FMHA_FWD_HEAD", "1")
+    bh, d = b * h, 64
+    q, k, v = make_qkv(bh, sq, sk, d, seed=bh + sk)
+    if packed and sq != sk:
+        packed = False   # (one packed buffer holds q, k and v of one length)
+    kw, okw = {}, {}
+    if p:
+        kw.update(drop_kind=capi.DROP_PHILOX, p_drop=p, seed=11, offset=5)
+        okw.update(philox=True, p_drop=p, seed=11, offset=5)
+    m = None
+    if masked:
+        m = pad_mask(b, sk, sk // 2, sk).half()
+        kw["mask"] = m.cuda()
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    o3, l3, _, _ = capi.fwd(qc, kc, vc, want_lse=True, **kw)
+    if packed:
+        q4, k4, v4 = _packed(qc, kc, vc, b, h)
+    else:
+        q4, k4, v4 = _bshd(qc, b, h), _bshd(kc, b, h), _bshd(vc, b, h)
+    o4, l4, _, _ = capi.fwd(q4, k4, v4, want_lse=True, **kw)
+    torch.cuda.synchronize()
+    assert o4.permute(0, 2, 1, 3).is_contiguous()
+    assert torch.equal(o4.reshape(bh, sq, d), o3)
+    assert torch.equal(l4.reshape(bh, sq), l3)
+    ref = oracle.attention(f32(q), f32(k), f32(v), mask=f32(m) if masked else None, want=("o", "lse"), **okw)
+    assert np.abs(f32(o4.reshape(bh, sq, d).cpu()) - ref["o"]).max() <= O_TOL["fp16"]
+    assert np.abs(l4.reshape(bh, sq).cpu().numpy() - ref["lse"]).max() <= 1e-3
