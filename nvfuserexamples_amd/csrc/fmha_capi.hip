@@ -564,7 +564,7 @@ int fmha_fwd_launch(const fmha_fwd_params *caller, void *hip_stream) {
                  v.drop != 1 && !p->kv_len && aligned16(a.mask) && (a.mask_sb % 8) == 0 && (a.mask_sq % 8) == 0 &&
                  (!a.drop_mask || aligned16(a.drop_mask)) && (!a.save_softmax || aligned16(a.save_softmax)) &&
                  (!a.save_dropout || aligned16(a.save_dropout)) && (!saving || a.drop_mask) &&
-                 (long long)p->sq * a.mask_sq < (1LL << 30) && // (the kernel forms 32-bit byte offsets within a head)
+                 (long long)p->sq * (a.mask_sq > 128 ? a.mask_sq : 128) < (1LL << 30) && // (the kernel forms 32-bit byte offsets within a head: mask rows, and [.., sq, sk] rows of up to 128 keys)
                  overrides().fwd_short != 0;
   // The same one-pass kernel without a full mask tensor: no mask, a per-key mask or valid key counts, no dropout or
   // the Philox rule (FMHA_FWD_SHORT=2 keeps these on the pipelined kernel while the operators' shape stays here).
